@@ -1,0 +1,112 @@
+/*
+ * snnlib_lif.h -- C ABI of libsnnlif_gfx950.so: the LIF "fire" forward / backward operators
+ * of snnlib as hand-written HIP kernels for MI355X (gfx950).
+ *
+ * The library is the device-side half of the Python extension module `snnlib`
+ * (reference binding table: snnlib/cuda/snn.cpp:798-830).  Every entry point below replaces one
+ * host launcher of the reference; the `snnlib` module (csrc/snnlib_ext.cpp) allocates the output
+ * tensors and forwards raw device pointers here, exactly where the reference's pybind forwarders
+ * (snnlib/cuda/snn.cpp:11-17, 270-279) call their *_cuda launchers.
+ *
+ * Conventions shared by all entry points
+ *   - Tensors are dense row-major [T, N]: T time steps, N = B*C*H*W (or B*C) neurons; element
+ *     (t, n) sits at index t*N + n (reference indexing: snnlib/cuda/snn_kernel_fp.cu:45 with
+ *     b*CHW + i folded into n -- neurons are independent, so the batch axis needs no loop).
+ *   - All pointers are DEVICE pointers on the current HIP device.  Inputs are only read; outputs
+ *     are fully overwritten.  Nothing is allocated, nothing is kept between calls, so calls are
+ *     thread-safe and may be issued on any stream.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only enqueue
+ *     work; they never synchronise.
+ *   - `dtype` selects the storage type of every tensor argument (see SNNLIF_DTYPE_*).  Arithmetic
+ *     is IEEE fp32 for F32 and BF16 storage and fp64 for F64 storage, in the reference's operation
+ *     order, without fused multiply-add contraction.
+ *   - Return value: SNNLIF_OK (0), a negative SNNLIF_ERR_* argument error, or a positive
+ *     hipError_t value reported by the launch.  T == 0 or N == 0 is a successful no-op.
+ */
+#ifndef SNNLIB_LIF_H
+#define SNNLIB_LIF_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SNNLIF_ABI_VERSION 1
+
+/* Storage types. */
+#define SNNLIF_DTYPE_F32  0 /* float storage, fp32 arithmetic (the reference's training dtype) */
+#define SNNLIF_DTYPE_F64  1 /* double storage, fp64 arithmetic */
+#define SNNLIF_DTYPE_BF16 2 /* bfloat16 storage, fp32 arithmetic, round-to-nearest-even stores */
+
+/* Return codes (hipError_t values are positive). */
+#define SNNLIF_OK              0
+#define SNNLIF_ERR_ARG        -1 /* NULL pointer with non-empty shape, negative T or N, T*N overflow */
+#define SNNLIF_ERR_DTYPE      -2 /* dtype is not one of SNNLIF_DTYPE_* */
+#define SNNLIF_ERR_WORKSPACE  -3 /* workspace missing or smaller than snnlif_fire_bp_workspace_bytes() */
+#define SNNLIF_ERR_ALIGN      -4 /* a pointer is not aligned to its element size */
+
+/* Largest T for which the backward keeps the recomputed membrane potential in registers and
+ * therefore needs no workspace. */
+#define SNNLIF_BP_FUSED_MAX_T 32
+
+/* ABI version of the loaded library (== SNNLIF_ABI_VERSION it was built with). */
+int snnlif_abi_version(void);
+
+/* Code-object target the kernels were compiled for ("gfx950"). */
+const char* snnlif_target_arch(void);
+
+/* Static, human-readable text for a return code of this library (negative codes) or of HIP
+ * (positive codes). Never NULL. */
+const char* snnlif_strerror(int code);
+
+/*
+ * Fire forward: spikes only.
+ *   u[t] = (alpha * u[t-1]) * (1 - s[t-1]) + x[t],   s[t] = u[t] > thresh,   u[-1] = s[-1] = 0
+ *   spike[t] = s[t] as 0.0 / 1.0 in the storage dtype.
+ * Replaces fire_s_fp_cuda + fire_s_fp_kernel (snnlib/cuda/snn_kernel_fp.cu:15-73), bound as
+ * snnlib.fire_s_fp (snnlib/cuda/snn.cpp:11-17, 799).
+ */
+int snnlif_fire_s_fp(const void* spatial, void* spike, int dtype, int64_t T, int64_t N,
+                     float alpha, float thresh, void* stream);
+
+/*
+ * Fire forward: membrane potential and spikes.  Same recurrence; mem[t] = u[t], spike[t] = s[t].
+ * Either output may be NULL to skip it (mem only = the reference's fire_u_fp_kernel,
+ * snnlib/cuda/snn_kernel_bp.cu:15-52; both = fire_us_fp_kernel, snnlib/cuda/snn_kernel_bp.cu:54-93,
+ * which the reference launches from fire_fc_bp_cuda :1089 and fire_conv_bp_cuda :1372).
+ */
+int snnlif_fire_us_fp(const void* spatial, void* mem, void* spike, int dtype, int64_t T, int64_t N,
+                      float alpha, float thresh, void* stream);
+
+/*
+ * Bytes of device workspace snnlif_fire_bp needs for this shape: 0 when
+ * T <= SNNLIF_BP_FUSED_MAX_T (membrane potential recomputed into registers), otherwise
+ * T*N*sizeof(arithmetic type) for the recomputed membrane potential (the reference always
+ * allocates this tensor: `mem`, snnlib/cuda/snn_kernel_bp.cu:154).  Returns 0 for invalid arguments.
+ */
+size_t snnlif_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t N);
+
+/*
+ * Fire backward: gradient of the loss w.r.t. the input current, given the input current saved by
+ * the forward and the gradient w.r.t. the spikes.  Recomputes u[t] from `spatial`, then for
+ * t = T-1 .. 0 with gu = 0 initially:
+ *   gs = ((u[t]-thresh) < interval && (thresh-u[t]) < interval) ? grad_spike[t] - (gu*alpha)*u[t] : 0
+ *   gu = gs*beta + (gu*alpha) * (u[t] <= thresh);      grad_spatial[t] = gu
+ * Replaces fire_bp_cuda + fire_u_fp_kernel + fire_bp_kernel
+ * (snnlib/cuda/snn_kernel_bp.cu:15-52, 95-168), bound as snnlib.fire_bp
+ * (snnlib/cuda/snn.cpp:270-279, 813).
+ * `workspace` may be NULL when snnlif_fire_bp_workspace_bytes() is 0; otherwise it must point to at
+ * least that many bytes of device memory aligned to 16 bytes, private to this call until the
+ * stream has run it.
+ */
+int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spatial, int dtype,
+                   int64_t T, int64_t N, float alpha, float thresh, float beta, float interval,
+                   void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* SNNLIB_LIF_H */

@@ -1,0 +1,89 @@
+"""ctypes binding of ``oracle/lif_oracle.c`` (TEST INFRASTRUCTURE ONLY).
+
+The C file restates the reference's fire kernels as scalar CPU loops
+(snnlib/cuda/snn_kernel_fp.cu:37-52, snnlib/cuda/snn_kernel_bp.cu:34-51 and :117-138).  Arrays are numpy,
+C-contiguous, shaped ``[T, B, ...]`` like the reference's tensors (``T = shape[0]``,
+``B = shape[1]``, snnlib/cuda/snn_kernel_fp.cu:60-63).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liblif_oracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile ``lif_oracle.c`` into ``liblif_oracle.so`` next to it (needs gcc and make)."""
+    if force:
+        subprocess.run(["make", "-C", _HERE, "clean"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+    return _LIB_PATH
+
+
+def _load():
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(_LIB_PATH):
+        build()
+    lib = ctypes.CDLL(_LIB_PATH)
+    i64, f32, ptr = ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+    for sfx in ("f32", "f64"):
+        getattr(lib, f"lif_oracle_forward_{sfx}").argtypes = [ptr, ptr, ptr, i64, i64, i64, f32, f32]
+        getattr(lib, f"lif_oracle_forward_{sfx}").restype = None
+        getattr(lib, f"lif_oracle_reverse_{sfx}").argtypes = [ptr, ptr, ptr, i64, i64, i64, f32, f32, f32, f32]
+        getattr(lib, f"lif_oracle_reverse_{sfx}").restype = None
+        getattr(lib, f"lif_oracle_backward_{sfx}").argtypes = [ptr, ptr, ptr, ptr, i64, i64, i64, f32, f32, f32, f32]
+        getattr(lib, f"lif_oracle_backward_{sfx}").restype = None
+    _lib = lib
+    return lib
+
+
+def _suffix(a):
+    if a.dtype == np.float32:
+        return "f32"
+    if a.dtype == np.float64:
+        return "f64"
+    raise TypeError(f"oracle supports float32/float64 arrays, got {a.dtype}")
+
+
+def _dims(a):
+    if a.ndim < 2:
+        raise ValueError("expected an array shaped [T, B, ...]")
+    T, B = a.shape[0], a.shape[1]
+    chw = int(np.prod(a.shape[2:], dtype=np.int64)) if a.ndim > 2 else 1
+    return T, B, chw
+
+
+def _p(a):
+    return ctypes.c_void_p(a.ctypes.data) if a is not None else ctypes.c_void_p(0)
+
+
+def fire_forward(x, alpha, thresh):
+    """Return ``(mem, spike)``, both shaped and typed like ``x``."""
+    x = np.ascontiguousarray(x)
+    sfx = _suffix(x)
+    T, B, chw = _dims(x)
+    mem = np.empty_like(x)
+    spike = np.empty_like(x)
+    getattr(_load(), f"lif_oracle_forward_{sfx}")(_p(x), _p(mem), _p(spike), T, B, chw, alpha, thresh)
+    return mem, spike
+
+
+def fire_backward(x, grad_spike, alpha, thresh, beta, interval):
+    """Return ``grad_x`` for the input current ``x`` and upstream spike gradient ``grad_spike``."""
+    x = np.ascontiguousarray(x)
+    g = np.ascontiguousarray(grad_spike, dtype=x.dtype)
+    if g.shape != x.shape:
+        raise ValueError("grad_spike must have the shape of x")
+    sfx = _suffix(x)
+    T, B, chw = _dims(x)
+    gx = np.empty_like(x)
+    scratch = np.empty_like(x)
+    getattr(_load(), f"lif_oracle_backward_{sfx}")(_p(x), _p(g), _p(gx), _p(scratch), T, B, chw,
+                                                  alpha, thresh, beta, interval)
+    return gx

@@ -1,0 +1,48 @@
+"""Pure-PyTorch restatement of the reference's gold LIF fire path (TEST INFRASTRUCTURE ONLY).
+
+Follows snnlib/example/gold_op.py:17-44 operation for operation -- Heaviside forward with the
+rectangular surrogate gradient (:17-29), and the time loop ``u[t] = x[t] + 0``,
+``u[t] += u[t-1] * (1 - s[t-1]) * alpha`` for t > 0, ``s[t] = fire(u[t])`` (:34-44) -- with two
+deliberate differences: the window length is ``x.shape[0]`` instead of the module constant
+``time_step`` (:12, :37), and the hyper-parameters are arguments instead of module constants (:8-11).
+The spike is not detached, so autograd carries the reset-path gradient exactly as the reference's
+graph does.  This is the parity target of the HIP kernels and the path ``bench.py`` times on the
+host CPU as ``cpu_baseline``.
+"""
+import torch
+
+
+class _Heaviside(torch.autograd.Function):
+    """``u > thresh`` forward; ``grad * 1[|u - thresh| < interval] * beta`` backward."""
+
+    @staticmethod
+    def forward(ctx, u, thresh, beta, interval):
+        ctx.save_for_backward(u)
+        ctx.hyper = (thresh, beta, interval)
+        return u.gt(thresh).to(u.dtype)
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        (u,) = ctx.saved_tensors
+        thresh, beta, interval = ctx.hyper
+        window = (abs(u - thresh) < interval).to(u.dtype)
+        return grad_out.clone() * window * beta, None, None, None
+
+
+def gold_fire(x, alpha, thresh, beta=1.0, interval=0.5):
+    """Return ``(u, s)`` stacked over time for input current ``x`` shaped ``[T, ...]``."""
+    u, s = [], []
+    for t in range(x.shape[0]):
+        u.append(x[t] + 0)
+        if t > 0:
+            u[t] += u[t - 1] * (1 - s[t - 1]) * alpha
+        s.append(_Heaviside.apply(u[t], thresh, beta, interval))
+    return torch.stack(u, dim=0), torch.stack(s, dim=0)
+
+
+def gold_fire_fwd_bwd(x, grad_spike, alpha, thresh, beta=1.0, interval=0.5):
+    """Forward plus ``s.backward(grad_spike)``; returns ``(u, s, grad_x)`` (all detached)."""
+    xr = x.detach().clone().requires_grad_(True)
+    u, s = gold_fire(xr, alpha, thresh, beta, interval)
+    s.backward(grad_spike)
+    return u.detach(), s.detach(), xr.grad.detach()

@@ -1,0 +1,133 @@
+"""ctypes view of the C ABI in ``include/snnlib_lif.h`` (``libsnnlif_gfx950.so``).
+
+This is the boundary the parity tests and the benchmark drive directly: raw device pointers, sizes
+and a stream handle, no torch types in any signature.  The helpers at the bottom only unwrap
+``torch.Tensor`` arguments into those pointers; they allocate nothing except the outputs the caller
+asks for and never fall back to another implementation -- if the library is missing, loading raises.
+"""
+import ctypes
+import os
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG_DIR, "libsnnlif_gfx950.so")
+
+DTYPE_F32, DTYPE_F64, DTYPE_BF16 = 0, 1, 2
+OK, ERR_ARG, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN = 0, -1, -2, -3, -4
+BP_FUSED_MAX_T = 32
+
+# name -> (restype, argtypes); must list every symbol include/snnlib_lif.h declares.
+_vp, _i64, _f32, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_size_t
+SYMBOLS = {
+    "snnlif_abi_version": (_int, []),
+    "snnlif_target_arch": (ctypes.c_char_p, []),
+    "snnlif_strerror": (ctypes.c_char_p, [_int]),
+    "snnlif_fire_s_fp": (_int, [_vp, _vp, _int, _i64, _i64, _f32, _f32, _vp]),
+    "snnlif_fire_us_fp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _vp]),
+    "snnlif_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64]),
+    "snnlif_fire_bp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
+}
+
+_lib = None
+
+
+class SnnlifError(RuntimeError):
+    def __init__(self, code, where):
+        self.code = code
+        super().__init__(f"{where}: {strerror(code)} (code {code})")
+
+
+def load():
+    """Load the library once and type its entry points.  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m snn_gpu_training_bptt_amd.build` "
+            "(there is no CPU or PyTorch fallback for the LIF fire kernels)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in SYMBOLS.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def strerror(code):
+    return load().snnlif_strerror(int(code)).decode()
+
+
+def _check(rc, where):
+    if rc != OK:
+        raise SnnlifError(rc, where)
+
+
+# ---- thin tensor-unwrapping helpers (used by tests and bench; torch is plumbing only) ----------
+
+def _torch_dtype_code(t):
+    import torch
+    codes = {torch.float32: DTYPE_F32, torch.float64: DTYPE_F64, torch.bfloat16: DTYPE_BF16}
+    if t.dtype not in codes:
+        raise TypeError(f"unsupported dtype {t.dtype}")
+    return codes[t.dtype]
+
+
+def _dims(t):
+    T = t.shape[0]
+    return T, (t.numel() // T if T else 0)
+
+
+def _stream_handle(t):
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def _require_dense_gpu(*tensors):
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise ValueError("device tensor required")
+        if not t.is_contiguous():
+            raise ValueError("dense (contiguous) tensor required")
+
+
+def fire_s_fp_into(spatial, spike, alpha, thresh):
+    """``snnlif_fire_s_fp`` on torch tensors already resident on the GPU; writes ``spike``."""
+    _require_dense_gpu(spatial, spike)
+    T, N = _dims(spatial)
+    rc = load().snnlif_fire_s_fp(spatial.data_ptr(), spike.data_ptr(), _torch_dtype_code(spatial),
+                                 T, N, alpha, thresh, _stream_handle(spatial))
+    _check(rc, "snnlif_fire_s_fp")
+    return spike
+
+
+def fire_us_fp_into(spatial, mem, spike, alpha, thresh):
+    """``snnlif_fire_us_fp``; ``mem`` or ``spike`` may be None to skip that output."""
+    _require_dense_gpu(spatial, mem, spike)
+    T, N = _dims(spatial)
+    rc = load().snnlif_fire_us_fp(spatial.data_ptr(),
+                                  mem.data_ptr() if mem is not None else None,
+                                  spike.data_ptr() if spike is not None else None,
+                                  _torch_dtype_code(spatial), T, N, alpha, thresh,
+                                  _stream_handle(spatial))
+    _check(rc, "snnlif_fire_us_fp")
+    return mem, spike
+
+
+def fire_bp_workspace_bytes(dtype_code, T, N):
+    return int(load().snnlif_fire_bp_workspace_bytes(dtype_code, T, N))
+
+
+def fire_bp_into(spatial, grad_spike, grad_spatial, alpha, thresh, beta, interval, workspace=None):
+    """``snnlif_fire_bp``; ``workspace`` is a uint8 device tensor when the shape needs one."""
+    _require_dense_gpu(spatial, grad_spike, grad_spatial, workspace)
+    T, N = _dims(spatial)
+    ws_ptr = workspace.data_ptr() if workspace is not None else None
+    ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    rc = load().snnlif_fire_bp(spatial.data_ptr(), grad_spike.data_ptr(), grad_spatial.data_ptr(),
+                               _torch_dtype_code(spatial), T, N, alpha, thresh, beta, interval,
+                               ws_ptr, ws_bytes, _stream_handle(spatial))
+    _check(rc, "snnlif_fire_bp")
+    return grad_spatial

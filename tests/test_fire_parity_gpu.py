@@ -1,0 +1,152 @@
+"""GPU parity of the HIP fire kernels against the CPU oracle, driven through the C ABI
+(``include/snnlib_lif.h``) on seeded inputs.
+
+Bars: spikes bit-exact; membrane potentials and input gradients compared for exact equality as
+well (the kernels keep the reference's operation order and are built without FMA contraction), with
+the stated tolerance of 1e-5 relative as the documented fallback bar.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import ALPHA, BETA, INTERVAL, THRESH
+
+pytestmark = pytest.mark.gpu
+
+RTOL = 1e-5  # stated bar for membrane potentials and gradients (relative)
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from snn_gpu_training_bptt_amd import lif_cabi
+    lif_cabi.load()
+    return lif_cabi
+
+
+@pytest.fixture(scope="module")
+def oracle():
+    from oracle import c_oracle
+    return c_oracle
+
+
+def make_inputs(shape, mean, std, seed, dtype=torch.float32):
+    gen = torch.Generator().manual_seed(seed)
+    x = (mean + std * torch.randn(shape, generator=gen)).to(dtype)
+    g = torch.randn(shape, generator=gen).to(dtype)
+    return x, g
+
+
+def run_gpu(cabi, x, g, alpha=ALPHA, thresh=THRESH, beta=BETA, interval=INTERVAL):
+    xd, gd = x.cuda(), g.cuda()
+    mem = torch.empty_like(xd)
+    spike_a = torch.empty_like(xd)
+    spike_b = torch.empty_like(xd)
+    gx = torch.empty_like(xd)
+    cabi.fire_s_fp_into(xd, spike_a, alpha, thresh)
+    cabi.fire_us_fp_into(xd, mem, spike_b, alpha, thresh)
+    code = {torch.float32: 0, torch.float64: 1, torch.bfloat16: 2}[x.dtype]
+    T = x.shape[0]
+    ws_bytes = cabi.fire_bp_workspace_bytes(code, T, x.numel() // T)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda") if ws_bytes else None
+    cabi.fire_bp_into(xd, gd, gx, alpha, thresh, beta, interval, workspace=ws)
+    torch.cuda.synchronize()
+    return mem.cpu(), spike_a.cpu(), spike_b.cpu(), gx.cpu()
+
+
+def assert_parity(oracle, x, g, outs, alpha=ALPHA, thresh=THRESH, beta=BETA, interval=INTERVAL):
+    mem, spike_a, spike_b, gx = outs
+    mem_o, spike_o = oracle.fire_forward(x.numpy(), alpha, thresh)
+    gx_o = oracle.fire_backward(x.numpy(), g.numpy(), alpha, thresh, beta, interval)
+    assert np.array_equal(spike_a.numpy(), spike_o), "spikes (fire_s_fp) differ from the oracle"
+    assert np.array_equal(spike_b.numpy(), spike_o), "spikes (fire_us_fp) differ from the oracle"
+    np.testing.assert_allclose(mem.numpy(), mem_o, rtol=RTOL, atol=0)
+    np.testing.assert_allclose(gx.numpy(), gx_o, rtol=RTOL, atol=0)
+    # stronger than the stated bar: same operation order, no contraction -> identical values
+    assert np.array_equal(mem.numpy(), mem_o), "membrane potential not bit-identical"
+    assert np.array_equal(gx.numpy(), gx_o), "input gradient not bit-identical"
+
+
+CASES = [
+    # (shape, mean, std)                                   what it covers
+    ((4, 8, 16, 8, 8), 0.5, 1.0),       # configuration 1 (the reference's CPU-runnable case)
+    ((6, 2, 8), 0.0, 1.0),              # the reference test's fc shape (test_utils.py:18)
+    ((6, 2, 8, 8, 8), 0.0, 1.0),        # the reference test's conv shape (test_utils.py:24)
+    ((8, 4, 16, 32, 32), 0.5, 1.0),     # T=8 register window, conv-like
+    ((1, 3, 5), 0.5, 1.0),              # T=1, odd N -> scalar lanes
+    ((3, 2, 7, 3), 0.5, 1.0),           # N=42: 2-wide lanes
+    ((5, 1, 1), 0.5, 1.0),              # a single neuron
+    ((7, 3, 1000), 0.5, 1.0),           # T=7 inside the T<=8 window
+    ((12, 2, 64, 9), 0.3, 0.8),         # T=12 inside the T<=16 window
+    ((16, 2, 32, 8, 8), 0.5, 1.0),      # T=16
+    ((32, 2, 16, 16, 16), 0.3, 0.8),    # T=32 (configuration 3's window)
+    ((29, 2, 300), 0.3, 0.8),           # T=29 inside the T<=32 window
+    ((33, 2, 16, 8, 8), 0.3, 0.8),      # first T on the workspace path
+    ((70, 3, 129), 0.3, 0.8),           # long window, odd N
+]
+
+
+@pytest.mark.parametrize("shape,mean,std", CASES)
+def test_fp32_parity(cabi, oracle, shape, mean, std):
+    x, g = make_inputs(shape, mean, std, seed=1234)
+    assert_parity(oracle, x, g, run_gpu(cabi, x, g))
+
+
+@pytest.mark.parametrize("alpha,thresh,beta,interval", [
+    (0.3, 0.5, 1.0, 0.5),      # decay that is not a power of two: exposes any FMA contraction
+    (0.25, 0.25, 1.0, 0.5),    # the reference's default threshold (snnlib_func.py:14)
+    (0.9, 1.0, 0.7, 0.3),
+    (0.0, 0.5, 1.0, 0.5),      # no memory: per-step Heaviside
+    (1.0, 0.5, 2.0, 1.5),
+])
+def test_fp32_parity_hyperparameters(cabi, oracle, alpha, thresh, beta, interval):
+    x, g = make_inputs((8, 4, 32, 8, 8), 0.5, 1.0, seed=7)
+    assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha, thresh, beta, interval),
+                  alpha, thresh, beta, interval)
+
+
+@pytest.mark.parametrize("shape", [(8, 4, 16, 8, 8), (6, 3, 7), (33, 2, 10)])
+def test_fp64_parity(cabi, oracle, shape):
+    x, g = make_inputs(shape, 0.5, 1.0, seed=99, dtype=torch.float64)
+    assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
+
+
+def test_empty_shapes_are_noops(cabi):
+    for shape in [(0, 4, 8), (4, 0, 8), (4, 2, 0)]:
+        x = torch.empty(shape, device="cuda")
+        spike = torch.empty_like(x)
+        gx = torch.empty_like(x)
+        cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+        cabi.fire_bp_into(x, x, gx, ALPHA, THRESH, BETA, INTERVAL)
+    torch.cuda.synchronize()
+
+
+def test_argument_errors(cabi):
+    lib = cabi.load()
+    x = torch.zeros(4, 8, device="cuda")
+    assert lib.snnlif_fire_s_fp(x.data_ptr(), None, 0, 4, 8, ALPHA, THRESH, None) == cabi.ERR_ARG
+    assert lib.snnlif_fire_s_fp(x.data_ptr(), x.data_ptr(), 9, 4, 8, ALPHA, THRESH, None) == cabi.ERR_DTYPE
+    assert lib.snnlif_fire_s_fp(x.data_ptr(), x.data_ptr(), 0, -1, 8, ALPHA, THRESH, None) == cabi.ERR_ARG
+    assert lib.snnlif_fire_s_fp(x.data_ptr() + 2, x.data_ptr(), 0, 2, 4, ALPHA, THRESH, None) == cabi.ERR_ALIGN
+    big = torch.zeros(40, 8, device="cuda")
+    rc = lib.snnlif_fire_bp(big.data_ptr(), big.data_ptr(), big.data_ptr(), 0, 40, 8,
+                            ALPHA, THRESH, BETA, INTERVAL, None, 0, None)
+    assert rc == cabi.ERR_WORKSPACE
+    torch.cuda.synchronize()
+
+
+def test_misaligned_views_take_narrow_lanes(cabi, oracle):
+    """A base pointer that is only 4-byte aligned must still give the oracle's bits."""
+    x, g = make_inputs((8, 2, 1024), 0.5, 1.0, seed=5)
+    T, N = 8, 2048
+    pad = 1  # one float: 4-byte aligned, not 16
+    xd = torch.empty(T * N + pad, device="cuda")[pad:].view(T, 2, 1024).copy_(x)
+    gd = torch.empty(T * N + pad, device="cuda")[pad:].view(T, 2, 1024).copy_(g)
+    spike = torch.empty(T * N + pad, device="cuda")[pad:].view(T, 2, 1024)
+    gx = torch.empty(T * N + pad, device="cuda")[pad:].view(T, 2, 1024)
+    cabi.fire_s_fp_into(xd, spike, ALPHA, THRESH)
+    cabi.fire_bp_into(xd, gd, gx, ALPHA, THRESH, BETA, INTERVAL)
+    torch.cuda.synchronize()
+    _, spike_o = oracle.fire_forward(x.numpy(), ALPHA, THRESH)
+    gx_o = oracle.fire_backward(x.numpy(), g.numpy(), ALPHA, THRESH, BETA, INTERVAL)
+    assert np.array_equal(spike.cpu().numpy(), spike_o)
+    assert np.array_equal(gx.cpu().numpy(), gx_o)
