@@ -1,0 +1,225 @@
+#!/usr/bin/env python3
+"""Benchmark of the LIF fire forward+backward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg5_bf16|cfg1]
+                    [--no-cpu-baseline]
+
+One "step" is one forward (spikes from the input current) plus one backward (input gradient from
+the saved input current and the spike gradient) over one synthetic batch that is already resident
+in HBM, launched through the C ABI of ``libsnnlif_gfx950.so`` on PyTorch's current stream with
+pre-allocated outputs.  The default workload is the headline configuration
+``T=8, B=64, C=128, 32x32`` fp32.  Exactly one JSON line is printed on stdout.
+
+* ``value``      neuron-steps per second over the K timed steps (wall clock between two device
+                 synchronisations).
+* ``roofline``   the backward kernel (the dominant one): algorithmic bytes per launch
+                 (12 B x neuron-steps in fp32: read x, read grad_spike, write grad_x) divided by its
+                 mean duration, measured with HIP events recorded around every launch inside the
+                 timed region, against the 8 TB/s HBM peak.  ``fwd`` and ``fwd_bwd`` give the same
+                 figure for the forward kernel (8 B) and for the pair (20 B).
+* ``cpu_baseline`` the pure-PyTorch restatement of the reference's gold path
+                 (``oracle/gold_fire.py``) on the host cores, forward + autograd backward on the same
+                 inputs, best of 3 after a warm-up; its outputs also serve as the parity check of
+                 this very run (``parity``).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+HBM_PEAK_GBPS = 8000.0
+ALPHA, THRESH, BETA, INTERVAL = 0.25, 0.5, 1.0, 0.5
+SEED = 0
+
+# name -> (shape [T,B,C,H,W], input mean, input std, storage dtype name)
+WORKLOADS = {
+    "cfg1": ((4, 8, 16, 8, 8), 0.5, 1.0, "float32"),
+    "cfg2": ((8, 64, 128, 32, 32), 0.5, 1.0, "float32"),
+    "cfg3": ((32, 32, 256, 16, 16), 0.3, 0.8, "float32"),
+    "cfg5": ((16, 128, 512, 16, 16), 0.5, 1.0, "float32"),
+    "cfg5_bf16": ((16, 128, 512, 16, 16), 0.5, 1.0, "bfloat16"),
+}
+METRIC = "LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T=8,B=64,C=128,32x32"
+
+
+def make_inputs(torch, shape, mean, std, dtype):
+    """Seeded on the CPU so the host baseline and the GPU see identical bits."""
+    gen = torch.Generator().manual_seed(SEED)
+    x = torch.randn(shape, generator=gen).mul_(std).add_(mean).to(dtype)
+    g = torch.randn(shape, generator=gen).to(dtype)
+    return x, g
+
+
+def cpu_baseline(torch, x, g, repeats=3):
+    """Time oracle/gold_fire.py (forward + autograd backward) on the host; return timing + outputs."""
+    from oracle import gold_fire
+
+    xf, gf = x.float(), g.float()
+    threads = torch.get_num_threads()
+    best = None
+    outs = None
+    for it in range(repeats + 1):  # first pass is the warm-up
+        xr = xf.clone().requires_grad_(True)
+        t0 = time.perf_counter()
+        u, s = gold_fire.gold_fire(xr, ALPHA, THRESH, BETA, INTERVAL)
+        t1 = time.perf_counter()
+        s.backward(gf)
+        t2 = time.perf_counter()
+        if it > 0 and (best is None or (t2 - t0) < best[0]):
+            best = (t2 - t0, t1 - t0, t2 - t1)
+        outs = (s.detach(), xr.grad.detach())
+        del u, s, xr
+    return best, threads, outs
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the fire op needs no communication; "
+                 "neurons shard across GPUs with zero exchange). Run with --gpus 1.")
+
+    import torch
+    from snn_gpu_training_bptt_amd import lif_cabi
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no ROCm GPU visible")
+    lif_cabi.load()  # raises if the HIP library has not been built
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    shape, mean, std, dtype_name = WORKLOADS[args.workload]
+    dtype = getattr(torch, dtype_name)
+    T = shape[0]
+    n_steps_total = 1
+    for d in shape:
+        n_steps_total *= d  # neuron-steps per pass
+    esize = torch.empty((), dtype=dtype).element_size()
+    bytes_fwd = 2 * esize * n_steps_total
+    bytes_bwd = 3 * esize * n_steps_total
+
+    x_cpu, g_cpu = make_inputs(torch, shape, mean, std, dtype)
+    x = x_cpu.to(dev)
+    g = g_cpu.to(dev)
+    spike = torch.empty_like(x)
+    gx = torch.empty_like(x)
+    code = {torch.float32: lif_cabi.DTYPE_F32, torch.bfloat16: lif_cabi.DTYPE_BF16}[dtype]
+    ws_bytes = lif_cabi.fire_bp_workspace_bytes(code, T, n_steps_total // T)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+
+    def step():
+        lif_cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+        lif_cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    # Timed region: K steps; events around every launch give the per-kernel durations.
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        lif_cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+        ev[k][1].record()
+        lif_cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws)
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+
+    wall = t1 - t0
+    ms_per_step = wall / args.steps * 1e3
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    value = n_steps_total * args.steps / wall
+
+    def gbps(nbytes, ms):
+        return nbytes / (ms * 1e-3) / 1e9
+
+    bwd_gbps = gbps(bytes_bwd, bwd_ms)
+    fwd_gbps = gbps(bytes_fwd, fwd_ms)
+    pair_gbps = gbps(bytes_fwd + bytes_bwd, fwd_ms + bwd_ms)
+    spike_rate = float(spike.float().mean().item())
+
+    result = {
+        "metric": METRIC,
+        "value": value,
+        "unit": "neuron-steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32" if dtype == torch.float32 else "bf16-storage/f32-arithmetic",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: LIF fire fwd+bwd, [T,B,C,H,W]={list(shape)} {dtype_name}, "
+                        f"x~N({mean},{std}) g~N(0,1) seed {SEED}, alpha={ALPHA} thresh={THRESH} "
+                        f"beta={BETA} interval={INTERVAL}",
+            "neuron_steps_per_step": n_steps_total,
+            "spike_rate": round(spike_rate, 4),
+        },
+        "roofline": {
+            "kernel": "lif_backward_fused_kernel" if ws is None else "lif_backward_stream_kernel",
+            "bound": "hbm",
+            "achieved": bwd_gbps,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": bwd_gbps / HBM_PEAK_GBPS,
+            "traffic": None,
+            "algorithmic_bytes_per_launch": bytes_bwd,
+            "avg_launch_ms": bwd_ms,
+            "fwd": {"kernel": "lif_forward_kernel", "algorithmic_bytes_per_launch": bytes_fwd,
+                    "avg_launch_ms": fwd_ms, "achieved": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS},
+            "fwd_bwd": {"algorithmic_bytes": bytes_fwd + bytes_bwd, "kernel_ms": fwd_ms + bwd_ms,
+                        "achieved": pair_gbps, "frac": pair_gbps / HBM_PEAK_GBPS},
+        },
+    }
+
+    if not args.no_cpu_baseline:
+        best, threads, (s_ref, gx_ref) = cpu_baseline(torch, x_cpu, g_cpu)
+        total_s, fwd_s, bwd_s = best
+        s_gpu = spike.float().cpu()
+        gx_gpu = gx.float().cpu()
+        if dtype != torch.float32:  # storage rounding of the outputs is the only difference
+            gx_ref_cmp = gx_ref.to(dtype).float()
+        else:
+            gx_ref_cmp = gx_ref
+        denom = gx_ref_cmp.abs().clamp_min(1e-30)
+        result["cpu_baseline"] = {
+            "value": n_steps_total / total_s,
+            "unit": "neuron-steps/s",
+            "cores": threads,
+            "kind": "port",
+            "sample": f"the full {args.workload} tensor, forward + autograd backward of "
+                      f"oracle/gold_fire.py (pure PyTorch, fp32) on the host, 1 warm-up then best of 3",
+            "fwd_s": fwd_s,
+            "bwd_s": bwd_s,
+            "host_cpus": os.cpu_count(),
+        }
+        result["parity"] = {
+            "spikes_bit_exact": bool(torch.equal(s_gpu, s_ref)),
+            "spike_mismatches": int((s_gpu != s_ref).sum().item()),
+            "grad_bit_exact": bool(torch.equal(gx_gpu, gx_ref_cmp)),
+            "grad_max_rel_err": float(((gx_gpu - gx_ref_cmp).abs() / denom).max().item()),
+        }
+
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -2,8 +2,9 @@
 
 Two artefacts land next to this file:
 
-* ``libsnnlif_gfx950.so`` -- HIP kernels + C ABI (``csrc/lif_kernels.hip``, ``include/snnlib_lif.h``),
-  compiled by hipcc for gfx950 only;
+* ``libsnnlif_gfx950.so`` -- HIP kernels + C ABI (``csrc/lif_kernels.h`` instantiated by
+  ``csrc/lif_f32.hip``, ``lif_f64.hip``, ``lif_bf16.hip``; entry points in ``csrc/lif_abi.hip``,
+  declared in ``include/snnlib_lif.h``), compiled by hipcc for gfx950 only;
 * ``snnlib.so``           -- the Python extension module ``snnlib`` (``csrc/snnlib_ext.cpp``), host
   C++ against PyTorch-ROCm's headers, linked to the library above through ``$ORIGIN``.
 
@@ -15,6 +16,8 @@ import shutil
 import subprocess
 import sys
 import sysconfig
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_DIR = os.path.dirname(PKG_DIR)
@@ -26,10 +29,11 @@ EXT_LIB = os.path.join(PKG_DIR, "snnlib.so")
 # -ffp-contract=off: products and sums stay separately rounded (bit parity with per-op fp32).
 # -packed-fp32-ops off: keep the compiler from forming packed fp32 VALU instructions.
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-ffp-contract=off",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+KERNEL_SOURCES = ["lif_abi.hip", "lif_f32.hip", "lif_f64.hip", "lif_bf16.hip"]
 
 
 def _run(cmd, verbose):
@@ -55,10 +59,21 @@ def hipcc_path():
 
 
 def build_kernels(verbose=False, extra_flags=(), output=KERNEL_LIB):
-    """Compile the HIP kernels and their C ABI into ``libsnnlif_gfx950.so``."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, f"-I{INCLUDE}",
-           os.path.join(CSRC, "lif_kernels.hip"), "-o", output]
-    _run(cmd, verbose)
+    """Compile the HIP kernels and their C ABI into ``libsnnlif_gfx950.so``.
+
+    One object per translation unit (compiled in parallel), then one link step.
+    """
+    hipcc = hipcc_path()
+    with tempfile.TemporaryDirectory(prefix="snnlif_build_") as tmp:
+        def compile_one(src):
+            obj = os.path.join(tmp, os.path.splitext(src)[0] + ".o")
+            _run([hipcc, *HIPCC_FLAGS, *extra_flags, f"-I{INCLUDE}", "-c",
+                  os.path.join(CSRC, src), "-o", obj], verbose)
+            return obj
+
+        with ThreadPoolExecutor(max_workers=len(KERNEL_SOURCES)) as pool:
+            objects = list(pool.map(compile_one, KERNEL_SOURCES))
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", output], verbose)
     return output
 
 

@@ -1,0 +1,95 @@
+// C ABI of libsnnlif_gfx950.so (include/snnlib_lif.h): argument checks and dtype dispatch in front
+// of the per-dtype kernel launchers.  No device code lives in this file.
+#include "lif_kernels.h"
+
+namespace {
+
+inline size_t arith_size(int dtype) {
+    switch (dtype) {
+        case SNNLIF_DTYPE_F32: return sizeof(float);
+        case SNNLIF_DTYPE_F64: return sizeof(double);
+        case SNNLIF_DTYPE_BF16: return sizeof(float);
+        default: return 0;
+    }
+}
+
+inline int shape_error(int64_t T, int64_t N) {
+    if (T < 0 || N < 0) return SNNLIF_ERR_ARG;
+    if (T > 0x7fffffff) return SNNLIF_ERR_ARG;
+    if (T > 0 && N > (INT64_MAX / 16) / T) return SNNLIF_ERR_ARG;
+    return SNNLIF_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int snnlif_abi_version(void) { return SNNLIF_ABI_VERSION; }
+
+const char* snnlif_target_arch(void) { return "gfx950"; }
+
+const char* snnlif_strerror(int code) {
+    switch (code) {
+        case SNNLIF_OK: return "success";
+        case SNNLIF_ERR_ARG: return "snnlif: invalid argument (NULL tensor pointer, negative or overflowing T/N)";
+        case SNNLIF_ERR_DTYPE: return "snnlif: unsupported dtype (expected SNNLIF_DTYPE_F32, _F64 or _BF16)";
+        case SNNLIF_ERR_WORKSPACE: return "snnlif: workspace missing or smaller than snnlif_fire_bp_workspace_bytes()";
+        case SNNLIF_ERR_ALIGN: return "snnlif: pointer not aligned to its element size (workspace: 16 bytes)";
+        default: break;
+    }
+    if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
+    return "snnlif: unknown error code";
+}
+
+int snnlif_fire_us_fp(const void* spatial, void* mem, void* spike, int dtype, int64_t T, int64_t N,
+                      float alpha, float thresh, void* stream) {
+    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
+    const int se = shape_error(T, N);
+    if (se != SNNLIF_OK) return se;
+    if (T == 0 || N == 0) return SNNLIF_OK;
+    if (spatial == nullptr || (mem == nullptr && spike == nullptr)) return SNNLIF_ERR_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case SNNLIF_DTYPE_F32: return snnlif::forward_f32(spatial, mem, spike, T, N, alpha, thresh, st);
+        case SNNLIF_DTYPE_F64: return snnlif::forward_f64(spatial, mem, spike, T, N, alpha, thresh, st);
+        default: return snnlif::forward_bf16(spatial, mem, spike, T, N, alpha, thresh, st);
+    }
+}
+
+int snnlif_fire_s_fp(const void* spatial, void* spike, int dtype, int64_t T, int64_t N,
+                     float alpha, float thresh, void* stream) {
+    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
+    const int se = shape_error(T, N);
+    if (se != SNNLIF_OK) return se;
+    if (T == 0 || N == 0) return SNNLIF_OK;
+    if (spike == nullptr) return SNNLIF_ERR_ARG;
+    return snnlif_fire_us_fp(spatial, nullptr, spike, dtype, T, N, alpha, thresh, stream);
+}
+
+size_t snnlif_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t N) {
+    const size_t es = arith_size(dtype);
+    if (es == 0 || shape_error(T, N) != SNNLIF_OK) return 0;
+    if (T <= SNNLIF_BP_FUSED_MAX_T) return 0;
+    return static_cast<size_t>(T) * static_cast<size_t>(N) * es;
+}
+
+int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spatial, int dtype,
+                   int64_t T, int64_t N, float alpha, float thresh, float beta, float interval,
+                   void* workspace, size_t workspace_bytes, void* stream) {
+    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
+    const int se = shape_error(T, N);
+    if (se != SNNLIF_OK) return se;
+    if (T == 0 || N == 0) return SNNLIF_OK;
+    if (spatial == nullptr || grad_spike == nullptr || grad_spatial == nullptr) return SNNLIF_ERR_ARG;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case SNNLIF_DTYPE_F32:
+            return snnlif::backward_f32(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, workspace, workspace_bytes, st);
+        case SNNLIF_DTYPE_F64:
+            return snnlif::backward_f64(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, workspace, workspace_bytes, st);
+        default:
+            return snnlif::backward_bf16(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, workspace, workspace_bytes, st);
+    }
+}
+
+}  // extern "C"

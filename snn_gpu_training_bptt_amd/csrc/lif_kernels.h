@@ -1,0 +1,706 @@
+// LIF "fire" forward / backward kernels for MI355X (gfx950, CDNA4): templates shared by the
+// per-dtype translation units (lif_f32.hip, lif_f64.hip, lif_bf16.hip).
+//
+// What is computed (reference: snnlib/cuda/snn_kernel_fp.cu:37-52, snnlib/cuda/snn_kernel_bp.cu:34-51
+// and :117-138; pure-PyTorch statement of the same maths: snnlib/example/gold_op.py:17-44):
+//
+//   forward, per neuron, u = s = 0 before t = 0:
+//       u = (alpha * u) * (1 - s) + x[t];   s = (u > thresh);   spike[t] = s;   (mem[t] = u)
+//   backward, per neuron, gu = 0 before t = T-1, walking t downwards:
+//       gs = in_window(u[t]) ? g[t] - (gu * alpha) * u[t] : 0
+//       gu = gs * beta + (gu * alpha) * (u[t] <= thresh);   gx[t] = gu
+//       in_window(u) = (u - thresh) < interval && (thresh - u) < interval
+//
+// How it is mapped to the machine (nothing here follows the reference's launch geometry, which
+// gives one thread a (c,h,w) position and makes it loop serially over the batch):
+//   * Tensors are viewed as [T, N] with N = all neurons of the batch.  Neurons are independent and
+//     time is the only dependency, so a lane owns V consecutive neurons and walks T itself: the
+//     membrane potential, the spike flag and the running gradient never leave VGPRs.
+//   * A lane moves one dword per access (V = 1 float, 2 bf16; a double takes two dwords): a
+//     64-lane wavefront touches 256 consecutive bytes per time step, and all T rows (which are
+//     N*sizeof apart) are requested before the first value is consumed.  Measured on MI355X this
+//     beats 16-byte lanes by 5-15 %: the narrow kernels need ~25 VGPRs, so every SIMD holds its full
+//     8 waves, and the many small in-flight requests of one wave stay within a few DRAM pages per
+//     row instead of spreading over sixteen.  It also removes every alignment constraint for fp32
+//     and fp64 (element alignment is all a dword lane needs).
+//   * The backward recomputes u[0..T-1] from x into registers (T <= 32) instead of writing a
+//     membrane tensor to HBM and reading it back: 12 bytes per neuron-step instead of 20.
+//     Gradient rows are streamed in reverse time order through a double-buffered register window.
+//     The register-resident window needs compile-time row indices, so the kernel is instantiated
+//     per window length; lengths without an instantiation of their own run the next larger one
+//     with the missing rows replaced by zeros (no per-row control flow around live registers,
+//     which costs the compiler hundreds of VGPRs).
+//   * The op is element-wise and HBM-bound: no LDS, no cross-lane traffic, no MFMA.
+//   * Cache policy per stream: spikes and gradients are touched once and carry the non-temporal
+//     hint; the input current x is read by the forward and again by the backward, so when it fits
+//     the 256 MB memory-side cache it is loaded with the default policy and left there.
+//   * Built with -ffp-contract=off: each product and sum is rounded on its own, as PyTorch's
+//     element-wise CPU/GPU ops do, which makes spikes, potentials and gradients bit-identical to
+//     the per-op rounded reference arithmetic.
+//
+// Longer windows (T > 32) use the same forward kernel to write u to a caller-provided workspace
+// and a streaming reverse kernel that reads it back.
+#ifndef SNNLIF_LIF_KERNELS_H
+#define SNNLIF_LIF_KERNELS_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstddef>
+#include <cstdint>
+#include <type_traits>
+
+#include "snnlib_lif.h"
+
+// Bytes one lane moves per memory instruction (storage types narrower than this are packed).
+#ifndef SNNLIF_LANE_BYTES
+#define SNNLIF_LANE_BYTES 4
+#endif
+// Threads per workgroup of the forward / backward kernels.
+#ifndef SNNLIF_FWD_BLOCK
+#define SNNLIF_FWD_BLOCK 256
+#endif
+#ifndef SNNLIF_BWD_BLOCK
+#define SNNLIF_BWD_BLOCK 256
+#endif
+// The input current x is the one tensor that is read twice (by the forward, then again by the
+// backward's recomputation).  When it is at most this many bytes it is loaded with the default
+// cache policy so that it may stay in the 256 MB memory-side cache between the two kernels; every
+// other stream (spikes, incoming and outgoing gradients, and x itself when it is larger) is
+// touched once and carries the non-temporal hint so that it does not displace x.
+#ifndef SNNLIF_KEEP_INPUT_BYTES
+#define SNNLIF_KEEP_INPUT_BYTES (int64_t(256) << 20)
+#endif
+// VGPR budget (in 32-bit words) the fused backward may spend on the recomputed membrane potential.
+#ifndef SNNLIF_FUSED_U_WORDS
+#define SNNLIF_FUSED_U_WORDS 128
+#endif
+// Rows of x the forward requests before consuming the first (windows longer than this are
+// streamed with the next group of rows in flight).
+#ifndef SNNLIF_FWD_ROWS
+#define SNNLIF_FWD_ROWS 8
+#endif
+// Rows of the gradient held in flight per buffer of the backward's reverse sweep.
+#ifndef SNNLIF_BWD_GCHUNK
+#define SNNLIF_BWD_GCHUNK 8
+#endif
+
+namespace snnlif {
+
+constexpr int kLaneBytes = SNNLIF_LANE_BYTES;
+constexpr int lane_vec(size_t elem_bytes) {
+    return kLaneBytes / static_cast<int>(elem_bytes) < 1 ? 1 : kLaneBytes / static_cast<int>(elem_bytes);
+}
+constexpr int kFwdBlock = SNNLIF_FWD_BLOCK;
+constexpr int kBwdBlock = SNNLIF_BWD_BLOCK;
+
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// bfloat16 as raw bits; conversions are done by hand so the rounding is spelled out.
+struct bf16_t {
+    uint16_t bits;
+};
+
+template <int BYTES> struct RawOf;
+template <> struct RawOf<2>  { using type = uint16_t; };
+template <> struct RawOf<4>  { using type = uint32_t; };
+template <> struct RawOf<8>  { using type = u32x2; };
+template <> struct RawOf<16> { using type = u32x4; };
+
+// V consecutive elements of storage type S, moved with one memory instruction.
+template <typename S, int V>
+struct Pack {
+    using raw_t = typename RawOf<sizeof(S) * V>::type;
+    union {
+        raw_t raw;
+        S e[V];
+    };
+};
+
+template <typename S, int V>
+__device__ __forceinline__ Pack<S, V> zero_pack() {
+    Pack<S, V> r;
+    r.raw = typename Pack<S, V>::raw_t(0);
+    return r;
+}
+
+// STREAM = true: single-use data, non-temporal hint.  STREAM = false: default policy (may be kept
+// by the caches for a later reader).
+template <typename S, int V, bool STREAM>
+__device__ __forceinline__ Pack<S, V> load_pack(const S* p) {
+    using raw_t = typename Pack<S, V>::raw_t;
+    Pack<S, V> r;
+    if (STREAM) {
+        r.raw = __builtin_nontemporal_load(reinterpret_cast<const raw_t*>(p));
+    } else {
+        r.raw = *reinterpret_cast<const raw_t*>(p);
+    }
+    return r;
+}
+
+template <typename S, int V>
+__device__ __forceinline__ void store_pack(S* p, const Pack<S, V>& v) {
+    using raw_t = typename Pack<S, V>::raw_t;
+    __builtin_nontemporal_store(v.raw, reinterpret_cast<raw_t*>(p));
+}
+
+// Storage type -> arithmetic type and conversions.
+template <typename S> struct Arith;
+template <> struct Arith<float> {
+    using type = float;
+    static constexpr int kMaxVec = lane_vec(sizeof(float));
+    __device__ static __forceinline__ float load(float v) { return v; }
+    __device__ static __forceinline__ float store(float v) { return v; }
+};
+template <> struct Arith<double> {
+    using type = double;
+    static constexpr int kMaxVec = lane_vec(sizeof(double));
+    __device__ static __forceinline__ double load(double v) { return v; }
+    __device__ static __forceinline__ double store(double v) { return v; }
+};
+template <> struct Arith<bf16_t> {
+    using type = float;
+    static constexpr int kMaxVec = lane_vec(sizeof(uint16_t));
+    __device__ static __forceinline__ float load(bf16_t v) {
+        return __uint_as_float(static_cast<uint32_t>(v.bits) << 16);
+    }
+    // Round to nearest, ties to even; every NaN becomes the canonical quiet NaN 0x7FC0.
+    __device__ static __forceinline__ bf16_t store(float f) {
+        uint32_t u = __float_as_uint(f);
+        bf16_t r;
+        if ((u & 0x7fffffffu) > 0x7f800000u) {
+            r.bits = 0x7fc0;
+        } else {
+            u += 0x7fffu + ((u >> 16) & 1u);
+            r.bits = static_cast<uint16_t>(u >> 16);
+        }
+        return r;
+    }
+};
+
+// One forward step for one neuron, in the reference's association:
+// ((alpha * u) * (1 - s)) + x, then the strict comparison.
+template <typename C>
+__device__ __forceinline__ void lif_step(C& u, C& s, C x, C alpha, C thresh) {
+    u = (alpha * u) * (C(1) - s) + x;
+    s = (u > thresh) ? C(1) : C(0);
+}
+
+// One reverse step for one neuron, given the membrane potential u of that step and the incoming
+// spike gradient g; gu is the gradient carried from step t+1 and becomes the result of step t.
+template <typename C>
+__device__ __forceinline__ void lif_reverse_step(C& gu, C u, C g, C alpha, C thresh, C beta,
+                                                 C interval) {
+    const C gua = gu * alpha;
+    C gs = C(0);
+    if ((u - thresh) < interval && (thresh - u) < interval) {
+        gs = g - gua * u;
+    }
+    gu = gs * beta + gua * ((u <= thresh) ? C(1) : C(0));
+}
+
+// ---------------------------------------------------------------------------------------------
+// Forward.  S: storage type of x / spike, M: storage type of the membrane output (S for the
+// public op, the arithmetic type when it is the backward's workspace), V: neurons per lane,
+// TC: rows requested before the first is consumed.  MULTI = false: the whole window fits in TC
+// rows.  MULTI = true: the window is streamed TC rows at a time with the next TC rows already in
+// flight while the current ones are processed.  KEEPX: load x with the default cache policy.
+// ---------------------------------------------------------------------------------------------
+template <typename S, typename M, int V, int TC, bool MULTI, bool KEEPX, bool WRITE_U, bool WRITE_S>
+__global__ void __launch_bounds__(kFwdBlock)
+lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__ spike, int T,
+                   int64_t N, int64_t nvec, typename Arith<S>::type alpha,
+                   typename Arith<S>::type thresh) {
+    using C = typename Arith<S>::type;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kFwdBlock;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * kFwdBlock + threadIdx.x; v < nvec;
+         v += stride) {
+        const int64_t col = v * V;
+        C u[V], s[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            u[j] = C(0);
+            s[j] = C(0);
+        }
+        Pack<S, V> cur[TC];
+        Pack<S, V> nxt[MULTI ? TC : 1];
+#pragma unroll
+        for (int k = 0; k < TC; ++k) {
+            if (k < T) cur[k] = load_pack<S, V, !KEEPX>(x + static_cast<int64_t>(k) * N + col);
+        }
+        for (int t0 = 0; t0 < T; t0 += TC) {
+            if (MULTI && t0 + TC < T) {
+#pragma unroll
+                for (int k = 0; k < TC; ++k) {
+                    const int t = t0 + TC + k;
+                    if (t < T)
+                        nxt[MULTI ? k : 0] =
+                            load_pack<S, V, !KEEPX>(x + static_cast<int64_t>(t) * N + col);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < TC; ++k) {
+                const int t = t0 + k;
+                if (t < T) {
+                    Pack<M, V> mo;
+                    Pack<S, V> so;
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        lif_step<C>(u[j], s[j], Arith<S>::load(cur[k].e[j]), alpha, thresh);
+                        if (WRITE_U) mo.e[j] = Arith<M>::store(u[j]);
+                        if (WRITE_S) so.e[j] = Arith<S>::store(s[j]);
+                    }
+                    const int64_t off = static_cast<int64_t>(t) * N + col;
+                    if (WRITE_U) store_pack<M, V>(mem + off, mo);
+                    if (WRITE_S) store_pack<S, V>(spike + off, so);
+                }
+            }
+            if (!MULTI) break;
+            if (t0 + TC < T) {
+#pragma unroll
+                for (int k = 0; k < TC; ++k) cur[k] = nxt[MULTI ? k : 0];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Fused backward for a window of at most TW rows: recompute u[0..T-1] into registers, then sweep t
+// downwards.  EXACT = true: T == TW, straight-line code.  EXACT = false: T < TW; rows t >= T are
+// not fetched (zeros stand in for them), the recomputation runs over all TW rows (rows past T only
+// produce values nobody reads) and the reverse sweep skips them.
+// Gradient rows are fetched in groups of at most GC, the newest time steps first; the fetch of the
+// next (earlier) group is issued before the current group is consumed.
+// ---------------------------------------------------------------------------------------------
+template <typename S, int V, int TW, bool EXACT, bool KEEPX>
+__global__ void __launch_bounds__(kBwdBlock)
+lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
+                          int T, int64_t N, int64_t nvec, typename Arith<S>::type alpha,
+                          typename Arith<S>::type thresh, typename Arith<S>::type beta,
+                          typename Arith<S>::type interval) {
+    using C = typename Arith<S>::type;
+    constexpr int GC = (TW < SNNLIF_BWD_GCHUNK) ? TW : SNNLIF_BWD_GCHUNK;
+    constexpr int NG = (TW + GC - 1) / GC;  // groups; group 0 holds the newest rows
+    // group q covers rows [lo(q), hi(q)) with hi(q) = TW - q*GC and lo(q) = max(0, hi(q) - GC)
+
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < nvec;
+         v += stride) {
+        const int64_t col = v * V;
+
+        Pack<S, V> xin[TW];
+#pragma unroll
+        for (int t = 0; t < TW; ++t) {
+            if (EXACT) {
+                xin[t] = load_pack<S, V, !KEEPX>(x + static_cast<int64_t>(t) * N + col);
+            } else {
+                xin[t] = zero_pack<S, V>();
+                if (t < T) xin[t] = load_pack<S, V, !KEEPX>(x + static_cast<int64_t>(t) * N + col);
+            }
+        }
+        Pack<S, V> gbuf[2][GC];
+#pragma unroll
+        for (int t = TW - 1; t >= ((TW - GC) > 0 ? (TW - GC) : 0); --t) {
+            const int k = t - ((TW - GC) > 0 ? (TW - GC) : 0);
+            if (EXACT) {
+                gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+            } else {
+                gbuf[0][k] = zero_pack<S, V>();
+                if (t < T) gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+            }
+        }
+
+        C u[TW][V];
+        {
+            C uc[V], sc[V];
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                uc[j] = C(0);
+                sc[j] = C(0);
+            }
+#pragma unroll
+            for (int t = 0; t < TW; ++t) {
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    lif_step<C>(uc[j], sc[j], Arith<S>::load(xin[t].e[j]), alpha, thresh);
+                    u[t][j] = uc[j];
+                }
+            }
+        }
+
+        C gu[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) gu[j] = C(0);
+
+#pragma unroll
+        for (int q = 0; q < NG; ++q) {
+            const int hi = TW - q * GC;
+            const int lo = (hi - GC) > 0 ? (hi - GC) : 0;
+            if (q + 1 < NG) {
+                const int nhi = lo;
+                const int nlo = (nhi - GC) > 0 ? (nhi - GC) : 0;
+#pragma unroll
+                for (int t = nhi - 1; t >= nlo; --t) {
+                    if (EXACT) {
+                        gbuf[(q + 1) & 1][t - nlo] =
+                            load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+                    } else {
+                        gbuf[(q + 1) & 1][t - nlo] = zero_pack<S, V>();
+                        if (t < T)
+                            gbuf[(q + 1) & 1][t - nlo] =
+                                load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+                    }
+                }
+            }
+#pragma unroll
+            for (int t = hi - 1; t >= lo; --t) {
+                if (EXACT || t < T) {
+                    Pack<S, V> out;
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        lif_reverse_step<C>(gu[j], u[t][j],
+                                            Arith<S>::load(gbuf[q & 1][t - lo].e[j]), alpha, thresh,
+                                            beta, interval);
+                        out.e[j] = Arith<S>::store(gu[j]);
+                    }
+                    store_pack<S, V>(gx + static_cast<int64_t>(t) * N + col, out);
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Streaming backward for long windows: the membrane potential comes from a workspace written by
+// lif_forward_kernel<.., WRITE_U>.  Rows are consumed TC at a time from the end of the window.
+// ---------------------------------------------------------------------------------------------
+template <typename S, int V, int TC>
+__global__ void __launch_bounds__(kBwdBlock)
+lif_backward_stream_kernel(const typename Arith<S>::type* __restrict__ mem,
+                           const S* __restrict__ g, S* __restrict__ gx, int T, int64_t N,
+                           int64_t nvec, typename Arith<S>::type alpha,
+                           typename Arith<S>::type thresh, typename Arith<S>::type beta,
+                           typename Arith<S>::type interval) {
+    using C = typename Arith<S>::type;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < nvec;
+         v += stride) {
+        const int64_t col = v * V;
+        C gu[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) gu[j] = C(0);
+
+        // Group c covers t in [c*TC, c*TC + TC); the last group may be partial.
+        const int ngroups = (T + TC - 1) / TC;
+        Pack<C, V> mcur[TC], mnxt[TC];
+        Pack<S, V> gcur[TC], gnxt[TC];
+#pragma unroll
+        for (int k = TC - 1; k >= 0; --k) {
+            const int t = (ngroups - 1) * TC + k;
+            mcur[k] = zero_pack<C, V>();
+            gcur[k] = zero_pack<S, V>();
+            if (t < T) {
+                mcur[k] = load_pack<C, V, true>(mem + static_cast<int64_t>(t) * N + col);
+                gcur[k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+            }
+        }
+        for (int c = ngroups - 1; c >= 0; --c) {
+            if (c > 0) {
+#pragma unroll
+                for (int k = TC - 1; k >= 0; --k) {
+                    const int64_t off = static_cast<int64_t>((c - 1) * TC + k) * N + col;
+                    mnxt[k] = load_pack<C, V, true>(mem + off);
+                    gnxt[k] = load_pack<S, V, true>(g + off);
+                }
+            }
+#pragma unroll
+            for (int k = TC - 1; k >= 0; --k) {
+                const int t = c * TC + k;
+                if (t < T) {
+                    Pack<S, V> out;
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        lif_reverse_step<C>(gu[j], mcur[k].e[j], Arith<S>::load(gcur[k].e[j]),
+                                            alpha, thresh, beta, interval);
+                        out.e[j] = Arith<S>::store(gu[j]);
+                    }
+                    store_pack<S, V>(gx + static_cast<int64_t>(t) * N + col, out);
+                }
+            }
+            if (c > 0) {
+#pragma unroll
+                for (int k = 0; k < TC; ++k) {
+                    mcur[k] = mnxt[k];
+                    gcur[k] = gnxt[k];
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Host side: vector-width selection and launches.
+// ---------------------------------------------------------------------------------------------
+
+// Upper bound on blocks per launch; beyond it lanes take further columns in the grid-stride loop.
+constexpr int64_t kMaxGrid = int64_t(1) << 24;
+
+inline unsigned grid_for(int64_t nvec, int block) {
+    int64_t blocks = (nvec + block - 1) / block;
+    if (blocks > kMaxGrid) blocks = kMaxGrid;
+    if (blocks < 1) blocks = 1;
+    return static_cast<unsigned>(blocks);
+}
+
+inline bool aligned_to(const void* p, size_t bytes) {
+    return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
+}
+
+// Largest power-of-two V <= maxv such that rows (N elements apart) and the bases of all given
+// pointers stay aligned to V elements.  elem[i] is the element size behind ptrs[i].
+inline int pick_vec(int maxv, int64_t N, const void* const* ptrs, const size_t* elem, int n) {
+    int v = maxv;
+    while (v > 1) {
+        bool ok = (N % v) == 0;
+        for (int i = 0; ok && i < n; ++i) ok = aligned_to(ptrs[i], elem[i] * v);
+        if (ok) break;
+        v >>= 1;
+    }
+    return v;
+}
+
+inline int launch_status() {
+    return static_cast<int>(hipGetLastError());
+}
+
+// Whether x is small enough to be left in the memory-side cache for its second reader.
+template <typename S>
+inline bool keep_input(int64_t T, int64_t N) {
+    return T * N <= SNNLIF_KEEP_INPUT_BYTES / static_cast<int64_t>(sizeof(S));
+}
+
+// Calls f(std::integral_constant<int, v>) for the runtime vector width v in {MAXV, MAXV/2, .., 1}.
+template <int MAXV, typename F>
+inline int with_vec(int v, F&& f) {
+    if constexpr (MAXV >= 8) {
+        if (v == 8) return f(std::integral_constant<int, 8>());
+    }
+    if constexpr (MAXV >= 4) {
+        if (v == 4) return f(std::integral_constant<int, 4>());
+    }
+    if constexpr (MAXV >= 2) {
+        if (v == 2) return f(std::integral_constant<int, 2>());
+    }
+    return f(std::integral_constant<int, 1>());
+}
+
+template <typename S, typename M, int V, bool KEEPX, bool WRITE_U, bool WRITE_S>
+int launch_forward_vk(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
+                      hipStream_t stream) {
+    using C = typename Arith<S>::type;
+    const int64_t nvec = N / V;
+    const dim3 grid(grid_for(nvec, kFwdBlock)), block(kFwdBlock);
+    const int Ti = static_cast<int>(T);
+    constexpr int TC = SNNLIF_FWD_ROWS;
+    if (T <= 4 && TC > 4) {
+        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, 4, false, KEEPX, WRITE_U, WRITE_S>), grid,
+                           block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
+    } else if (T <= TC) {
+        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, TC, false, KEEPX, WRITE_U, WRITE_S>), grid,
+                           block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
+    } else {
+        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, TC, true, KEEPX, WRITE_U, WRITE_S>), grid,
+                           block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
+    }
+    return launch_status();
+}
+
+template <typename S, typename M, bool WRITE_U, bool WRITE_S>
+int launch_forward(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
+                   hipStream_t stream) {
+    // lanes are sized by the narrower of the two element types; the wider one (the fp32 workspace
+    // behind bf16 storage) then moves V of its elements, at most 16 bytes
+    constexpr size_t narrowest = sizeof(S) < sizeof(M) ? sizeof(S) : sizeof(M);
+    constexpr size_t widest = sizeof(S) > sizeof(M) ? sizeof(S) : sizeof(M);
+    constexpr int maxv = lane_vec(narrowest) < static_cast<int>(16 / widest)
+                             ? lane_vec(narrowest)
+                             : static_cast<int>(16 / widest);
+    const void* ptrs[3] = {x, WRITE_U ? mem : nullptr, WRITE_S ? spike : nullptr};
+    const size_t elem[3] = {sizeof(S), sizeof(M), sizeof(S)};
+    for (int i = 0; i < 3; ++i)
+        if (!aligned_to(ptrs[i], elem[i])) return SNNLIF_ERR_ALIGN;
+    const int v = pick_vec(maxv, N, ptrs, elem, 3);
+    // Only full-width lanes get the cache-resident variant; narrow lanes are the odd-shape path.
+    const bool keep = (v == maxv) && keep_input<S>(T, N);
+    return with_vec<maxv>(v, [&](auto vc) {
+        constexpr int V = decltype(vc)::value;
+        if constexpr (V == maxv) {
+            if (keep)
+                return launch_forward_vk<S, M, V, true, WRITE_U, WRITE_S>(x, mem, spike, T, N, alpha,
+                                                                           thresh, stream);
+        }
+        return launch_forward_vk<S, M, V, false, WRITE_U, WRITE_S>(x, mem, spike, T, N, alpha,
+                                                                    thresh, stream);
+    });
+}
+
+template <typename S>
+int forward_dispatch(const void* x, void* mem, void* spike, int64_t T, int64_t N, float alpha,
+                     float thresh, hipStream_t stream) {
+    const S* xs = static_cast<const S*>(x);
+    S* ms = static_cast<S*>(mem);
+    S* ss = static_cast<S*>(spike);
+    if (mem != nullptr && spike != nullptr)
+        return launch_forward<S, S, true, true>(xs, ms, ss, T, N, alpha, thresh, stream);
+    if (mem != nullptr)
+        return launch_forward<S, S, true, false>(xs, ms, nullptr, T, N, alpha, thresh, stream);
+    return launch_forward<S, S, false, true>(xs, nullptr, ss, T, N, alpha, thresh, stream);
+}
+
+// Register budget of the fused backward: TW*V arithmetic values for u plus two gradient
+// buffers.  V is capped so that u stays within SNNLIF_FUSED_U_WORDS VGPRs.
+template <typename S, int TW>
+constexpr int fused_max_vec() {
+    using C = typename Arith<S>::type;
+    constexpr int words = static_cast<int>(sizeof(C) / 4);
+    constexpr int cap = SNNLIF_FUSED_U_WORDS / (TW * words);
+    constexpr int hw = Arith<S>::kMaxVec;
+    return cap < 1 ? 1 : (cap < hw ? cap : hw);
+}
+
+template <typename S, int TW>
+int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, float alpha,
+                          float thresh, float beta, float interval, hipStream_t stream) {
+    using C = typename Arith<S>::type;
+    constexpr int maxv = fused_max_vec<S, TW>();
+    const void* ptrs[3] = {x, g, gx};
+    const size_t elem[3] = {sizeof(S), sizeof(S), sizeof(S)};
+    const int v = pick_vec(maxv, N, ptrs, elem, 3);
+    const bool keep = (v == maxv) && keep_input<S>(T, N);
+    // Every window of at most 8 rows has an instantiation of its own, so only the longer ones
+    // are ever entered with T < TW.
+    constexpr bool can_be_inexact = TW > 8;
+    const bool exact = !can_be_inexact || (T == TW);
+    return with_vec<maxv>(v, [&](auto vc) {
+        constexpr int V = decltype(vc)::value;
+        const int64_t nvec = N / V;
+        const dim3 grid(grid_for(nvec, kBwdBlock)), block(kBwdBlock);
+        const int Ti = static_cast<int>(T);
+#define SNNLIF_LAUNCH_BWD(EXACT_, KEEP_)                                                         \
+    hipLaunchKernelGGL((lif_backward_fused_kernel<S, V, TW, EXACT_, KEEP_>), grid, block, 0,     \
+                       stream, x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval))
+        if constexpr (V == maxv) {
+            if (keep) {
+                if (exact) {
+                    SNNLIF_LAUNCH_BWD(true, true);
+                } else if constexpr (can_be_inexact) {
+                    SNNLIF_LAUNCH_BWD(false, true);
+                }
+                return launch_status();
+            }
+        }
+        if (exact) {
+            SNNLIF_LAUNCH_BWD(true, false);
+        } else if constexpr (can_be_inexact) {
+            SNNLIF_LAUNCH_BWD(false, false);
+        }
+#undef SNNLIF_LAUNCH_BWD
+        return launch_status();
+    });
+}
+
+template <typename S, int V>
+int launch_backward_stream_v(const typename Arith<S>::type* mem, const S* g, S* gx, int64_t T,
+                             int64_t N, float alpha, float thresh, float beta, float interval,
+                             hipStream_t stream) {
+    using C = typename Arith<S>::type;
+    const int64_t nvec = N / V;
+    hipLaunchKernelGGL((lif_backward_stream_kernel<S, V, 8>), dim3(grid_for(nvec, kBwdBlock)),
+                       dim3(kBwdBlock), 0, stream, mem, g, gx, static_cast<int>(T), N, nvec,
+                       C(alpha), C(thresh), C(beta), C(interval));
+    return launch_status();
+}
+
+template <typename S>
+int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int64_t N, float alpha,
+                      float thresh, float beta, float interval, void* workspace,
+                      size_t workspace_bytes, hipStream_t stream) {
+    using C = typename Arith<S>::type;
+    const S* x = static_cast<const S*>(x_);
+    const S* g = static_cast<const S*>(g_);
+    S* gx = static_cast<S*>(gx_);
+    if (!aligned_to(x, sizeof(S)) || !aligned_to(g, sizeof(S)) || !aligned_to(gx, sizeof(S)))
+        return SNNLIF_ERR_ALIGN;
+
+    // Window lengths with an instantiation of their own; any other T <= 32 runs the next larger
+    // one in its zero-filled form.
+#define SNNLIF_BWD_WINDOW(TW)                                                                    \
+    if (T <= TW)                                                                                 \
+        return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, stream);
+    SNNLIF_BWD_WINDOW(1)
+    SNNLIF_BWD_WINDOW(2)
+    SNNLIF_BWD_WINDOW(3)
+    SNNLIF_BWD_WINDOW(4)
+    SNNLIF_BWD_WINDOW(5)
+    SNNLIF_BWD_WINDOW(6)
+    SNNLIF_BWD_WINDOW(7)
+    SNNLIF_BWD_WINDOW(8)
+    SNNLIF_BWD_WINDOW(10)
+    SNNLIF_BWD_WINDOW(12)
+    SNNLIF_BWD_WINDOW(16)
+    SNNLIF_BWD_WINDOW(20)
+    SNNLIF_BWD_WINDOW(24)
+    SNNLIF_BWD_WINDOW(28)
+    SNNLIF_BWD_WINDOW(32)
+#undef SNNLIF_BWD_WINDOW
+    static_assert(SNNLIF_BP_FUSED_MAX_T == 32, "windows above must cover the fused range");
+
+    // Long window: u -> workspace (arithmetic type), then the streaming reverse sweep.
+    const size_t need = static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(C);
+    if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
+    if (!aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
+    C* mem = static_cast<C*>(workspace);
+    int rc = launch_forward<S, C, true, false>(x, mem, nullptr, T, N, alpha, thresh, stream);
+    if (rc != SNNLIF_OK) return rc;
+
+    constexpr int maxv = Arith<S>::kMaxVec < static_cast<int>(16 / sizeof(C))
+                             ? Arith<S>::kMaxVec
+                             : static_cast<int>(16 / sizeof(C));
+    const void* ptrs[3] = {mem, g, gx};
+    const size_t elem[3] = {sizeof(C), sizeof(S), sizeof(S)};
+    const int v = pick_vec(maxv, N, ptrs, elem, 3);
+    return with_vec<maxv>(v, [&](auto vc) {
+        constexpr int V = decltype(vc)::value;
+        return launch_backward_stream_v<S, V>(mem, g, gx, T, N, alpha, thresh, beta, interval,
+                                              stream);
+    });
+}
+
+// Entry points of the per-dtype translation units (defined in lif_f32.hip, lif_f64.hip,
+// lif_bf16.hip; called from lif_abi.hip).
+#define SNNLIF_DECLARE_DTYPE(NAME)                                                                  \
+    int forward_##NAME(const void* x, void* mem, void* spike, int64_t T, int64_t N, float alpha,    \
+                       float thresh, hipStream_t stream);                                           \
+    int backward_##NAME(const void* x, const void* g, void* gx, int64_t T, int64_t N, float alpha,  \
+                        float thresh, float beta, float interval, void* workspace,                  \
+                        size_t workspace_bytes, hipStream_t stream);
+SNNLIF_DECLARE_DTYPE(f32)
+SNNLIF_DECLARE_DTYPE(f64)
+SNNLIF_DECLARE_DTYPE(bf16)
+#undef SNNLIF_DECLARE_DTYPE
+
+#define SNNLIF_DEFINE_DTYPE(NAME, S)                                                                \
+    int forward_##NAME(const void* x, void* mem, void* spike, int64_t T, int64_t N, float alpha,    \
+                       float thresh, hipStream_t stream) {                                          \
+        return forward_dispatch<S>(x, mem, spike, T, N, alpha, thresh, stream);                     \
+    }                                                                                               \
+    int backward_##NAME(const void* x, const void* g, void* gx, int64_t T, int64_t N, float alpha,  \
+                        float thresh, float beta, float interval, void* workspace,                  \
+                        size_t workspace_bytes, hipStream_t stream) {                               \
+        return backward_dispatch<S>(x, g, gx, T, N, alpha, thresh, beta, interval, workspace,       \
+                                    workspace_bytes, stream);                                       \
+    }
+
+}  // namespace snnlif
+
+#endif  // SNNLIF_LIF_KERNELS_H

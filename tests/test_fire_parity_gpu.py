@@ -91,6 +91,15 @@ def test_fp32_parity(cabi, oracle, shape, mean, std):
     assert_parity(oracle, x, g, run_gpu(cabi, x, g))
 
 
+@pytest.mark.parametrize("T", list(range(1, 35)))
+def test_fp32_every_window_length(cabi, oracle, T):
+    """Each window length up to 32 maps to its own or the next larger register window; 33 and 34
+    take the workspace path.  Full-width lanes (N % 4 == 0) and scalar lanes (odd N)."""
+    for n_inner in (256, 77):
+        x, g = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=1000 + T)
+        assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
+
+
 @pytest.mark.parametrize("alpha,thresh,beta,interval", [
     (0.3, 0.5, 1.0, 0.5),      # decay that is not a power of two: exposes any FMA contraction
     (0.25, 0.25, 1.0, 0.5),    # the reference's default threshold (snnlib_func.py:14)
