@@ -84,6 +84,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain device copies of the input tensor (known size: one "
+                         "read + one write of it) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
+                         "readings can be scaled to bytes")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -125,6 +129,13 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+
+    if args.copy_calibration:
+        scratch_copy = torch.empty_like(x)
+        for _ in range(3):
+            scratch_copy.copy_(x)
+        torch.cuda.synchronize()
+        del scratch_copy
 
     # Timed region: K steps; events around every launch give the per-kernel durations.
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
