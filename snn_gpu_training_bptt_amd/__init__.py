@@ -1,8 +1,8 @@
 """LIF "fire" forward / backward operators of snnlib as hand-written HIP kernels for MI355X.
 
 Layout
-    csrc/lif_kernels.hip   kernels + C ABI            -> libsnnlif_gfx950.so  (include/snnlib_lif.h)
-    csrc/snnlib_ext.cpp    PyTorch-ROCm binding       -> snnlib.so            (module ``snnlib``)
+    csrc/lif_*.hip, lif_kernels.h   kernels + C ABI            -> lib/libsnnlif_gfx950.so  (include/snnlib_lif.h)
+    csrc/snnlib_ext.cpp    PyTorch-ROCm binding       -> lib/snnlib.so            (module ``snnlib``)
     lif_cabi.py            ctypes view of the C ABI
     snnlib_func.py         ``FireFunc`` / ``fire_func`` / hyper-parameters
     snnlib_op.py           ``Fire`` layer module

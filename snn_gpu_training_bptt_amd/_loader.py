@@ -2,7 +2,7 @@
 
 The reference installs its extension as a top-level module and ``snnlib_func.py`` does
 ``import snnlib`` (snnlib/example/snnlib_func.py:8).  Here the module is built in-tree as
-``snn_gpu_training_bptt_amd/snnlib.so``; it is loaded under the same top-level name and registered
+``snn_gpu_training_bptt_amd/lib/snnlib.so``; it is loaded under the same top-level name and registered
 in ``sys.modules`` so that reference-style code doing ``import snnlib`` afterwards gets this build.
 There is no fallback: without the built extension the import fails.
 """
@@ -12,7 +12,7 @@ import os
 import sys
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-EXT_PATH = os.path.join(PKG_DIR, "snnlib.so")
+EXT_PATH = os.path.join(PKG_DIR, "lib", "snnlib.so")
 
 
 def load_snnlib():

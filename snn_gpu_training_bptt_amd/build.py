@@ -1,6 +1,7 @@
 """In-tree build of the native pieces (no setuptools, no JIT cache).
 
-Two artefacts land next to this file:
+Two artefacts land in ``lib/`` next to this file (a directory that holds nothing else, so it can
+be put on ``sys.path`` to make ``import snnlib`` work for reference-style code):
 
 * ``libsnnlif_gfx950.so`` -- HIP kernels + C ABI (``csrc/lif_kernels.h`` instantiated by
   ``csrc/lif_f32.hip``, ``lif_f64.hip``, ``lif_bf16.hip``; entry points in ``csrc/lif_abi.hip``,
@@ -23,8 +24,9 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 REPO_DIR = os.path.dirname(PKG_DIR)
 CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(REPO_DIR, "include")
-KERNEL_LIB = os.path.join(PKG_DIR, "libsnnlif_gfx950.so")
-EXT_LIB = os.path.join(PKG_DIR, "snnlib.so")
+LIB_DIR = os.path.join(PKG_DIR, "lib")
+KERNEL_LIB = os.path.join(LIB_DIR, "libsnnlif_gfx950.so")
+EXT_LIB = os.path.join(LIB_DIR, "snnlib.so")
 
 # -ffp-contract=off: products and sums stay separately rounded (bit parity with per-op fp32).
 # -packed-fp32-ops off: keep the compiler from forming packed fp32 VALU instructions.
@@ -64,6 +66,7 @@ def build_kernels(verbose=False, extra_flags=(), output=KERNEL_LIB):
     One object per translation unit (compiled in parallel), then one link step.
     """
     hipcc = hipcc_path()
+    os.makedirs(os.path.dirname(output), exist_ok=True)
     with tempfile.TemporaryDirectory(prefix="snnlif_build_") as tmp:
         def compile_one(src):
             obj = os.path.join(tmp, os.path.splitext(src)[0] + ".o")
@@ -95,7 +98,7 @@ def build_extension(verbose=False):
         f"-I{os.path.join(rocm, 'include')}", f"-I{sysconfig.get_paths()['include']}",
         os.path.join(CSRC, "snnlib_ext.cpp"), "-o", EXT_LIB,
         f"-L{tlib}", "-ltorch", "-ltorch_cpu", "-ltorch_hip", "-ltorch_python", "-lc10", "-lc10_hip",
-        f"-L{PKG_DIR}", "-l:libsnnlif_gfx950.so",
+        f"-L{LIB_DIR}", "-l:libsnnlif_gfx950.so",
         "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}",
     ]
     _run(cmd, verbose)

@@ -9,7 +9,7 @@ import ctypes
 import os
 
 PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG_DIR, "libsnnlif_gfx950.so")
+LIB_PATH = os.path.join(PKG_DIR, "lib", "libsnnlif_gfx950.so")
 
 DTYPE_F32, DTYPE_F64, DTYPE_BF16 = 0, 1, 2
 OK, ERR_ARG, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN = 0, -1, -2, -3, -4
