@@ -32,8 +32,11 @@
 //     which costs the compiler hundreds of VGPRs).
 //   * The op is element-wise and HBM-bound: no LDS, no cross-lane traffic, no MFMA.
 //   * Cache policy per stream: spikes and gradients are touched once and carry the non-temporal
-//     hint; the input current x is read by the forward and again by the backward, so when it fits
-//     the 256 MB memory-side cache it is loaded with the default policy and left there.
+//     hint; the input current x is read by the forward and again by the backward, so it alone is
+//     loaded with the default policy and may stay in the 256 MB memory-side cache.  The forward
+//     walks the neuron axis upwards and the backward downwards, so whatever part of x is still
+//     cached when the backward starts (all of it up to 256 MiB, the most recently read part
+//     otherwise) is the part the backward asks for first.
 //   * Built with -ffp-contract=off: each product and sum is rounded on its own, as PyTorch's
 //     element-wise CPU/GPU ops do, which makes spikes, potentials and gradients bit-identical to
 //     the per-op rounded reference arithmetic.
@@ -62,17 +65,14 @@
 #ifndef SNNLIF_BWD_BLOCK
 #define SNNLIF_BWD_BLOCK 256
 #endif
-// The input current x is the one tensor that is read twice (by the forward, then again by the
-// backward's recomputation).  When it is at most this many bytes it is loaded with the default
-// cache policy so that it may stay in the 256 MB memory-side cache between the two kernels; every
-// other stream (spikes, incoming and outgoing gradients, and x itself when it is larger) is
-// touched once and carries the non-temporal hint so that it does not displace x.
-#ifndef SNNLIF_KEEP_INPUT_BYTES
-#define SNNLIF_KEEP_INPUT_BYTES (int64_t(256) << 20)
-#endif
 // VGPR budget (in 32-bit words) the fused backward may spend on the recomputed membrane potential.
 #ifndef SNNLIF_FUSED_U_WORDS
 #define SNNLIF_FUSED_U_WORDS 128
+#endif
+// Column order of the fused backward: 1 = workgroups walk the neuron axis from its end, i.e.
+// opposite to the forward (the cached tail of x is consumed before it can be displaced).
+#ifndef SNNLIF_BWD_DESCENDING
+#define SNNLIF_BWD_DESCENDING 1
 #endif
 // Rows of x the forward requests before consuming the first (windows longer than this are
 // streamed with the next group of rows in flight).
@@ -204,9 +204,9 @@ __device__ __forceinline__ void lif_reverse_step(C& gu, C u, C g, C alpha, C thr
 // public op, the arithmetic type when it is the backward's workspace), V: neurons per lane,
 // TC: rows requested before the first is consumed.  MULTI = false: the whole window fits in TC
 // rows.  MULTI = true: the window is streamed TC rows at a time with the next TC rows already in
-// flight while the current ones are processed.  KEEPX: load x with the default cache policy.
+// flight while the current ones are processed.
 // ---------------------------------------------------------------------------------------------
-template <typename S, typename M, int V, int TC, bool MULTI, bool KEEPX, bool WRITE_U, bool WRITE_S>
+template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S>
 __global__ void __launch_bounds__(kFwdBlock)
 lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__ spike, int T,
                    int64_t N, int64_t nvec, typename Arith<S>::type alpha,
@@ -226,7 +226,7 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
         Pack<S, V> nxt[MULTI ? TC : 1];
 #pragma unroll
         for (int k = 0; k < TC; ++k) {
-            if (k < T) cur[k] = load_pack<S, V, !KEEPX>(x + static_cast<int64_t>(k) * N + col);
+            if (k < T) cur[k] = load_pack<S, V, false>(x + static_cast<int64_t>(k) * N + col);
         }
         for (int t0 = 0; t0 < T; t0 += TC) {
             if (MULTI && t0 + TC < T) {
@@ -235,7 +235,7 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
                     const int t = t0 + TC + k;
                     if (t < T)
                         nxt[MULTI ? k : 0] =
-                            load_pack<S, V, !KEEPX>(x + static_cast<int64_t>(t) * N + col);
+                            load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
                 }
             }
 #pragma unroll
@@ -272,7 +272,7 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 // Gradient rows are fetched in groups of at most GC, the newest time steps first; the fetch of the
 // next (earlier) group is issued before the current group is consumed.
 // ---------------------------------------------------------------------------------------------
-template <typename S, int V, int TW, bool EXACT, bool KEEPX>
+template <typename S, int V, int TW, bool EXACT>
 __global__ void __launch_bounds__(kBwdBlock)
 lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
                           int T, int64_t N, int64_t nvec, typename Arith<S>::type alpha,
@@ -286,16 +286,20 @@ lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* _
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
     for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < nvec;
          v += stride) {
+#if SNNLIF_BWD_DESCENDING
+        const int64_t col = (nvec - 1 - v) * V;
+#else
         const int64_t col = v * V;
+#endif
 
         Pack<S, V> xin[TW];
 #pragma unroll
         for (int t = 0; t < TW; ++t) {
             if (EXACT) {
-                xin[t] = load_pack<S, V, !KEEPX>(x + static_cast<int64_t>(t) * N + col);
+                xin[t] = load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
             } else {
                 xin[t] = zero_pack<S, V>();
-                if (t < T) xin[t] = load_pack<S, V, !KEEPX>(x + static_cast<int64_t>(t) * N + col);
+                if (t < T) xin[t] = load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
             }
         }
         Pack<S, V> gbuf[2][GC];
@@ -473,12 +477,6 @@ inline int launch_status() {
     return static_cast<int>(hipGetLastError());
 }
 
-// Whether x is small enough to be left in the memory-side cache for its second reader.
-template <typename S>
-inline bool keep_input(int64_t T, int64_t N) {
-    return T * N <= SNNLIF_KEEP_INPUT_BYTES / static_cast<int64_t>(sizeof(S));
-}
-
 // Calls f(std::integral_constant<int, v>) for the runtime vector width v in {MAXV, MAXV/2, .., 1}.
 template <int MAXV, typename F>
 inline int with_vec(int v, F&& f) {
@@ -494,8 +492,8 @@ inline int with_vec(int v, F&& f) {
     return f(std::integral_constant<int, 1>());
 }
 
-template <typename S, typename M, int V, bool KEEPX, bool WRITE_U, bool WRITE_S>
-int launch_forward_vk(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
+template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S>
+int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
                       hipStream_t stream) {
     using C = typename Arith<S>::type;
     const int64_t nvec = N / V;
@@ -503,13 +501,13 @@ int launch_forward_vk(const S* x, M* mem, S* spike, int64_t T, int64_t N, float 
     const int Ti = static_cast<int>(T);
     constexpr int TC = SNNLIF_FWD_ROWS;
     if (T <= 4 && TC > 4) {
-        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, 4, false, KEEPX, WRITE_U, WRITE_S>), grid,
+        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, 4, false, WRITE_U, WRITE_S>), grid,
                            block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
     } else if (T <= TC) {
-        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, TC, false, KEEPX, WRITE_U, WRITE_S>), grid,
+        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, TC, false, WRITE_U, WRITE_S>), grid,
                            block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
     } else {
-        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, TC, true, KEEPX, WRITE_U, WRITE_S>), grid,
+        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, TC, true, WRITE_U, WRITE_S>), grid,
                            block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
     }
     return launch_status();
@@ -530,17 +528,9 @@ int launch_forward(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alp
     for (int i = 0; i < 3; ++i)
         if (!aligned_to(ptrs[i], elem[i])) return SNNLIF_ERR_ALIGN;
     const int v = pick_vec(maxv, N, ptrs, elem, 3);
-    // Only full-width lanes get the cache-resident variant; narrow lanes are the odd-shape path.
-    const bool keep = (v == maxv) && keep_input<S>(T, N);
     return with_vec<maxv>(v, [&](auto vc) {
         constexpr int V = decltype(vc)::value;
-        if constexpr (V == maxv) {
-            if (keep)
-                return launch_forward_vk<S, M, V, true, WRITE_U, WRITE_S>(x, mem, spike, T, N, alpha,
-                                                                           thresh, stream);
-        }
-        return launch_forward_vk<S, M, V, false, WRITE_U, WRITE_S>(x, mem, spike, T, N, alpha,
-                                                                    thresh, stream);
+        return launch_forward_v<S, M, V, WRITE_U, WRITE_S>(x, mem, spike, T, N, alpha, thresh, stream);
     });
 }
 
@@ -576,7 +566,6 @@ int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, f
     const void* ptrs[3] = {x, g, gx};
     const size_t elem[3] = {sizeof(S), sizeof(S), sizeof(S)};
     const int v = pick_vec(maxv, N, ptrs, elem, 3);
-    const bool keep = (v == maxv) && keep_input<S>(T, N);
     // Every window of at most 8 rows has an instantiation of its own, so only the longer ones
     // are ever entered with T < TW.
     constexpr bool can_be_inexact = TW > 8;
@@ -586,25 +575,13 @@ int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, f
         const int64_t nvec = N / V;
         const dim3 grid(grid_for(nvec, kBwdBlock)), block(kBwdBlock);
         const int Ti = static_cast<int>(T);
-#define SNNLIF_LAUNCH_BWD(EXACT_, KEEP_)                                                         \
-    hipLaunchKernelGGL((lif_backward_fused_kernel<S, V, TW, EXACT_, KEEP_>), grid, block, 0,     \
-                       stream, x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval))
-        if constexpr (V == maxv) {
-            if (keep) {
-                if (exact) {
-                    SNNLIF_LAUNCH_BWD(true, true);
-                } else if constexpr (can_be_inexact) {
-                    SNNLIF_LAUNCH_BWD(false, true);
-                }
-                return launch_status();
-            }
-        }
         if (exact) {
-            SNNLIF_LAUNCH_BWD(true, false);
+            hipLaunchKernelGGL((lif_backward_fused_kernel<S, V, TW, true>), grid, block, 0, stream,
+                               x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval));
         } else if constexpr (can_be_inexact) {
-            SNNLIF_LAUNCH_BWD(false, false);
+            hipLaunchKernelGGL((lif_backward_fused_kernel<S, V, TW, false>), grid, block, 0, stream,
+                               x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval));
         }
-#undef SNNLIF_LAUNCH_BWD
         return launch_status();
     });
 }
