@@ -3,6 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg5_bf16|cfg1]
                     [--no-cpu-baseline]
+    python bench.py --workload train_step [--steps K] [--warmup W]     (context figure, see below)
 
 One "step" is one forward (spikes from the input current) plus one backward (input gradient from
 the saved input current and the spike gradient) over one synthetic batch that is already resident
@@ -21,6 +22,11 @@ pre-allocated outputs.  The default workload is the headline configuration
                  (``oracle/gold_fire.py``) on the host cores, forward + autograd backward on the same
                  inputs, best of 3 after a warm-up; its outputs also serve as the parity check of
                  this very run (``parity``).
+
+``--workload train_step`` is not the headline metric: it runs one SGD step of a small synthetic
+spiking CNN on CIFAR-shaped random data (conv / linear / pooling on PyTorch-ROCm, the four LIF layers
+through ``snnlib_op.Fire``) and reports the end-to-end step time and the share of it spent in the
+fire kernels, measured with events around the ``snnlib.fire_s_fp`` / ``snnlib.fire_bp`` calls.
 """
 import argparse
 import json
@@ -77,12 +83,129 @@ def cpu_baseline(torch, x, g, repeats=3):
     return best, threads, outs
 
 
+def build_synthetic_snn(torch, fire_factory, seed=0):
+    """conv3x3(3->128)-LIF-conv3x3(128->256)-LIF-avgpool2-conv3x3(256->256)-LIF-avgpool2-
+    linear(256*8*8->1024)-LIF-linear(1024->10) on [T, B, ...] tensors; output averaged over T.
+    Convolutions and linears see T folded into the batch.  Kaiming-normal weights, zero biases."""
+    nn = torch.nn
+
+    class TimeFolded(nn.Module):
+        def __init__(self, layer):
+            super().__init__()
+            self.layer = layer
+
+        def forward(self, x):
+            T, B = x.shape[0], x.shape[1]
+            y = self.layer(x.reshape(T * B, *x.shape[2:]))
+            return y.reshape(T, B, *y.shape[1:])
+
+    class Flatten(nn.Module):
+        def forward(self, x):
+            return x.reshape(x.shape[0], x.shape[1], -1)
+
+    torch.manual_seed(seed)
+    net = nn.Sequential(
+        TimeFolded(nn.Conv2d(3, 128, 3, padding=1)), fire_factory(),
+        TimeFolded(nn.Conv2d(128, 256, 3, padding=1)), fire_factory(),
+        TimeFolded(nn.AvgPool2d(2)),
+        TimeFolded(nn.Conv2d(256, 256, 3, padding=1)), fire_factory(),
+        TimeFolded(nn.AvgPool2d(2)),
+        Flatten(),
+        TimeFolded(nn.Linear(256 * 8 * 8, 1024)), fire_factory(),
+        TimeFolded(nn.Linear(1024, 10)),
+    )
+    for m in net.modules():
+        if isinstance(m, (nn.Conv2d, nn.Linear)):
+            nn.init.kaiming_normal_(m.weight)
+            nn.init.zeros_(m.bias)
+    return net
+
+
+def synthetic_batch(torch, T=8, B=64, seed=0):
+    gen = torch.Generator().manual_seed(seed)
+    images = torch.rand((B, 3, 32, 32), generator=gen)
+    labels = torch.randint(0, 10, (B,), generator=gen)
+    return images.unsqueeze(0).repeat(T, 1, 1, 1, 1), labels
+
+
+def run_train_step(args):
+    import torch
+    from snn_gpu_training_bptt_amd import snnlib_func as sf
+    from snn_gpu_training_bptt_amd import snnlib_op as sop
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no ROCm GPU visible")
+    dev = torch.device("cuda:0")
+    sf.alpha, sf.thresh, sf.beta, sf.interval = ALPHA, THRESH, BETA, INTERVAL
+    T, B = 8, 64
+    net = build_synthetic_snn(torch, sop.Fire).to(dev)
+    opt = torch.optim.SGD(net.parameters(), lr=0.1)
+    crit = torch.nn.CrossEntropyLoss()
+    x, labels = synthetic_batch(torch, T, B)
+    x, labels = x.to(dev), labels.to(dev)
+
+    # events around the native fire calls: a proxy in place of the module object snnlib_func uses
+    native = sf.snnlib
+    spans = []
+
+    class TimedOps:
+        def __getattr__(self, name):
+            fn = getattr(native, name)
+
+            def timed(*a):
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+                out = fn(*a)
+                e1.record()
+                spans.append((name, a[0].numel(), e0, e1))
+                return out
+            return timed
+
+    def one_step():
+        opt.zero_grad(set_to_none=True)
+        out = net(x).mean(dim=0)
+        loss = crit(out, labels)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(args.warmup):
+        one_step()
+    torch.cuda.synchronize()
+    sf.snnlib = TimedOps()
+    try:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = one_step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    finally:
+        sf.snnlib = native
+    step_ms = (t1 - t0) / args.steps * 1e3
+    lif_ms = sum(e0.elapsed_time(e1) for _, _, e0, e1 in spans) / args.steps
+    lif_ns = sum(n for _, n, _, _ in spans) // (2 * args.steps)   # each layer appears in fwd and bwd
+    print(json.dumps({
+        "metric": "synthetic SNN training step (context figure, not the headline metric)",
+        "value": step_ms, "unit": "ms/step", "higher_is_better": False, "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": step_ms, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "train_step: conv3x3(3-128)-LIF-conv3x3(128-256)-LIF-pool-conv3x3(256-256)-"
+                               "LIF-pool-fc(16384-1024)-LIF-fc(1024-10), T=8 B=64 CIFAR-shaped random data, "
+                               "SGD lr 0.1, CE on the time-averaged output"},
+        "lif_ms_per_step": lif_ms, "lif_share": lif_ms / step_ms,
+        "lif_neuron_steps_per_step": lif_ns,
+        "lif_algorithmic_GBps": 20 * lif_ns / (lif_ms * 1e-3) / 1e9,
+        "final_loss": float(loss.item()),
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain device copies of the input tensor (known size: one "
@@ -93,6 +216,13 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the fire op needs no communication; "
                  "neurons shard across GPUs with zero exchange). Run with --gpus 1.")
+
+    if args.workload == "train_step":
+        if args.steps == 200:
+            args.steps = 10
+        if args.warmup == 20:
+            args.warmup = 3
+        return run_train_step(args)
 
     import torch
     from snn_gpu_training_bptt_amd import lif_cabi

@@ -1,0 +1,49 @@
+"""One SGD step of the synthetic spiking CNN of the benchmark's ``train_step`` workload: the network
+built on ``snnlib_op.Fire`` must train exactly like the same network built on the pure-PyTorch gold
+fire (same convolution / linear kernels on both sides, so the only difference is the fire op)."""
+import pytest
+import torch
+
+from conftest import ALPHA, BETA, INTERVAL, THRESH
+
+pytestmark = pytest.mark.gpu
+
+
+def test_training_step_matches_gold_fire_network():
+    import bench
+    from oracle import gold_fire
+    from snn_gpu_training_bptt_amd import snnlib_func as sf
+    from snn_gpu_training_bptt_amd import snnlib_op as sop
+
+    saved = (sf.alpha, sf.thresh, sf.beta, sf.interval)
+    sf.alpha, sf.thresh, sf.beta, sf.interval = ALPHA, THRESH, BETA, INTERVAL
+
+    class GoldFire(torch.nn.Module):
+        def forward(self, x):
+            return gold_fire.gold_fire(x, ALPHA, THRESH, BETA, INTERVAL)[1]
+
+    try:
+        T, B = 4, 8          # same layers, smaller batch and window: the check is per-op exactness
+        x, labels = bench.synthetic_batch(torch, T, B, seed=1)
+        x, labels = x.cuda(), labels.cuda()
+        results = []
+        for factory in (sop.Fire, GoldFire):
+            torch.backends.cudnn.deterministic = True
+            net = bench.build_synthetic_snn(torch, factory, seed=5).cuda()
+            opt = torch.optim.SGD(net.parameters(), lr=0.1)
+            out = net(x).mean(dim=0)
+            loss = torch.nn.functional.cross_entropy(out, labels)
+            loss.backward()
+            grads = [p.grad.clone() for p in net.parameters()]
+            opt.step()
+            results.append((out.detach(), loss.detach(), grads, [p.detach().clone() for p in net.parameters()]))
+        (out_a, loss_a, grads_a, params_a), (out_b, loss_b, grads_b, params_b) = results
+        # spikes are bit-exact, so the forward is identical op for op
+        assert torch.equal(out_a, out_b)
+        assert torch.equal(loss_a, loss_b)
+        for ga, gb in zip(grads_a, grads_b):
+            torch.testing.assert_close(ga, gb, rtol=1e-4, atol=1e-6)
+        for pa, pb in zip(params_a, params_b):
+            torch.testing.assert_close(pa, pb, rtol=1e-4, atol=1e-6)
+    finally:
+        sf.alpha, sf.thresh, sf.beta, sf.interval = saved
