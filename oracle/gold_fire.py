@@ -46,3 +46,20 @@ def gold_fire_fwd_bwd(x, grad_spike, alpha, thresh, beta=1.0, interval=0.5):
     u, s = gold_fire(xr, alpha, thresh, beta, interval)
     s.backward(grad_spike)
     return u.detach(), s.detach(), xr.grad.detach()
+
+
+def gold_fire_fc(x, weight, bias, alpha, thresh, beta=1.0, interval=0.5):
+    """Fire, then one ``linear`` per time step on the flattened spikes
+    (snnlib/example/gold_op.py:113-145 with ``fire=True``).  Returns ``[T, B, cout]``."""
+    _, s = gold_fire(x, alpha, thresh, beta, interval)
+    if s.dim() == 5:
+        s = s.view(s.shape[0], s.shape[1], -1)
+    return torch.stack([torch.nn.functional.linear(s[t], weight, bias) for t in range(s.shape[0])], dim=0)
+
+
+def gold_fire_conv(x, weight, bias, stride, padding, alpha, thresh, beta=1.0, interval=0.5):
+    """Fire, then one ``conv2d`` per time step (snnlib/example/gold_op.py:148-179 with
+    ``fire=True``).  Returns ``[T, B, cout, Hout, Wout]``."""
+    _, s = gold_fire(x, alpha, thresh, beta, interval)
+    return torch.stack([torch.nn.functional.conv2d(s[t], weight, bias, stride, padding)
+                        for t in range(s.shape[0])], dim=0)

@@ -6,7 +6,21 @@
 //     fire_s_fp(spatial, alpha, thresh)                               -> spike
 //     fire_bp(spatial, grad_spike, alpha, thresh, beta, interval)     -> grad_spatial
 // plus fire_us_fp(spatial, alpha, thresh) -> (mem, spike), the public face of the reference's
-// internal fire_us_fp_kernel (snnlib/cuda/snn_kernel_bp.cu:54-93).
+// internal fire_us_fp_kernel (snnlib/cuda/snn_kernel_bp.cu:54-93), and the fire-then-linear /
+// fire-then-convolution layer ops with the reference's signatures
+// (snnlib/cuda/snn.cpp:112-120, 206-223, 569-582, 740-761; bound at :806, :810, :817, :821)
+//     fire_fc_fp(spatial, weight_fc, bias_fc, alpha, thresh)                              -> fc
+//     fire_fc_bp(spatial, grad_fc, weight_fc, bias_fc, dim_fc, alpha, thresh, beta, interval)
+//                                                     -> [grad_spatial, grad_weight_fc, grad_bias_fc]
+//     fire_conv_fp(spatial, weight_conv, bias_conv, stride, padding, dilation, groups, benchmark,
+//                  deterministic, alpha, thresh)                                           -> conv
+//     fire_conv_bp(spatial, grad_conv, weight_conv, stride, padding, dilation, groups, benchmark,
+//                  deterministic, allow_tf32, dim_conv, alpha, thresh, beta, interval)
+//                                                 -> [grad_spatial, grad_weight_conv, grad_bias_conv]
+// in which the fire part runs on this library's kernels and the linear / convolution part stays on
+// PyTorch-ROCm (rocBLAS / MIOpen through ATen), issued once with the time axis folded into the
+// batch instead of once per time step as the reference's host loops do
+// (snnlib/cuda/snn_kernel_fp.cu:314-326, 444-447; snnlib/cuda/snn_kernel_bp.cu:1099-1117, 1382-1390).
 //
 // This file only validates tensors, allocates outputs and forwards raw device pointers to the C ABI
 // of libsnnlif_gfx950.so (include/snnlib_lif.h); all device code lives there.  Unlike the reference
@@ -20,6 +34,7 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <tuple>
+#include <vector>
 
 #include "snnlib_lif.h"
 
@@ -127,6 +142,121 @@ torch::Tensor fire_bp(torch::Tensor spatial, torch::Tensor grad_spike, float alp
     return grad_spatial;
 }
 
+// ---- fire followed by a fully connected layer ---------------------------------------------------
+
+// [T, B, ...] -> [T*B, prod(...)]
+torch::Tensor fold_time_flat(const torch::Tensor& t) {
+    return t.reshape({t.size(0) * t.size(1), -1});
+}
+
+void check_param(const torch::Tensor& p, const torch::Tensor& like, const char* op, const char* name) {
+    TORCH_CHECK(p.defined(), "snnlib.", op, ": ", name, " is undefined");
+    TORCH_CHECK(p.device() == like.device(), "snnlib.", op, ": ", name, " (", p.device(),
+                ") must be on the device of spatial (", like.device(), ")");
+    TORCH_CHECK(p.scalar_type() == like.scalar_type(), "snnlib.", op, ": ", name, " (",
+                p.scalar_type(), ") must have the dtype of spatial (", like.scalar_type(), ")");
+}
+
+torch::Tensor fire_fc_fp(torch::Tensor spatial, torch::Tensor weight_fc, torch::Tensor bias_fc,
+                         float alpha, float thresh) {
+    check_input(spatial, "fire_fc_fp", "spatial");
+    check_param(weight_fc, spatial, "fire_fc_fp", "weight_fc");
+    check_param(bias_fc, spatial, "fire_fc_fp", "bias_fc");
+    TORCH_CHECK(weight_fc.dim() == 2, "snnlib.fire_fc_fp: weight_fc must be [cout, cin]");
+    const int64_t T = spatial.size(0), B = spatial.size(1);
+    const int64_t cin = (T * B) ? spatial.numel() / (T * B) : weight_fc.size(1);
+    TORCH_CHECK(weight_fc.size(1) == cin, "snnlib.fire_fc_fp: weight_fc expects ", weight_fc.size(1),
+                " inputs per sample, spatial has ", cin);
+    torch::Tensor spike = fire_s_fp(spatial, alpha, thresh);
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(spatial.device());
+    torch::Tensor fc = at::linear(fold_time_flat(spike), weight_fc, bias_fc);
+    return fc.view({T, B, weight_fc.size(0)});
+}
+
+std::vector<torch::Tensor> fire_fc_bp(torch::Tensor spatial, torch::Tensor grad_fc,
+                                      torch::Tensor weight_fc, torch::Tensor bias_fc,
+                                      std::vector<int64_t> dim_fc, float alpha, float thresh,
+                                      float beta, float interval) {
+    check_input(spatial, "fire_fc_bp", "spatial");
+    check_param(weight_fc, spatial, "fire_fc_bp", "weight_fc");
+    check_param(grad_fc, spatial, "fire_fc_bp", "grad_fc");
+    const int64_t T = spatial.size(0), B = spatial.size(1);
+    TORCH_CHECK(grad_fc.dim() == 3 && grad_fc.size(0) == T && grad_fc.size(1) == B &&
+                    grad_fc.size(2) == weight_fc.size(0),
+                "snnlib.fire_fc_bp: grad_fc must be [T, B, cout] = [", T, ", ", B, ", ",
+                weight_fc.size(0), "], got ", grad_fc.sizes());
+    (void)bias_fc;  // kept for signature parity; the bias gradient needs only grad_fc
+    // recompute the spikes (only the input current is saved between forward and backward)
+    torch::Tensor spike = fire_s_fp(spatial, alpha, thresh);
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(spatial.device());
+    torch::Tensor g2 = fold_time_flat(grad_fc.contiguous());           // [T*B, cout]
+    torch::Tensor grad_spike = at::mm(g2, weight_fc).view(spatial.sizes());
+    torch::Tensor grad_weight = at::mm(g2.t(), fold_time_flat(spike));  // [cout, cin]
+    torch::Tensor grad_bias = at::sum(grad_fc, dim_fc);
+    torch::Tensor grad_spatial = fire_bp(spatial, grad_spike, alpha, thresh, beta, interval);
+    return {grad_spatial, grad_weight, grad_bias};
+}
+
+// ---- fire followed by a 2-d convolution ---------------------------------------------------------
+
+// [T, B, C, H, W] -> [T*B, C, H, W]
+torch::Tensor fold_time_image(const torch::Tensor& t) {
+    return t.reshape({t.size(0) * t.size(1), t.size(2), t.size(3), t.size(4)});
+}
+
+torch::Tensor fire_conv_fp(torch::Tensor spatial, torch::Tensor weight_conv,
+                           torch::Tensor bias_conv, std::vector<int64_t> stride,
+                           std::vector<int64_t> padding, std::vector<int64_t> dilation,
+                           int64_t groups, bool benchmark, bool deterministic, float alpha,
+                           float thresh) {
+    // `benchmark` / `deterministic` select cuDNN behaviour in the reference; on ROCm the
+    // convolution algorithm is MIOpen's choice under torch.backends.cudnn.{benchmark,deterministic}.
+    (void)benchmark;
+    (void)deterministic;
+    check_input(spatial, "fire_conv_fp", "spatial");
+    TORCH_CHECK(spatial.dim() == 5, "snnlib.fire_conv_fp: spatial must be [T, B, C, H, W]");
+    check_param(weight_conv, spatial, "fire_conv_fp", "weight_conv");
+    check_param(bias_conv, spatial, "fire_conv_fp", "bias_conv");
+    const int64_t T = spatial.size(0), B = spatial.size(1);
+    torch::Tensor spike = fire_s_fp(spatial, alpha, thresh);
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(spatial.device());
+    torch::Tensor conv = at::convolution(fold_time_image(spike), weight_conv, bias_conv, stride,
+                                         padding, dilation, /*transposed=*/false,
+                                         /*output_padding=*/{0, 0}, groups);
+    return conv.view({T, B, conv.size(1), conv.size(2), conv.size(3)});
+}
+
+std::vector<torch::Tensor> fire_conv_bp(torch::Tensor spatial, torch::Tensor grad_conv,
+                                        torch::Tensor weight_conv, std::vector<int64_t> stride,
+                                        std::vector<int64_t> padding,
+                                        std::vector<int64_t> dilation, int64_t groups,
+                                        bool benchmark, bool deterministic, bool allow_tf32,
+                                        std::vector<int64_t> dim_conv, float alpha, float thresh,
+                                        float beta, float interval) {
+    (void)benchmark;
+    (void)deterministic;
+    (void)allow_tf32;
+    check_input(spatial, "fire_conv_bp", "spatial");
+    TORCH_CHECK(spatial.dim() == 5, "snnlib.fire_conv_bp: spatial must be [T, B, C, H, W]");
+    check_param(weight_conv, spatial, "fire_conv_bp", "weight_conv");
+    check_param(grad_conv, spatial, "fire_conv_bp", "grad_conv");
+    TORCH_CHECK(grad_conv.dim() == 5 && grad_conv.size(0) == spatial.size(0) &&
+                    grad_conv.size(1) == spatial.size(1) && grad_conv.size(2) == weight_conv.size(0),
+                "snnlib.fire_conv_bp: grad_conv must be [T, B, cout, Hout, Wout], got ",
+                grad_conv.sizes());
+    torch::Tensor spike = fire_s_fp(spatial, alpha, thresh);
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(spatial.device());
+    auto grads = at::convolution_backward(
+        fold_time_image(grad_conv.contiguous()), fold_time_image(spike), weight_conv,
+        /*bias_sizes=*/c10::nullopt, stride, padding, dilation, /*transposed=*/false,
+        /*output_padding=*/{0, 0}, groups, /*output_mask=*/{true, true, false});
+    torch::Tensor grad_spike = std::get<0>(grads).view(spatial.sizes());
+    torch::Tensor grad_weight = std::get<1>(grads);
+    torch::Tensor grad_bias = at::sum(grad_conv, dim_conv);
+    torch::Tensor grad_spatial = fire_bp(spatial, grad_spike, alpha, thresh, beta, interval);
+    return {grad_spatial, grad_weight, grad_bias};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -136,4 +266,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("fire_s_fp", &fire_s_fp, "fire (spike) forward");
     m.def("fire_us_fp", &fire_us_fp, "fire (membrane potential, spike) forward");
     m.def("fire_bp", &fire_bp, "fire backward");
+    m.def("fire_fc_fp", &fire_fc_fp, "fire fc forward");
+    m.def("fire_fc_bp", &fire_fc_bp, "fire fc backward");
+    m.def("fire_conv_fp", &fire_conv_fp, "fire conv forward");
+    m.def("fire_conv_bp", &fire_conv_bp, "fire conv backward");
 }
