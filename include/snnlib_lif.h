@@ -46,6 +46,7 @@ extern "C" {
 #define SNNLIF_ERR_DTYPE      -2 /* dtype is not one of SNNLIF_DTYPE_* */
 #define SNNLIF_ERR_WORKSPACE  -3 /* workspace missing or smaller than snnlif_fire_bp_workspace_bytes() */
 #define SNNLIF_ERR_ALIGN      -4 /* a pointer is not aligned to its element size */
+#define SNNLIF_ERR_UNSUPPORTED -5 /* valid arguments this entry point does not implement (see its comment) */
 
 /* Largest T for which the backward keeps the recomputed membrane potential in registers and
  * therefore needs no workspace. */
@@ -104,6 +105,40 @@ size_t snnlif_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t N);
 int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spatial, int dtype,
                    int64_t T, int64_t N, float alpha, float thresh, float beta, float interval,
                    void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Batch-norm + fire forward (fp32 only: dtype must be SNNLIF_DTYPE_F32, else SNNLIF_ERR_UNSUPPORTED).
+ * Tensors are [T, B, C, HW] (HW = 1 for [T, B, C]); weight, bias, var, mean, ivar are [C].
+ *   scale[c] = weight[c] / sqrt(var[c] + eps);   ivar[c] = scale[c] / weight[c]
+ *   u[t] = (alpha*u[t-1])*(1-s[t-1]) + (x[t] - mean[c])*scale[c] + bias[c];   s[t] = u[t] > thresh
+ * Replaces bn_fire_s_fp_cuda + bn_fire_s_fp_kernel (snnlib/cuda/snn_kernel_fp.cu:157-240), bound as
+ * snnlib.bn_fire_s_fp (snnlib/cuda/snn.cpp:800).
+ */
+int snnlif_bn_fire_s_fp(const void* spatial, const void* weight, const void* bias, const void* var,
+                        const void* mean, void* ivar, void* spike, int dtype, int64_t T, int64_t B,
+                        int64_t C, int64_t HW, float eps, float alpha, float thresh, void* stream);
+
+/* Bytes of device workspace snnlif_bn_fire_bp needs (two floats per neuron plus per-channel
+ * staging).  0 for invalid arguments. */
+size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);
+
+/*
+ * Batch-norm + fire backward (fp32 only; T <= SNNLIF_BP_FUSED_MAX_T, else SNNLIF_ERR_UNSUPPORTED).
+ * With u recomputed from scale[c] = weight[c]*ivar[c], gy the fire reverse chain (see
+ * snnlif_fire_bp), xhat = (x - mean[c])*ivar[c] and M = T*B*HW:
+ *   grad_bias[c] = sum gy;   grad_weight[c] = sum gy*xhat
+ *   grad_spatial = (gy*weight[c])*ivar[c]
+ *                  - ivar[c]*((xhat*(weight[c]*grad_weight[c]/M)) + weight[c]*grad_bias[c]/M)
+ * Replaces bn_fire_bp_cuda and its three kernels (snnlib/cuda/snn_kernel_bp.cu:432-479, 533-750),
+ * bound as snnlib.bn_fire_bp (snnlib/cuda/snn.cpp:814).  `workspace` must hold
+ * snnlif_bn_fire_bp_workspace_bytes() bytes, 16-byte aligned, private to the call until the
+ * stream has run it.  Per-channel sums are formed in a fixed order: results are reproducible.
+ */
+int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias, const void* ivar,
+                      const void* mean, const void* grad_spike, void* grad_spatial,
+                      void* grad_weight, void* grad_bias, int dtype, int64_t T, int64_t B, int64_t C,
+                      int64_t HW, float alpha, float thresh, float beta, float interval,
+                      void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,111 @@
+// Launchers of the batch-norm + fire kernels (fp32); see lif_bn_kernels.h.
+#include "lif_bn_kernels.h"
+
+namespace snnlif {
+
+int bn_forward_f32(const float* x, const float* weight, const float* bias, const float* var,
+                   const float* mean, float* ivar, float* spike, int64_t T, int64_t B, int64_t C,
+                   int64_t HW, float eps, float alpha, float thresh, hipStream_t stream) {
+    const int64_t N = B * C * HW;
+    const dim3 grid(grid_for(N, kFwdBlock)), block(kFwdBlock);
+    const int Ti = static_cast<int>(T);
+    constexpr int TC = SNNLIF_FWD_ROWS;
+    if (T <= 4 && TC > 4) {
+        hipLaunchKernelGGL((lif_bn_forward_kernel<4, false>), grid, block, 0, stream, x, weight, bias,
+                           var, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
+    } else if (T <= TC) {
+        hipLaunchKernelGGL((lif_bn_forward_kernel<TC, false>), grid, block, 0, stream, x, weight,
+                           bias, var, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
+    } else {
+        hipLaunchKernelGGL((lif_bn_forward_kernel<TC, true>), grid, block, 0, stream, x, weight,
+                           bias, var, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
+    }
+    return launch_status();
+}
+
+namespace {
+
+template <int TW>
+int bn_backward_window(const float* x, const float* weight, const float* bias, const float* ivar,
+                       const float* mean, const float* g, float* gx, float* grad_weight,
+                       float* grad_bias, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
+                       float thresh, float beta, float interval, float* workspace,
+                       hipStream_t stream) {
+    const int64_t N = B * C * HW;
+    const int S = bn_reduce_splits(B, C);
+    float* part_gy = workspace;
+    float* part_gyx = part_gy + N;
+    float* split = part_gyx + N;
+    float* coef = split + static_cast<int64_t>(2) * S * C;
+    const dim3 grid(grid_for(N, kBwdBlock)), block(kBwdBlock);
+    const int Ti = static_cast<int>(T);
+    constexpr bool can_be_inexact = TW > 8;
+    const bool exact = !can_be_inexact || (T == TW);
+
+    if (exact) {
+        hipLaunchKernelGGL((lif_bn_backward_partial_kernel<TW, true>), grid, block, 0, stream, x, g,
+                           weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha, thresh,
+                           beta, interval);
+    } else if constexpr (can_be_inexact) {
+        hipLaunchKernelGGL((lif_bn_backward_partial_kernel<TW, false>), grid, block, 0, stream, x, g,
+                           weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha, thresh,
+                           beta, interval);
+    }
+    int rc = launch_status();
+    if (rc != SNNLIF_OK) return rc;
+
+    const int64_t bs = (B + S - 1) / S;
+    hipLaunchKernelGGL(bn_channel_reduce_kernel, dim3(static_cast<unsigned>(C), S),
+                       dim3(kReduceBlock), 0, stream, part_gy, part_gyx, split, B, C, HW, bs, S);
+    rc = launch_status();
+    if (rc != SNNLIF_OK) return rc;
+    hipLaunchKernelGGL(bn_channel_finalize_kernel,
+                       dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
+                       dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias, coef, C,
+                       S, static_cast<float>(T * B * HW));
+    rc = launch_status();
+    if (rc != SNNLIF_OK) return rc;
+
+    if (exact) {
+        hipLaunchKernelGGL((lif_bn_backward_input_kernel<TW, true>), grid, block, 0, stream, x, g,
+                           weight, bias, ivar, mean, coef, gx, Ti, N, C, HW, alpha, thresh, beta,
+                           interval);
+    } else if constexpr (can_be_inexact) {
+        hipLaunchKernelGGL((lif_bn_backward_input_kernel<TW, false>), grid, block, 0, stream, x, g,
+                           weight, bias, ivar, mean, coef, gx, Ti, N, C, HW, alpha, thresh, beta,
+                           interval);
+    }
+    return launch_status();
+}
+
+}  // namespace
+
+int bn_backward_f32(const float* x, const float* weight, const float* bias, const float* ivar,
+                    const float* mean, const float* g, float* gx, float* grad_weight,
+                    float* grad_bias, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
+                    float thresh, float beta, float interval, float* workspace,
+                    hipStream_t stream) {
+#define SNNLIF_BN_WINDOW(TW)                                                                      \
+    if (T <= TW)                                                                                  \
+        return bn_backward_window<TW>(x, weight, bias, ivar, mean, g, gx, grad_weight, grad_bias, \
+                                      T, B, C, HW, alpha, thresh, beta, interval, workspace, stream);
+    SNNLIF_BN_WINDOW(1)
+    SNNLIF_BN_WINDOW(2)
+    SNNLIF_BN_WINDOW(3)
+    SNNLIF_BN_WINDOW(4)
+    SNNLIF_BN_WINDOW(5)
+    SNNLIF_BN_WINDOW(6)
+    SNNLIF_BN_WINDOW(7)
+    SNNLIF_BN_WINDOW(8)
+    SNNLIF_BN_WINDOW(10)
+    SNNLIF_BN_WINDOW(12)
+    SNNLIF_BN_WINDOW(16)
+    SNNLIF_BN_WINDOW(20)
+    SNNLIF_BN_WINDOW(24)
+    SNNLIF_BN_WINDOW(28)
+    SNNLIF_BN_WINDOW(32)
+#undef SNNLIF_BN_WINDOW
+    return SNNLIF_ERR_UNSUPPORTED;
+}
+
+}  // namespace snnlif

@@ -1,0 +1,287 @@
+// Batch-norm + LIF fire kernels (fp32) for MI355X: the per-channel affine of a batch norm is
+// applied to the input current inside the fire recurrence, forward and backward.
+//
+// Reference: snnlib/cuda/snn_kernel_fp.cu:157-240 (bn_fire_s_fp_kernel + launcher) and
+// snnlib/cuda/snn_kernel_bp.cu:432-479 (bn_fire_u_fp_kernel), :533-610 (bn_fire_bp_wb_kernel),
+// :613-677 (bn_fire_bp_x_kernel), :680-750 (bn_fire_bp_cuda).
+//
+//   forward   y = (x - mean[c]) * (weight[c] / sqrt(var[c] + eps)) + bias[c]   folded as
+//             u = (alpha*u)*(1-s) + (x - mean[c]) * scale[c] + bias[c];  s = u > thresh
+//             ivar[c] = scale[c] / weight[c]
+//   backward  gy[t] = the fire reverse chain on u recomputed with scale[c] = weight[c] * ivar[c]
+//             xhat  = (x - mean[c]) * ivar[c]
+//             grad_bias[c]   = sum gy            grad_weight[c] = sum gy * xhat      (over T,B,H,W)
+//             gxhat[c]  = weight[c] * grad_bias[c]   / M      gxhatx[c] = weight[c] * grad_weight[c] / M
+//             gx = (gy * weight[c]) * ivar[c] - ivar[c] * ((xhat * gxhatx[c]) + gxhat[c]),  M = T*B*H*W
+//
+// Mapping.  Same lanes as the plain fire kernels (one neuron per lane, time in registers).  The
+// backward needs per-channel sums over everything before any input gradient can be formed, so it
+// is two sweeps over (x, g) with a reduction between them:
+//   1. lif_bn_backward_partial_kernel: reverse chain per neuron, sums over its T steps -> two
+//      floats per neuron (1/T of a tensor, not a tensor);
+//   2. bn_channel_reduce_kernel / bn_channel_finalize_kernel: per-channel sums of those partials
+//      (wavefront shuffles, then LDS across the waves of a workgroup; the only place in this library
+//      where lanes cooperate), in a fixed order -> bit-reproducible results;
+//   3. lif_bn_backward_input_kernel: the chain again (x and g re-read: 8 B per neuron-step, the
+//      same as storing and re-loading gy would cost) and the input gradient.
+// HBM traffic: forward 8 B, backward 20 B (+ 16/T B) per neuron-step; the reference moves 8 and 36.
+#ifndef SNNLIF_LIF_BN_KERNELS_H
+#define SNNLIF_LIF_BN_KERNELS_H
+
+#include "lif_bn.h"
+#include "lif_kernels.h"
+
+namespace snnlif {
+
+constexpr int kReduceBlock = 256;
+
+// Channel of a neuron column in a [B, C, HW] neuron axis.
+__device__ __forceinline__ int channel_of(int64_t col, int64_t C, int64_t HW, bool small) {
+    if (small) {  // everything fits 32 bits: cheap unsigned division
+        const uint32_t q = static_cast<uint32_t>(col) / static_cast<uint32_t>(HW);
+        return static_cast<int>(q % static_cast<uint32_t>(C));
+    }
+    return static_cast<int>((col / HW) % C);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Forward: spikes (and the inverse standard deviation per channel).
+// ---------------------------------------------------------------------------------------------
+template <int TC, bool MULTI>
+__global__ void __launch_bounds__(kFwdBlock)
+lif_bn_forward_kernel(const float* __restrict__ x, const float* __restrict__ weight,
+                      const float* __restrict__ bias, const float* __restrict__ var,
+                      const float* __restrict__ mean, float* __restrict__ ivar,
+                      float* __restrict__ spike, int T, int64_t N, int64_t C, int64_t HW, float eps,
+                      float alpha, float thresh) {
+    const bool small = N <= 0xffffffffll;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kFwdBlock;
+    for (int64_t col = static_cast<int64_t>(blockIdx.x) * kFwdBlock + threadIdx.x; col < N;
+         col += stride) {
+        const int c = channel_of(col, C, HW, small);
+        const float m = mean[c];
+        const float wgt = weight[c];
+        const float scale = wgt / sqrtf(var[c] + eps);
+        const float b = bias[c];
+        // first neuron of the channel in batch entry 0 publishes the channel's ivar
+        if (col == static_cast<int64_t>(c) * HW) ivar[c] = scale / wgt;
+
+        float u = 0.f, s = 0.f;
+        Pack<float, 1> cur[TC];
+        Pack<float, 1> nxt[MULTI ? TC : 1];
+#pragma unroll
+        for (int k = 0; k < TC; ++k) {
+            if (k < T) cur[k] = load_pack<float, 1, false>(x + static_cast<int64_t>(k) * N + col);
+        }
+        for (int t0 = 0; t0 < T; t0 += TC) {
+            if (MULTI && t0 + TC < T) {
+#pragma unroll
+                for (int k = 0; k < TC; ++k) {
+                    const int t = t0 + TC + k;
+                    if (t < T)
+                        nxt[MULTI ? k : 0] =
+                            load_pack<float, 1, false>(x + static_cast<int64_t>(t) * N + col);
+                }
+            }
+#pragma unroll
+            for (int k = 0; k < TC; ++k) {
+                const int t = t0 + k;
+                if (t < T) {
+                    u = (alpha * u) * (1.f - s) + (cur[k].e[0] - m) * scale + b;
+                    s = (u > thresh) ? 1.f : 0.f;
+                    Pack<float, 1> so;
+                    so.e[0] = s;
+                    store_pack<float, 1>(spike + static_cast<int64_t>(t) * N + col, so);
+                }
+            }
+            if (!MULTI) break;
+            if (t0 + TC < T) {
+#pragma unroll
+                for (int k = 0; k < TC; ++k) cur[k] = nxt[MULTI ? k : 0];
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Shared front half of both backward sweeps: load the window, recompute u, run the reverse chain.
+// Calls emit(t, gy, x_t) for t = T-1 .. 0.
+// ---------------------------------------------------------------------------------------------
+template <int TW, bool EXACT, typename Emit>
+__device__ __forceinline__ void bn_reverse_chain(const float* __restrict__ x,
+                                                 const float* __restrict__ g, int T, int64_t N,
+                                                 int64_t col, float m, float scale, float b,
+                                                 float alpha, float thresh, float beta,
+                                                 float interval, Emit&& emit) {
+    float xin[TW], gin[TW], u[TW];
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+        xin[t] = 0.f;
+        if (EXACT || t < T)
+            xin[t] = load_pack<float, 1, false>(x + static_cast<int64_t>(t) * N + col).e[0];
+    }
+#pragma unroll
+    for (int t = TW - 1; t >= 0; --t) {
+        gin[t] = 0.f;
+        if (EXACT || t < T)
+            gin[t] = load_pack<float, 1, true>(g + static_cast<int64_t>(t) * N + col).e[0];
+    }
+    {
+        float uc = 0.f, sc = 0.f;
+#pragma unroll
+        for (int t = 0; t < TW; ++t) {
+            uc = (alpha * uc) * (1.f - sc) + (xin[t] - m) * scale + b;
+            sc = (uc > thresh) ? 1.f : 0.f;
+            u[t] = uc;
+        }
+    }
+    float gu = 0.f;
+#pragma unroll
+    for (int t = TW - 1; t >= 0; --t) {
+        if (EXACT || t < T) {
+            lif_reverse_step<float>(gu, u[t], gin[t], alpha, thresh, beta, interval);
+            emit(t, gu, xin[t]);
+        }
+    }
+}
+
+// Sweep 1: per-neuron sums over time of gy and gy * xhat.
+template <int TW, bool EXACT>
+__global__ void __launch_bounds__(kBwdBlock)
+lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restrict__ g,
+                               const float* __restrict__ weight, const float* __restrict__ bias,
+                               const float* __restrict__ ivar, const float* __restrict__ mean,
+                               float* __restrict__ part_gy, float* __restrict__ part_gyx, int T,
+                               int64_t N, int64_t C, int64_t HW, float alpha, float thresh,
+                               float beta, float interval) {
+    const bool small = N <= 0xffffffffll;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
+    for (int64_t col = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; col < N;
+         col += stride) {
+        const int c = channel_of(col, C, HW, small);
+        const float m = mean[c], iv = ivar[c];
+        const float scale = weight[c] * iv;
+        const float b = bias[c];
+        float acc_gy = 0.f, acc_gyx = 0.f;
+        bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval,
+                                    [&](int, float gy, float xt) {
+                                        const float xhat = (xt - m) * iv;
+                                        acc_gy += gy;
+                                        acc_gyx += gy * xhat;
+                                    });
+        part_gy[col] = acc_gy;
+        part_gyx[col] = acc_gyx;
+    }
+}
+
+// Sweep 2: input gradient.  coef = {gxhat[C], gxhatx[C]}.
+template <int TW, bool EXACT>
+__global__ void __launch_bounds__(kBwdBlock)
+lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restrict__ g,
+                             const float* __restrict__ weight, const float* __restrict__ bias,
+                             const float* __restrict__ ivar, const float* __restrict__ mean,
+                             const float* __restrict__ coef, float* __restrict__ gx, int T,
+                             int64_t N, int64_t C, int64_t HW, float alpha, float thresh, float beta,
+                             float interval) {
+    const bool small = N <= 0xffffffffll;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < N;
+         v += stride) {
+        const int64_t col = N - 1 - v;  // opposite direction to sweep 1: its tail is still cached
+        const int c = channel_of(col, C, HW, small);
+        const float m = mean[c], iv = ivar[c], wgt = weight[c];
+        const float scale = wgt * iv;
+        const float b = bias[c];
+        const float gxhat = coef[c], gxhatx = coef[C + c];
+        bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval,
+                                    [&](int t, float gy, float xt) {
+                                        Pack<float, 1> out;
+                                        out.e[0] = gy * wgt * iv - iv * ((xt - m) * iv * gxhatx + gxhat);
+                                        store_pack<float, 1>(gx + static_cast<int64_t>(t) * N + col, out);
+                                    });
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Per-channel reduction of the per-neuron partials.  Block (c, s) sums the batch entries
+// [s*bs, min(B, (s+1)*bs)) of channel c; lanes stride over the HW positions of one batch entry
+// (consecutive addresses), so the sum order is fixed by the geometry alone.
+// split = {gy[S][C], gyx[S][C]}.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    return v;
+}
+
+__global__ void __launch_bounds__(kReduceBlock)
+bn_channel_reduce_kernel(const float* __restrict__ part_gy, const float* __restrict__ part_gyx,
+                         float* __restrict__ split, int64_t B, int64_t C, int64_t HW, int64_t bs,
+                         int S) {
+    const int c = blockIdx.x;
+    const int s = blockIdx.y;
+    const int64_t b0 = static_cast<int64_t>(s) * bs;
+    const int64_t b1 = (b0 + bs < B) ? (b0 + bs) : B;
+    const int64_t CHW = C * HW;
+    float a = 0.f, ax = 0.f;
+    if (HW >= kReduceBlock / 4) {
+        for (int64_t b = b0; b < b1; ++b) {
+            const int64_t base = b * CHW + static_cast<int64_t>(c) * HW;
+            for (int64_t i = threadIdx.x; i < HW; i += kReduceBlock) {
+                a += part_gy[base + i];
+                ax += part_gyx[base + i];
+            }
+        }
+    } else {  // few positions per channel (fully connected shapes): lanes stride over (b, hw) pairs
+        const int64_t n = (b1 - b0) * HW;
+        for (int64_t e = threadIdx.x; e < n; e += kReduceBlock) {
+            const int64_t b = b0 + e / HW, i = e % HW;
+            const int64_t at = b * CHW + static_cast<int64_t>(c) * HW + i;
+            a += part_gy[at];
+            ax += part_gyx[at];
+        }
+    }
+    __shared__ float lds[2][kReduceBlock / 64];
+    a = wave_sum(a);
+    ax = wave_sum(ax);
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    if (lane == 0) {
+        lds[0][wave] = a;
+        lds[1][wave] = ax;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float ta = 0.f, tax = 0.f;
+#pragma unroll
+        for (int w = 0; w < kReduceBlock / 64; ++w) {
+            ta += lds[0][w];
+            tax += lds[1][w];
+        }
+        split[static_cast<int64_t>(s) * C + c] = ta;
+        split[static_cast<int64_t>(S) * C + static_cast<int64_t>(s) * C + c] = tax;
+    }
+}
+
+// One lane per channel: fold the S splits in order, emit the parameter gradients and the two
+// coefficients the input-gradient sweep needs.
+__global__ void __launch_bounds__(kReduceBlock)
+bn_channel_finalize_kernel(const float* __restrict__ split, const float* __restrict__ weight,
+                           float* __restrict__ grad_weight, float* __restrict__ grad_bias,
+                           float* __restrict__ coef, int64_t C, int S, float count) {
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * kReduceBlock + threadIdx.x;
+    if (c >= C) return;
+    float a = 0.f, ax = 0.f;
+    for (int s = 0; s < S; ++s) {
+        a += split[static_cast<int64_t>(s) * C + c];
+        ax += split[static_cast<int64_t>(S) * C + static_cast<int64_t>(s) * C + c];
+    }
+    grad_bias[c] = a;
+    grad_weight[c] = ax;
+    const float wgt = weight[c];
+    coef[c] = (a * wgt) / count;
+    coef[C + c] = (ax * wgt) / count;
+}
+
+}  // namespace snnlif
+
+#endif  // SNNLIF_LIF_BN_KERNELS_H

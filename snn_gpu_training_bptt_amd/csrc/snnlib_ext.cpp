@@ -17,6 +17,10 @@
 //     fire_conv_bp(spatial, grad_conv, weight_conv, stride, padding, dilation, groups, benchmark,
 //                  deterministic, allow_tf32, dim_conv, alpha, thresh, beta, interval)
 //                                                 -> [grad_spatial, grad_weight_conv, grad_bias_conv]
+// and the batch-norm + fire op (snnlib/cuda/snn.cpp:20-40 region for bn_fire_s_fp, :800; bn_fire_bp :814)
+//     bn_fire_s_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn, alpha, thresh)  -> [ivar, spike]
+//     bn_fire_bp(spatial, weight_bn, bias_bn, ivar, mean, dim_bn, grad_spike, alpha, thresh, beta,
+//                interval)                       -> [grad_spatial, grad_weight_bn, grad_bias_bn]
 // in which the fire part runs on this library's kernels and the linear / convolution part stays on
 // PyTorch-ROCm (rocBLAS / MIOpen through ATen), issued once with the time axis folded into the
 // batch instead of once per time step as the reference's host loops do
@@ -257,6 +261,88 @@ std::vector<torch::Tensor> fire_conv_bp(torch::Tensor spatial, torch::Tensor gra
     return {grad_spatial, grad_weight, grad_bias};
 }
 
+// ---- batch norm folded into the fire recurrence -------------------------------------------------
+
+struct BnDims {
+    int64_t T, B, C, HW;
+};
+
+BnDims bn_dims_of(const torch::Tensor& t, const char* op) {
+    TORCH_CHECK(t.dim() >= 3, "snnlib.", op, ": spatial must be shaped [T, B, C, ...]");
+    const int64_t T = t.size(0), B = t.size(1), C = t.size(2);
+    const int64_t tbc = T * B * C;
+    return BnDims{T, B, C, tbc ? t.numel() / tbc : 0};
+}
+
+torch::Tensor channel_param(const torch::Tensor& p, const torch::Tensor& like, int64_t C,
+                            const char* op, const char* name) {
+    check_param(p, like, op, name);
+    TORCH_CHECK(p.numel() == C, "snnlib.", op, ": ", name, " must have one value per channel (", C,
+                "), got ", p.sizes());
+    return p.contiguous();
+}
+
+std::vector<torch::Tensor> bn_fire_s_fp(torch::Tensor spatial, torch::Tensor weight_bn,
+                                        torch::Tensor bias_bn, torch::Tensor var,
+                                        torch::Tensor mean, float eps_bn, float alpha,
+                                        float thresh) {
+    check_input(spatial, "bn_fire_s_fp", "spatial");
+    TORCH_CHECK(spatial.scalar_type() == at::kFloat,
+                "snnlib.bn_fire_s_fp: only float32 is supported, got ", spatial.scalar_type());
+    const BnDims d = bn_dims_of(spatial, "bn_fire_s_fp");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(spatial.device());
+    torch::Tensor x = spatial.contiguous();
+    torch::Tensor w = channel_param(weight_bn, x, d.C, "bn_fire_s_fp", "weight_bn");
+    torch::Tensor b = channel_param(bias_bn, x, d.C, "bn_fire_s_fp", "bias_bn");
+    torch::Tensor v = channel_param(var, x, d.C, "bn_fire_s_fp", "var");
+    torch::Tensor m = channel_param(mean, x, d.C, "bn_fire_s_fp", "mean");
+    torch::Tensor ivar = torch::empty_like(v, at::MemoryFormat::Contiguous);
+    torch::Tensor spike = torch::empty_like(x, at::MemoryFormat::Contiguous);
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    check_rc(snnlif_bn_fire_s_fp(x.data_ptr(), w.data_ptr(), b.data_ptr(), v.data_ptr(),
+                                 m.data_ptr(), ivar.data_ptr(), spike.data_ptr(), SNNLIF_DTYPE_F32,
+                                 d.T, d.B, d.C, d.HW, eps_bn, alpha, thresh, stream.stream()),
+             "bn_fire_s_fp");
+    return {ivar, spike};
+}
+
+std::vector<torch::Tensor> bn_fire_bp(torch::Tensor spatial, torch::Tensor weight_bn,
+                                      torch::Tensor bias_bn, torch::Tensor ivar, torch::Tensor mean,
+                                      std::vector<int64_t> dim_bn, torch::Tensor grad_spike,
+                                      float alpha, float thresh, float beta, float interval) {
+    // dim_bn names the reduced axes ((0,1) or (0,1,3,4)); they follow from the shape here
+    (void)dim_bn;
+    check_input(spatial, "bn_fire_bp", "spatial");
+    check_input(grad_spike, "bn_fire_bp", "grad_spike");
+    TORCH_CHECK(spatial.scalar_type() == at::kFloat,
+                "snnlib.bn_fire_bp: only float32 is supported, got ", spatial.scalar_type());
+    TORCH_CHECK(spatial.sizes() == grad_spike.sizes() &&
+                    spatial.scalar_type() == grad_spike.scalar_type() &&
+                    spatial.device() == grad_spike.device(),
+                "snnlib.bn_fire_bp: spatial and grad_spike must agree in shape, dtype and device");
+    const BnDims d = bn_dims_of(spatial, "bn_fire_bp");
+    const c10::hip::HIPGuardMasqueradingAsCUDA guard(spatial.device());
+    torch::Tensor x = spatial.contiguous();
+    torch::Tensor g = grad_spike.contiguous();
+    torch::Tensor w = channel_param(weight_bn, x, d.C, "bn_fire_bp", "weight_bn");
+    torch::Tensor b = channel_param(bias_bn, x, d.C, "bn_fire_bp", "bias_bn");
+    torch::Tensor iv = channel_param(ivar, x, d.C, "bn_fire_bp", "ivar");
+    torch::Tensor m = channel_param(mean, x, d.C, "bn_fire_bp", "mean");
+    torch::Tensor grad_spatial = torch::empty_like(x, at::MemoryFormat::Contiguous);
+    torch::Tensor grad_weight = torch::empty_like(w, at::MemoryFormat::Contiguous);
+    torch::Tensor grad_bias = torch::empty_like(w, at::MemoryFormat::Contiguous);
+    const size_t ws_bytes = snnlif_bn_fire_bp_workspace_bytes(SNNLIF_DTYPE_F32, d.T, d.B, d.C, d.HW);
+    torch::Tensor workspace = torch::empty({static_cast<int64_t>(ws_bytes)}, x.options().dtype(at::kByte));
+    auto stream = c10::hip::getCurrentHIPStreamMasqueradingAsCUDA();
+    check_rc(snnlif_bn_fire_bp(x.data_ptr(), w.data_ptr(), b.data_ptr(), iv.data_ptr(), m.data_ptr(),
+                               g.data_ptr(), grad_spatial.data_ptr(), grad_weight.data_ptr(),
+                               grad_bias.data_ptr(), SNNLIF_DTYPE_F32, d.T, d.B, d.C, d.HW, alpha,
+                               thresh, beta, interval, ws_bytes ? workspace.data_ptr() : nullptr,
+                               ws_bytes, stream.stream()),
+             "bn_fire_bp");
+    return {grad_spatial, grad_weight.view_as(weight_bn), grad_bias.view_as(weight_bn)};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -266,6 +352,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("fire_s_fp", &fire_s_fp, "fire (spike) forward");
     m.def("fire_us_fp", &fire_us_fp, "fire (membrane potential, spike) forward");
     m.def("fire_bp", &fire_bp, "fire backward");
+    m.def("bn_fire_s_fp", &bn_fire_s_fp, "bn fire (spike) forward");
+    m.def("bn_fire_bp", &bn_fire_bp, "bn fire backward");
     m.def("fire_fc_fp", &fire_fc_fp, "fire fc forward");
     m.def("fire_fc_bp", &fire_fc_bp, "fire fc backward");
     m.def("fire_conv_fp", &fire_conv_fp, "fire conv forward");

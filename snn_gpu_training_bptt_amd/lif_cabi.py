@@ -12,7 +12,7 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "lib", "libsnnlif_gfx950.so")
 
 DTYPE_F32, DTYPE_F64, DTYPE_BF16 = 0, 1, 2
-OK, ERR_ARG, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN = 0, -1, -2, -3, -4
+OK, ERR_ARG, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_UNSUPPORTED = 0, -1, -2, -3, -4, -5
 BP_FUSED_MAX_T = 32
 
 # name -> (restype, argtypes); must list every symbol include/snnlib_lif.h declares.
@@ -25,6 +25,9 @@ SYMBOLS = {
     "snnlif_fire_us_fp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64]),
     "snnlif_fire_bp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
+    "snnlif_bn_fire_s_fp": (_int, [_vp] * 7 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _vp]),
+    "snnlif_bn_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
+    "snnlif_bn_fire_bp": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
 }
 
 _lib = None
@@ -131,3 +134,42 @@ def fire_bp_into(spatial, grad_spike, grad_spatial, alpha, thresh, beta, interva
                                ws_ptr, ws_bytes, _stream_handle(spatial))
     _check(rc, "snnlif_fire_bp")
     return grad_spatial
+
+
+def _bn_dims(t):
+    T, B, C = t.shape[0], t.shape[1], t.shape[2]
+    HW = t.numel() // (T * B * C) if T * B * C else 0
+    return T, B, C, HW
+
+
+def bn_fire_s_fp_into(spatial, weight, bias, var, mean, ivar, spike, eps, alpha, thresh):
+    """``snnlif_bn_fire_s_fp`` on fp32 device tensors; writes ``ivar`` ([C]) and ``spike``."""
+    _require_dense_gpu(spatial, weight, bias, var, mean, ivar, spike)
+    T, B, C, HW = _bn_dims(spatial)
+    rc = load().snnlif_bn_fire_s_fp(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                    var.data_ptr(), mean.data_ptr(), ivar.data_ptr(),
+                                    spike.data_ptr(), _torch_dtype_code(spatial), T, B, C, HW, eps,
+                                    alpha, thresh, _stream_handle(spatial))
+    _check(rc, "snnlif_bn_fire_s_fp")
+    return ivar, spike
+
+
+def bn_fire_bp_workspace_bytes(dtype_code, T, B, C, HW):
+    return int(load().snnlif_bn_fire_bp_workspace_bytes(dtype_code, T, B, C, HW))
+
+
+def bn_fire_bp_into(spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
+                    grad_bias, alpha, thresh, beta, interval, workspace):
+    """``snnlif_bn_fire_bp`` on fp32 device tensors; ``workspace`` is a uint8 device tensor."""
+    _require_dense_gpu(spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
+                       grad_bias, workspace)
+    T, B, C, HW = _bn_dims(spatial)
+    rc = load().snnlif_bn_fire_bp(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                  ivar.data_ptr(), mean.data_ptr(), grad_spike.data_ptr(),
+                                  grad_spatial.data_ptr(), grad_weight.data_ptr(),
+                                  grad_bias.data_ptr(), _torch_dtype_code(spatial), T, B, C, HW,
+                                  alpha, thresh, beta, interval, workspace.data_ptr(),
+                                  workspace.numel() * workspace.element_size(),
+                                  _stream_handle(spatial))
+    _check(rc, "snnlif_bn_fire_bp")
+    return grad_spatial, grad_weight, grad_bias

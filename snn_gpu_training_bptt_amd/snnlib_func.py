@@ -2,7 +2,7 @@
 
 Same surface as the reference's ``snnlib_func.py`` for the fire path
 (snnlib/example/snnlib_func.py:10-17 for the module-level settings, :22-36 for ``FireFunc`` /
-``fire_func``, :116-132 for ``FireFcFunc`` / ``fire_fc_func``, :197-223 for ``FireConvFunc`` /
+``fire_func``, :67-85 for ``BnFireFunc`` / ``bn_fire_func``, :116-132 for ``FireFcFunc`` / ``fire_fc_func``, :197-223 for ``FireConvFunc`` /
 ``fire_conv_func``): every forward saves only its inputs (never spikes or membrane potentials) and
 calls the native ``snnlib.<op>_fp``; every backward calls ``snnlib.<op>_bp``, which recomputes what
 it needs.  The hyper-parameters are module globals read at call time, so
@@ -41,6 +41,29 @@ class FireFunc(torch.autograd.Function):
 
 
 fire_func = FireFunc.apply
+
+
+class BnFireFunc(torch.autograd.Function):
+    """spike = fire(batch_norm(spatial)) with the given per-channel statistics
+    (snnlib/example/snnlib_func.py:67-85).  Saves the input current, the affine parameters, the
+    inverse standard deviation returned by the forward, and the mean."""
+
+    @staticmethod
+    def forward(ctx, spatial, weight_bn, bias_bn, var, mean, dim_bn, eps_bn):
+        ivar, spike = snnlib.bn_fire_s_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn, alpha, thresh)
+        ctx.save_for_backward(spatial, weight_bn, bias_bn, ivar, mean)
+        ctx.dim_bn = dim_bn
+        return spike
+
+    @staticmethod
+    def backward(ctx, grad_spike):
+        spatial, weight_bn, bias_bn, ivar, mean = ctx.saved_tensors
+        grad_spatial, grad_weight_bn, grad_bias_bn = snnlib.bn_fire_bp(
+            spatial, weight_bn, bias_bn, ivar, mean, ctx.dim_bn, grad_spike, alpha, thresh, beta, interval)
+        return grad_spatial, grad_weight_bn, grad_bias_bn, None, None, None, None
+
+
+bn_fire_func = BnFireFunc.apply
 
 
 class FireFcFunc(torch.autograd.Function):

@@ -1,0 +1,172 @@
+"""Batch-norm + fire on the GPU.
+
+Through the C ABI against the CPU oracle (``oracle/lif_oracle.c``, which follows the reference's
+bn_fire kernels): spikes and the per-channel inverse standard deviation bit-exact (same operation
+order; needs the device's fp32 divide and square root to be correctly rounded, which is part of what
+is being tested); gradients within 1e-5 of the tensor's scale (the reference itself reduces the
+per-channel sums in no defined order).
+
+Through the PyTorch interface against autograd of ``batch_norm`` + the gold fire loop, the way the
+reference's test_bn_fire.py compares its layer with gold_op.BnFire.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import ALPHA, BETA, INTERVAL, THRESH
+
+pytestmark = pytest.mark.gpu
+EPS = 1e-5
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from snn_gpu_training_bptt_amd import lif_cabi
+    lif_cabi.load()
+    return lif_cabi
+
+
+def rel_close(a, b, what, tol=1e-5):
+    scale = np.abs(b).max() + 1e-12
+    err = np.abs(a - b).max()
+    assert err <= tol * scale, f"{what}: max abs err {err:.3e} vs scale {scale:.3e}"
+
+
+def make(shape, seed):
+    gen = torch.Generator().manual_seed(seed)
+    C = shape[2]
+    x = 0.5 + torch.randn(shape, generator=gen) * (0.5 + torch.rand((C,) + (1,) * (len(shape) - 3), generator=gen))
+    g = torch.randn(shape, generator=gen)
+    w = 0.5 + torch.rand(C, generator=gen)
+    b = 0.2 * torch.randn(C, generator=gen)
+    dims = (0, 1) + tuple(range(3, len(shape)))
+    var, mean = torch.var_mean(x, dim=dims, unbiased=False)
+    return x, g, w, b, var, mean
+
+
+SHAPES = [
+    (6, 2, 8),                # the reference test's fc shape
+    (6, 2, 8, 8, 8),          # the reference test's conv shape
+    (8, 16, 32, 16, 16),      # HW = 256
+    (4, 5, 7, 7, 7),          # HW = 49, odd everything
+    (13, 3, 20, 5, 3),        # window without an instantiation of its own
+    (32, 2, 16, 4, 4),
+    (8, 64, 1024),            # fully connected, many channels
+    (8, 32, 128, 32, 32),     # few channels, many positions: exercises the split reduction
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_bn_fire_against_oracle(cabi, shape):
+    from oracle import c_oracle
+    x, g, w, b, var, mean = make(shape, seed=31)
+    T, B, C = shape[:3]
+    HW = int(np.prod(shape[3:])) if len(shape) > 3 else 1
+    dev = lambda t: t.cuda()
+    xd, gd, wd, bd, vd, md = map(dev, (x, g, w, b, var, mean))
+    ivar = torch.empty_like(vd)
+    spike = torch.empty_like(xd)
+    cabi.bn_fire_s_fp_into(xd, wd, bd, vd, md, ivar, spike, EPS, ALPHA, THRESH)
+    gx, gw, gb = torch.empty_like(xd), torch.empty_like(wd), torch.empty_like(wd)
+    ws = torch.empty(cabi.bn_fire_bp_workspace_bytes(cabi.DTYPE_F32, T, B, C, HW), dtype=torch.uint8, device="cuda")
+    cabi.bn_fire_bp_into(xd, wd, bd, ivar, md, gd, gx, gw, gb, ALPHA, THRESH, BETA, INTERVAL, ws)
+    torch.cuda.synchronize()
+
+    ivar_o, _, spike_o = c_oracle.bn_fire_forward(x.numpy(), w.numpy(), b.numpy(), var.numpy(), mean.numpy(), EPS, ALPHA, THRESH)
+    gx_o, gw_o, gb_o = c_oracle.bn_fire_backward(x.numpy(), w.numpy(), b.numpy(), ivar_o, mean.numpy(), g.numpy(),
+                                                 ALPHA, THRESH, BETA, INTERVAL)
+    assert np.array_equal(ivar.cpu().numpy(), ivar_o), "inverse standard deviation differs"
+    assert np.array_equal(spike.cpu().numpy(), spike_o), "spikes differ from the oracle"
+    rel_close(gb.cpu().numpy(), gb_o, "bias gradient")
+    rel_close(gw.cpu().numpy(), gw_o, "weight gradient")
+    rel_close(gx.cpu().numpy(), gx_o, "input-current gradient")
+
+    # reproducibility: the reduction order is fixed
+    gx2, gw2, gb2 = torch.empty_like(xd), torch.empty_like(wd), torch.empty_like(wd)
+    cabi.bn_fire_bp_into(xd, wd, bd, ivar, md, gd, gx2, gw2, gb2, ALPHA, THRESH, BETA, INTERVAL, ws)
+    assert torch.equal(gx, gx2) and torch.equal(gw, gw2) and torch.equal(gb, gb2)
+
+
+def test_identity_statistics_reduce_to_plain_fire(cabi):
+    """mean 0, var 1-eps, weight 1, bias 0 -> scale == 1 exactly and the spikes are those of fire."""
+    gen = torch.Generator().manual_seed(32)
+    x = (0.5 + torch.randn((8, 4, 16, 8, 8), generator=gen)).cuda()
+    C = 16
+    one = torch.ones(C, device="cuda")
+    zero = torch.zeros(C, device="cuda")
+    var = torch.full((C,), 1.0 - EPS, device="cuda")
+    assert float(var[0] + EPS) == 1.0
+    ivar, spike = torch.empty(C, device="cuda"), torch.empty_like(x)
+    cabi.bn_fire_s_fp_into(x, one, zero, var, zero, ivar, spike, EPS, ALPHA, THRESH)
+    plain = torch.empty_like(x)
+    cabi.fire_s_fp_into(x, plain, ALPHA, THRESH)
+    assert torch.equal(spike, plain)
+    assert torch.equal(ivar, one)
+
+
+@pytest.mark.parametrize("shape,dim_bn", [((6, 2, 8), (0, 1)), ((6, 2, 8, 8, 8), (0, 1, 3, 4)), ((8, 8, 32, 16, 16), (0, 1, 3, 4))])
+@pytest.mark.parametrize("train_bn", [True, False])
+def test_bn_fire_layer_like_reference_test(shape, dim_bn, train_bn):
+    from oracle import gold_fire
+    from snn_gpu_training_bptt_amd import snnlib_func as sf
+    from snn_gpu_training_bptt_amd import snnlib_op as sop
+    saved = (sf.alpha, sf.thresh, sf.beta, sf.interval)
+    sf.alpha, sf.thresh, sf.beta, sf.interval = ALPHA, THRESH, BETA, INTERVAL
+    try:
+        torch.manual_seed(33)
+        C = shape[2]
+        x_cpu = torch.randn(shape)
+        w0, b0 = torch.randn(C).abs() + 0.3, torch.randn(C) * 0.3
+        rv, rm = torch.rand(C) + 0.5, torch.randn(C) * 0.1
+        labels = torch.tensor([1, 0] + [0] * (shape[1] - 2))[: shape[1]].cuda()
+        crit = torch.nn.CrossEntropyLoss()
+
+        layer = sop.BnFire(C, dim_bn, EPS).cuda()
+        layer.weight_bn, layer.bias_bn = torch.nn.Parameter(w0.clone().cuda()), torch.nn.Parameter(b0.clone().cuda())
+        layer.running_var, layer.running_mean = torch.nn.Parameter(rv.clone().cuda()), torch.nn.Parameter(rm.clone().cuda())
+        layer.train_bn = train_bn
+        x = x_cpu.cuda().requires_grad_(True)
+        spikes = layer(x)
+        crit(spikes.view(shape[0], shape[1], -1).mean(dim=0), labels).backward()
+
+        xg = x_cpu.cuda().requires_grad_(True)
+        wg, bg = w0.clone().cuda().requires_grad_(True), b0.clone().cuda().requires_grad_(True)
+        run_m, run_v = rm.clone().cuda(), rv.clone().cuda()
+        _, s_ref = gold_fire.gold_bn_fire(xg, wg, bg, run_m, run_v, train_bn, EPS, ALPHA, THRESH, BETA, INTERVAL)
+        crit(s_ref.view(shape[0], shape[1], -1).mean(dim=0), labels).backward()
+
+        mismatches = (spikes.detach() != s_ref.detach()).sum().item()
+        assert mismatches <= max(1, int(1e-5 * spikes.numel())), f"{mismatches} spike mismatches"
+        if mismatches == 0:
+            rel = lambda a, b_, what: rel_close(a.cpu().numpy(), b_.cpu().numpy(), what, tol=2e-5)
+            rel(layer.weight_bn.grad, wg.grad, "weight gradient")
+            rel(layer.bias_bn.grad, bg.grad, "bias gradient")
+            if train_bn:
+                rel(x.grad, xg.grad, "input-current gradient")
+        if train_bn:
+            # running statistics follow nn.BatchNorm's update (momentum 0.1, unbiased variance)
+            torch.testing.assert_close(layer.running_mean.detach(), run_m, rtol=1e-5, atol=1e-6)
+            torch.testing.assert_close(layer.running_var.detach(), run_v, rtol=1e-5, atol=1e-6)
+    finally:
+        sf.alpha, sf.thresh, sf.beta, sf.interval = saved
+
+
+def test_bn_fire_errors(cabi):
+    import snnlib
+    x = torch.zeros(4, 2, 8, device="cuda")
+    p = torch.ones(8, device="cuda")
+    with pytest.raises(RuntimeError, match="float32"):
+        snnlib.bn_fire_s_fp(x.double(), p.double(), p.double(), p.double(), p.double(), EPS, ALPHA, THRESH)
+    with pytest.raises(RuntimeError, match="per channel"):
+        snnlib.bn_fire_s_fp(x, p[:4], p, p, p, EPS, ALPHA, THRESH)
+    lib = cabi.load()
+    big = torch.zeros(40, 2, 8, device="cuda")
+    rc = lib.snnlif_bn_fire_bp(big.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), big.data_ptr(),
+                               big.data_ptr(), p.data_ptr(), p.data_ptr(), 0, 40, 2, 8, 1, ALPHA, THRESH, BETA, INTERVAL,
+                               None, 0, None)
+    assert rc == cabi.ERR_UNSUPPORTED
+    rc = lib.snnlif_bn_fire_bp(x.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), x.data_ptr(),
+                               x.data_ptr(), p.data_ptr(), p.data_ptr(), 0, 4, 2, 8, 1, ALPHA, THRESH, BETA, INTERVAL,
+                               None, 0, None)
+    assert rc == cabi.ERR_WORKSPACE
+    torch.cuda.synchronize()

@@ -281,3 +281,86 @@ def test_scalar_loops_match_autograd_of_the_gold_graph(shape, mean, std, alpha, 
     assert np.array_equal(spike_c, s.numpy())
     assert np.array_equal(mem_c, u.numpy())
     assert np.array_equal(gx_c, gx.numpy())
+
+
+# ---- batch-norm + fire ---------------------------------------------------------------------------
+
+def _bn_case(shape, seed):
+    gen = torch.Generator().manual_seed(seed)
+    C = shape[2]
+    x = 0.5 + torch.randn(shape, generator=gen)
+    g = torch.randn(shape, generator=gen)
+    w = 0.5 + torch.rand(C, generator=gen)
+    b = 0.2 * torch.randn(C, generator=gen)
+    dims = (0, 1) + tuple(range(3, len(shape)))
+    var, mean = torch.var_mean(x, dim=dims, unbiased=False)
+    return x, g, w, b, var, mean
+
+
+def test_bn_fire_with_identity_statistics_is_plain_fire():
+    """mean 0, var + eps == 1, weight 1, bias 0: the affine is exactly the identity, so spikes and
+    potentials equal the plain fire op's and the input gradient is the plain one minus the two
+    batch-norm projection terms computed from it."""
+    eps = 1e-5
+    x, g, _, _, _, _ = _bn_case((5, 3, 4, 6), 40)
+    C = 4
+    one, zero = np.ones(C, np.float32), np.zeros(C, np.float32)
+    var = np.full(C, np.float32(1.0) - np.float32(eps), np.float32)
+    assert np.float32(var[0] + np.float32(eps)) == np.float32(1.0)
+    ivar, mem, spike = c_oracle.bn_fire_forward(x.numpy(), one, zero, var, zero, eps, 0.25, 0.5)
+    mem_p, spike_p = c_oracle.fire_forward(x.numpy(), 0.25, 0.5)
+    assert np.array_equal(ivar, one) and np.array_equal(mem, mem_p) and np.array_equal(spike, spike_p)
+    gx, gw, gb = c_oracle.bn_fire_backward(x.numpy(), one, zero, one, zero, g.numpy(), 0.25, 0.5, 1.0, 0.5)
+    gy = c_oracle.fire_backward(x.numpy(), g.numpy(), 0.25, 0.5, 1.0, 0.5).astype(np.float64)
+    xs = x.numpy().astype(np.float64)
+    axes = (0, 1, 3)
+    np.testing.assert_allclose(gb, gy.sum(axis=axes), rtol=1e-5)
+    np.testing.assert_allclose(gw, (gy * xs).sum(axis=axes), rtol=1e-5, atol=1e-5)
+    expect = gy - gy.mean(axis=axes, keepdims=True) - xs * (gy * xs).mean(axis=axes, keepdims=True)
+    np.testing.assert_allclose(gx, expect, rtol=1e-5, atol=1e-5)
+
+
+def test_bn_fire_single_step_is_textbook_batch_norm_backward():
+    """T = 1: no recurrence; spikes = (bn(x) > thresh) and the backward is batch-norm's with the
+    upstream gradient g * window(bn(x)) * beta (closed form evaluated in float64)."""
+    eps, thresh, beta, interval = 1e-5, 0.5, 0.8, 0.6
+    x, g, w, b, var, mean = _bn_case((1, 6, 3, 5), 41)
+    ivar, mem, spike = c_oracle.bn_fire_forward(x.numpy(), w.numpy(), b.numpy(), var.numpy(), mean.numpy(), eps, 0.25, thresh)
+    xs, gs = x.numpy().astype(np.float64), g.numpy().astype(np.float64)
+    sh = (1, 1, 3, 1)
+    m64, v64 = mean.numpy().astype(np.float64).reshape(sh), var.numpy().astype(np.float64).reshape(sh)
+    w64, b64 = w.numpy().astype(np.float64).reshape(sh), b.numpy().astype(np.float64).reshape(sh)
+    iv64 = 1.0 / np.sqrt(v64 + eps)
+    xhat = (xs - m64) * iv64
+    y = xhat * w64 + b64
+    np.testing.assert_allclose(mem, y, rtol=1e-5, atol=1e-6)
+    safe = np.abs(y - thresh) > 1e-4            # away from the threshold the spike is unambiguous
+    assert np.array_equal(spike[safe], (y > thresh)[safe].astype(np.float32))
+    gy = gs * (np.abs(y - thresh) < interval) * beta
+    axes = (0, 1, 3)
+    gx, gw, gb = c_oracle.bn_fire_backward(x.numpy(), w.numpy(), b.numpy(), ivar, mean.numpy(), g.numpy(),
+                                           0.25, thresh, beta, interval)
+    np.testing.assert_allclose(gb, gy.sum(axis=axes), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(gw, (gy * xhat).sum(axis=axes), rtol=1e-5, atol=1e-6)
+    gxhat = gy * w64
+    expect = iv64 * (gxhat - gxhat.mean(axis=axes, keepdims=True) - xhat * (gxhat * xhat).mean(axis=axes, keepdims=True))
+    np.testing.assert_allclose(gx, expect, rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape", [(6, 4, 8, 8, 8), (6, 16, 8), (3, 2, 5, 7)])
+def test_bn_fire_loops_match_autograd_through_batch_norm(shape):
+    """The C loops (the reference kernels' formulae) against autograd of
+    torch.nn.functional.batch_norm + the gold fire loop: two derivations of the same backward."""
+    eps = 1e-5
+    x, g, w, b, var, mean = _bn_case(shape, 42)
+    ivar, mem, spike = c_oracle.bn_fire_forward(x.numpy(), w.numpy(), b.numpy(), var.numpy(), mean.numpy(), eps, 0.25, 0.5)
+    gx, gw, gb = c_oracle.bn_fire_backward(x.numpy(), w.numpy(), b.numpy(), ivar, mean.numpy(), g.numpy(), 0.25, 0.5, 1.0, 0.5)
+    xr, wr, br = x.clone().requires_grad_(True), w.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    u, s = gold_fire.gold_bn_fire(xr, wr, br, None, None, True, eps, 0.25, 0.5, 1.0, 0.5)
+    s.backward(g)
+    assert np.array_equal(spike, s.detach().numpy())
+    np.testing.assert_allclose(mem, u.detach().numpy(), rtol=1e-5, atol=1e-6)
+    scale = lambda a: np.abs(a).max()
+    assert np.abs(gx - xr.grad.numpy()).max() <= 1e-5 * scale(gx)
+    assert np.abs(gw - wr.grad.numpy()).max() <= 1e-5 * scale(gw)
+    assert np.abs(gb - br.grad.numpy()).max() <= 1e-5 * scale(gb)
