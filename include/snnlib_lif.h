@@ -118,6 +118,19 @@ int snnlif_bn_fire_s_fp(const void* spatial, const void* weight, const void* bia
                         const void* mean, void* ivar, void* spike, int dtype, int64_t T, int64_t B,
                         int64_t C, int64_t HW, float eps, float alpha, float thresh, void* stream);
 
+/*
+ * Spikes of the batch-norm + fire layer recomputed from saved statistics, the way the backward of
+ * the fused layers sees them: scale[c] = weight[c] * ivar[c] (not weight / sqrt(var + eps)), same
+ * recurrence as snnlif_bn_fire_s_fp, fp32 only.  Replaces bn_fire_us_fp_kernel
+ * (snnlib/cuda/snn_kernel_bp.cu:481-530) as used by bn_fire_fc_bp_cuda (:890) and bn_fire_conv_bp_cuda
+ * (:1215); the membrane potential it also writes there is not needed here because
+ * snnlif_bn_fire_bp recomputes it in registers.
+ */
+int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const void* bias,
+                               const void* ivar, const void* mean, void* spike, int dtype, int64_t T,
+                               int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
+                               void* stream);
+
 /* Bytes of device workspace snnlif_bn_fire_bp needs (two floats per neuron plus per-channel
  * staging).  0 for invalid arguments. */
 size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);

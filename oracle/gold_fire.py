@@ -75,3 +75,43 @@ def gold_bn_fire(x, weight, bias, running_mean, running_var, training, eps, alph
     y = torch.nn.functional.batch_norm(x.reshape(shape[0] * shape[1], *shape[2:]), running_mean,
                                        running_var, weight, bias, training, 0.1, eps).reshape(shape)
     return gold_fire(y, alpha, thresh, beta, interval)
+
+
+def _per_step(fn, x):
+    return torch.stack([fn(x[t]) for t in range(x.shape[0])], dim=0)
+
+
+def gold_bn(x, weight, bias, running_mean, running_var, training, eps):
+    """Batch norm over the folded (T*B) batch (snnlib/example/gold_op.py:49-62)."""
+    shape = x.shape
+    return torch.nn.functional.batch_norm(x.reshape(shape[0] * shape[1], *shape[2:]), running_mean,
+                                          running_var, weight, bias, training, 0.1, eps).reshape(shape)
+
+
+def gold_fc(x, weight, bias):
+    """One ``linear`` per time step on the flattened input (snnlib/example/gold_op.py:113-145 with
+    neither ``bn_fire`` nor ``fire``)."""
+    if x.dim() == 5:
+        x = x.view(x.shape[0], x.shape[1], -1)
+    return _per_step(lambda xt: torch.nn.functional.linear(xt, weight, bias), x)
+
+
+def gold_conv(x, weight, bias, stride, padding):
+    """One ``conv2d`` per time step (snnlib/example/gold_op.py:148-179 with neither flag)."""
+    return _per_step(lambda xt: torch.nn.functional.conv2d(xt, weight, bias, stride, padding), x)
+
+
+def gold_bn_fire_fc(x, weight_bn, bias_bn, running_mean, running_var, training, eps, weight_fc, bias_fc,
+                    alpha, thresh, beta=1.0, interval=0.5):
+    """snnlib/example/gold_op.py:113-145 with ``bn_fire=True``."""
+    _, s = gold_bn_fire(x, weight_bn, bias_bn, running_mean, running_var, training, eps, alpha, thresh,
+                        beta, interval)
+    return gold_fc(s, weight_fc, bias_fc)
+
+
+def gold_bn_fire_conv(x, weight_bn, bias_bn, running_mean, running_var, training, eps, weight_conv,
+                      bias_conv, stride, padding, alpha, thresh, beta=1.0, interval=0.5):
+    """snnlib/example/gold_op.py:148-179 with ``bn_fire=True``."""
+    _, s = gold_bn_fire(x, weight_bn, bias_bn, running_mean, running_var, training, eps, alpha, thresh,
+                        beta, interval)
+    return gold_conv(s, weight_conv, bias_conv, stride, padding)

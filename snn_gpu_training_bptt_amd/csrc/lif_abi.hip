@@ -122,8 +122,28 @@ int snnlif_bn_fire_s_fp(const void* spatial, const void* weight, const void* bia
     return snnlif::bn_forward_f32(
         static_cast<const float*>(spatial), static_cast<const float*>(weight),
         static_cast<const float*>(bias), static_cast<const float*>(var),
-        static_cast<const float*>(mean), static_cast<float*>(ivar), static_cast<float*>(spike), T, B,
-        C, HW, eps, alpha, thresh, static_cast<hipStream_t>(stream));
+        static_cast<const float*>(mean), static_cast<float*>(ivar), static_cast<float*>(spike),
+        /*from_ivar=*/false, T, B, C, HW, eps, alpha, thresh, static_cast<hipStream_t>(stream));
+}
+
+int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const void* bias,
+                               const void* ivar, const void* mean, void* spike, int dtype, int64_t T,
+                               int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
+                               void* stream) {
+    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
+    if (dtype != SNNLIF_DTYPE_F32) return SNNLIF_ERR_UNSUPPORTED;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
+    if (!spatial || !weight || !bias || !ivar || !mean || !spike) return SNNLIF_ERR_ARG;
+    const void* ptrs[6] = {spatial, weight, bias, ivar, mean, spike};
+    for (const void* p : ptrs)
+        if (!snnlif::aligned_to(p, sizeof(float))) return SNNLIF_ERR_ALIGN;
+    return snnlif::bn_forward_f32(
+        static_cast<const float*>(spatial), static_cast<const float*>(weight),
+        static_cast<const float*>(bias), static_cast<const float*>(ivar),
+        static_cast<const float*>(mean), nullptr, static_cast<float*>(spike), /*from_ivar=*/true, T,
+        B, C, HW, 0.f, alpha, thresh, static_cast<hipStream_t>(stream));
 }
 
 size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW) {

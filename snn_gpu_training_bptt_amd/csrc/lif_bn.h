@@ -27,9 +27,12 @@ inline size_t bn_backward_workspace_floats(int64_t B, int64_t C, int64_t HW) {
            static_cast<size_t>(2 * C);
 }
 
-int bn_forward_f32(const float* x, const float* weight, const float* bias, const float* var,
-                   const float* mean, float* ivar, float* spike, int64_t T, int64_t B, int64_t C,
-                   int64_t HW, float eps, float alpha, float thresh, hipStream_t stream);
+// from_ivar = false: stat is the variance and ivar is written; true: stat is the inverse standard
+// deviation and ivar is not touched.
+int bn_forward_f32(const float* x, const float* weight, const float* bias, const float* stat,
+                   const float* mean, float* ivar, float* spike, bool from_ivar, int64_t T,
+                   int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,
+                   hipStream_t stream);
 
 int bn_backward_f32(const float* x, const float* weight, const float* bias, const float* ivar,
                     const float* mean, const float* g, float* gx, float* grad_weight,

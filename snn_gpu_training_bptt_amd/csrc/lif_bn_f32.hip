@@ -3,24 +3,40 @@
 
 namespace snnlif {
 
-int bn_forward_f32(const float* x, const float* weight, const float* bias, const float* var,
-                   const float* mean, float* ivar, float* spike, int64_t T, int64_t B, int64_t C,
-                   int64_t HW, float eps, float alpha, float thresh, hipStream_t stream) {
+namespace {
+
+template <bool FROM_IVAR>
+int bn_forward_launch(const float* x, const float* weight, const float* bias, const float* stat,
+                      const float* mean, float* ivar, float* spike, int64_t T, int64_t B, int64_t C,
+                      int64_t HW, float eps, float alpha, float thresh, hipStream_t stream) {
     const int64_t N = B * C * HW;
     const dim3 grid(grid_for(N, kFwdBlock)), block(kFwdBlock);
     const int Ti = static_cast<int>(T);
     constexpr int TC = SNNLIF_FWD_ROWS;
     if (T <= 4 && TC > 4) {
-        hipLaunchKernelGGL((lif_bn_forward_kernel<4, false>), grid, block, 0, stream, x, weight, bias,
-                           var, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
+        hipLaunchKernelGGL((lif_bn_forward_kernel<4, false, FROM_IVAR>), grid, block, 0, stream, x,
+                           weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
     } else if (T <= TC) {
-        hipLaunchKernelGGL((lif_bn_forward_kernel<TC, false>), grid, block, 0, stream, x, weight,
-                           bias, var, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
+        hipLaunchKernelGGL((lif_bn_forward_kernel<TC, false, FROM_IVAR>), grid, block, 0, stream, x,
+                           weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
     } else {
-        hipLaunchKernelGGL((lif_bn_forward_kernel<TC, true>), grid, block, 0, stream, x, weight,
-                           bias, var, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
+        hipLaunchKernelGGL((lif_bn_forward_kernel<TC, true, FROM_IVAR>), grid, block, 0, stream, x,
+                           weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
     }
     return launch_status();
+}
+
+}  // namespace
+
+int bn_forward_f32(const float* x, const float* weight, const float* bias, const float* stat,
+                   const float* mean, float* ivar, float* spike, bool from_ivar, int64_t T,
+                   int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,
+                   hipStream_t stream) {
+    if (from_ivar)
+        return bn_forward_launch<true>(x, weight, bias, stat, mean, ivar, spike, T, B, C, HW, eps,
+                                       alpha, thresh, stream);
+    return bn_forward_launch<false>(x, weight, bias, stat, mean, ivar, spike, T, B, C, HW, eps, alpha,
+                                    thresh, stream);
 }
 
 namespace {

@@ -45,12 +45,16 @@ __device__ __forceinline__ int channel_of(int64_t col, int64_t C, int64_t HW, bo
 }
 
 // ---------------------------------------------------------------------------------------------
-// Forward: spikes (and the inverse standard deviation per channel).
+// Forward: spikes.  FROM_IVAR = false: `stat` is the variance, scale = weight / sqrt(var + eps), and
+// the inverse standard deviation scale / weight is published per channel (the layer's forward).
+// FROM_IVAR = true: `stat` is that inverse standard deviation, scale = weight * ivar, nothing is
+// published (how the backward of the fused layers recomputes the spikes, as the reference's
+// bn_fire_us_fp_kernel does, snnlib/cuda/snn_kernel_bp.cu:481-530).
 // ---------------------------------------------------------------------------------------------
-template <int TC, bool MULTI>
+template <int TC, bool MULTI, bool FROM_IVAR>
 __global__ void __launch_bounds__(kFwdBlock)
 lif_bn_forward_kernel(const float* __restrict__ x, const float* __restrict__ weight,
-                      const float* __restrict__ bias, const float* __restrict__ var,
+                      const float* __restrict__ bias, const float* __restrict__ stat,
                       const float* __restrict__ mean, float* __restrict__ ivar,
                       float* __restrict__ spike, int T, int64_t N, int64_t C, int64_t HW, float eps,
                       float alpha, float thresh) {
@@ -61,10 +65,10 @@ lif_bn_forward_kernel(const float* __restrict__ x, const float* __restrict__ wei
         const int c = channel_of(col, C, HW, small);
         const float m = mean[c];
         const float wgt = weight[c];
-        const float scale = wgt / sqrtf(var[c] + eps);
+        const float scale = FROM_IVAR ? wgt * stat[c] : wgt / sqrtf(stat[c] + eps);
         const float b = bias[c];
         // first neuron of the channel in batch entry 0 publishes the channel's ivar
-        if (col == static_cast<int64_t>(c) * HW) ivar[c] = scale / wgt;
+        if (!FROM_IVAR && col == static_cast<int64_t>(c) * HW) ivar[c] = scale / wgt;
 
         float u = 0.f, s = 0.f;
         Pack<float, 1> cur[TC];

@@ -26,6 +26,7 @@ SYMBOLS = {
     "snnlif_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64]),
     "snnlif_fire_bp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
     "snnlif_bn_fire_s_fp": (_int, [_vp] * 7 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _vp]),
+    "snnlif_bn_fire_s_recompute": (_int, [_vp] * 6 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_bn_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "snnlif_bn_fire_bp": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
 }
@@ -152,6 +153,18 @@ def bn_fire_s_fp_into(spatial, weight, bias, var, mean, ivar, spike, eps, alpha,
                                     alpha, thresh, _stream_handle(spatial))
     _check(rc, "snnlif_bn_fire_s_fp")
     return ivar, spike
+
+
+def bn_fire_s_recompute_into(spatial, weight, bias, ivar, mean, spike, alpha, thresh):
+    """``snnlif_bn_fire_s_recompute``: spikes from saved ``ivar`` / ``mean`` (backward-side scale)."""
+    _require_dense_gpu(spatial, weight, bias, ivar, mean, spike)
+    T, B, C, HW = _bn_dims(spatial)
+    rc = load().snnlif_bn_fire_s_recompute(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                           ivar.data_ptr(), mean.data_ptr(), spike.data_ptr(),
+                                           _torch_dtype_code(spatial), T, B, C, HW, alpha, thresh,
+                                           _stream_handle(spatial))
+    _check(rc, "snnlif_bn_fire_s_recompute")
+    return spike
 
 
 def bn_fire_bp_workspace_bytes(dtype_code, T, B, C, HW):

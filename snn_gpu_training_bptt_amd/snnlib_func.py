@@ -1,12 +1,17 @@
-"""Autograd functions of the LIF fire layers and the hyper-parameters they read.
+"""Autograd functions of the snnlib layers and the hyper-parameters they read.
 
-Same surface as the reference's ``snnlib_func.py`` for the fire path
-(snnlib/example/snnlib_func.py:10-17 for the module-level settings, :22-36 for ``FireFunc`` /
-``fire_func``, :67-85 for ``BnFireFunc`` / ``bn_fire_func``, :116-132 for ``FireFcFunc`` / ``fire_fc_func``, :197-223 for ``FireConvFunc`` /
-``fire_conv_func``): every forward saves only its inputs (never spikes or membrane potentials) and
-calls the native ``snnlib.<op>_fp``; every backward calls ``snnlib.<op>_bp``, which recomputes what
-it needs.  The hyper-parameters are module globals read at call time, so
-``snnlib_func.thresh = 0.5`` takes effect on the next call, as it does in the reference.
+Same surface as the reference's ``snnlib_func.py`` for every single-GPU layer
+(snnlib/example/snnlib_func.py:10-17 module-level settings; ``BnFunc`` :42-59, ``BnFireFunc`` :67-85,
+``BnFireFcFunc`` :91-110, ``FireFcFunc`` :116-132, ``FcFunc`` :138-154, ``BnFireConvFunc`` :162-191,
+``FireConvFunc`` :197-223, ``ConvFunc`` :229-253, ``FireFunc`` :22-36, each with its
+``<name>_func = <Class>.apply`` alias).  The multi-GPU ``*Dist`` functions (:261-379) are not
+provided.
+
+Contract shared by all of them, as in the reference: a forward saves only its *inputs* (plus the
+per-channel inverse standard deviation a batch-norm forward returns) -- never spikes or membrane
+potentials -- and calls the native ``snnlib.<op>_fp``; the backward calls ``snnlib.<op>_bp``, which
+recomputes what it needs.  Hyper-parameters are module globals read at call time, so
+``snnlib_func.thresh = 0.5`` takes effect on the next call.
 """
 import torch
 
@@ -23,9 +28,18 @@ time_step = 6
 
 conv_benchmark = False  # accepted for interface parity; MIOpen's search follows torch.backends.cudnn
 
+_DIM_FC = (0, 1)            # axes a fully connected bias gradient sums over
+_DIM_CONV = (0, 1, 3, 4)    # axes a convolution bias gradient / conv-shaped batch norm sums over
+_DILATION, _GROUPS = (1, 1), 1
+
+
+def _pad(grads, n):
+    """Gradients for the first inputs, ``None`` for the remaining non-tensor ones."""
+    return tuple(grads) + (None,) * (n - len(grads))
+
 
 class FireFunc(torch.autograd.Function):
-    """spike = fire(spatial); only ``spatial`` is kept for the backward."""
+    """spike = fire(spatial)."""
 
     @staticmethod
     def forward(ctx, spatial):
@@ -40,13 +54,24 @@ class FireFunc(torch.autograd.Function):
         return snnlib.fire_bp(spatial, grad_spike, alpha, thresh, beta, interval)
 
 
-fire_func = FireFunc.apply
+class BnFunc(torch.autograd.Function):
+    """y = batch_norm(x) with the per-channel statistics handed in (no fire)."""
+
+    @staticmethod
+    def forward(ctx, x_bn, weight_bn, bias_bn, var, mean, dim_bn, eps_bn):
+        ivar, y_bn = snnlib.bn_fp(x_bn, weight_bn, bias_bn, var, mean, eps_bn)
+        ctx.save_for_backward(x_bn, weight_bn, bias_bn, ivar, mean)
+        ctx.dim_bn = dim_bn
+        return y_bn
+
+    @staticmethod
+    def backward(ctx, grad_y_bn):
+        x_bn, weight_bn, bias_bn, ivar, mean = ctx.saved_tensors
+        return _pad(snnlib.bn_bp(x_bn, weight_bn, bias_bn, ivar, mean, ctx.dim_bn, grad_y_bn), 7)
 
 
 class BnFireFunc(torch.autograd.Function):
-    """spike = fire(batch_norm(spatial)) with the given per-channel statistics
-    (snnlib/example/snnlib_func.py:67-85).  Saves the input current, the affine parameters, the
-    inverse standard deviation returned by the forward, and the mean."""
+    """spike = fire(batch_norm(spatial))."""
 
     @staticmethod
     def forward(ctx, spatial, weight_bn, bias_bn, var, mean, dim_bn, eps_bn):
@@ -58,54 +83,133 @@ class BnFireFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_spike):
         spatial, weight_bn, bias_bn, ivar, mean = ctx.saved_tensors
-        grad_spatial, grad_weight_bn, grad_bias_bn = snnlib.bn_fire_bp(
-            spatial, weight_bn, bias_bn, ivar, mean, ctx.dim_bn, grad_spike, alpha, thresh, beta, interval)
-        return grad_spatial, grad_weight_bn, grad_bias_bn, None, None, None, None
+        return _pad(snnlib.bn_fire_bp(spatial, weight_bn, bias_bn, ivar, mean, ctx.dim_bn, grad_spike,
+                                      alpha, thresh, beta, interval), 7)
 
 
-bn_fire_func = BnFireFunc.apply
-
-
-class FireFcFunc(torch.autograd.Function):
-    """fc = linear(fire(spatial)) per time step; gradients for the input current, weight and bias."""
+class BnFireFcFunc(torch.autograd.Function):
+    """fc = linear(fire(batch_norm(spatial)))."""
 
     @staticmethod
-    def forward(ctx, spatial, weight_fc, bias_fc):
-        fc = snnlib.fire_fc_fp(spatial, weight_fc, bias_fc, alpha, thresh)
-        ctx.save_for_backward(spatial, weight_fc, bias_fc)
+    def forward(ctx, spatial, weight_bn, bias_bn, var, mean, dim_bn, eps_bn, weight_fc, bias_fc):
+        ivar, fc = snnlib.bn_fire_fc_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn,
+                                        weight_fc, bias_fc, alpha, thresh)
+        ctx.save_for_backward(spatial, weight_bn, bias_bn, ivar, mean, weight_fc, bias_fc)
+        ctx.dim_bn = dim_bn
         return fc
 
     @staticmethod
     def backward(ctx, grad_fc):
-        spatial, weight_fc, bias_fc = ctx.saved_tensors
-        grad_spatial, grad_weight_fc, grad_bias_fc = snnlib.fire_fc_bp(
-            spatial, grad_fc, weight_fc, bias_fc, (0, 1), alpha, thresh, beta, interval)
-        return grad_spatial, grad_weight_fc, grad_bias_fc
+        spatial, weight_bn, bias_bn, ivar, mean, weight_fc, bias_fc = ctx.saved_tensors
+        g_spatial, g_weight_bn, g_bias_bn, g_weight_fc, g_bias_fc = snnlib.bn_fire_fc_bp(
+            spatial, weight_bn, bias_bn, ivar, mean, ctx.dim_bn, grad_fc, weight_fc, bias_fc, _DIM_FC,
+            alpha, thresh, beta, interval)
+        return g_spatial, g_weight_bn, g_bias_bn, None, None, None, None, g_weight_fc, g_bias_fc
 
 
-fire_fc_func = FireFcFunc.apply
-
-
-class FireConvFunc(torch.autograd.Function):
-    """conv = conv2d(fire(spatial)) per time step (dilation 1, groups 1, as in the reference)."""
+class FireFcFunc(torch.autograd.Function):
+    """fc = linear(fire(spatial))."""
 
     @staticmethod
-    def forward(ctx, spatial, weight_conv, bias_conv, stride, padding, if_bias_conv):
-        conv = snnlib.fire_conv_fp(spatial, weight_conv, bias_conv, stride, padding, (1, 1), 1,
-                                   conv_benchmark, False, alpha, thresh)
-        ctx.save_for_backward(spatial, weight_conv, bias_conv)
+    def forward(ctx, spatial, weight_fc, bias_fc):
+        ctx.save_for_backward(spatial, weight_fc, bias_fc)
+        return snnlib.fire_fc_fp(spatial, weight_fc, bias_fc, alpha, thresh)
+
+    @staticmethod
+    def backward(ctx, grad_fc):
+        spatial, weight_fc, bias_fc = ctx.saved_tensors
+        return tuple(snnlib.fire_fc_bp(spatial, grad_fc, weight_fc, bias_fc, _DIM_FC,
+                                       alpha, thresh, beta, interval))
+
+
+class FcFunc(torch.autograd.Function):
+    """fc = linear(spatial) per time step (no fire)."""
+
+    @staticmethod
+    def forward(ctx, spatial, weight_fc, bias_fc):
+        ctx.save_for_backward(spatial, weight_fc, bias_fc)
+        return snnlib.fc_fp(spatial, weight_fc, bias_fc)
+
+    @staticmethod
+    def backward(ctx, grad_fc):
+        spatial, weight_fc, bias_fc = ctx.saved_tensors
+        return tuple(snnlib.fc_bp(spatial, grad_fc, weight_fc, bias_fc, _DIM_FC))
+
+
+def _conv_grads(ctx, g_spatial, g_weight, g_bias, leading=()):
+    """Order the convolution-layer gradients the way ``forward``'s arguments are ordered; the bias
+    gradient is dropped when the layer was built with ``if_bias_conv=False``."""
+    return leading + (g_weight, g_bias if ctx.if_bias_conv else None, None, None, None)
+
+
+class BnFireConvFunc(torch.autograd.Function):
+    """conv = conv2d(fire(batch_norm(spatial))) (dilation 1, groups 1, as in the reference)."""
+
+    @staticmethod
+    def forward(ctx, spatial, weight_bn, bias_bn, var, mean, eps_bn,
+                weight_conv, bias_conv, stride, padding, if_bias_conv):
+        ivar, conv = snnlib.bn_fire_conv_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn,
+                                            weight_conv, bias_conv, stride, padding, _DILATION, _GROUPS,
+                                            conv_benchmark, False, alpha, thresh)
+        ctx.save_for_backward(spatial, weight_bn, bias_bn, ivar, mean, weight_conv, bias_conv)
         ctx.stride, ctx.padding, ctx.if_bias_conv = stride, padding, if_bias_conv
         return conv
 
     @staticmethod
     def backward(ctx, grad_conv):
+        spatial, weight_bn, bias_bn, ivar, mean, weight_conv, bias_conv = ctx.saved_tensors
+        g_spatial, g_weight_bn, g_bias_bn, g_weight_conv, g_bias_conv = snnlib.bn_fire_conv_bp(
+            spatial, weight_bn, bias_bn, ivar, mean, _DIM_CONV, grad_conv, weight_conv,
+            ctx.stride, ctx.padding, _DILATION, _GROUPS, conv_benchmark, False, True, _DIM_CONV,
+            alpha, thresh, beta, interval)
+        return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv,
+                           leading=(g_spatial, g_weight_bn, g_bias_bn, None, None, None))
+
+
+class FireConvFunc(torch.autograd.Function):
+    """conv = conv2d(fire(spatial))."""
+
+    @staticmethod
+    def forward(ctx, spatial, weight_conv, bias_conv, stride, padding, if_bias_conv):
+        ctx.save_for_backward(spatial, weight_conv, bias_conv)
+        ctx.stride, ctx.padding, ctx.if_bias_conv = stride, padding, if_bias_conv
+        return snnlib.fire_conv_fp(spatial, weight_conv, bias_conv, stride, padding, _DILATION, _GROUPS,
+                                   conv_benchmark, False, alpha, thresh)
+
+    @staticmethod
+    def backward(ctx, grad_conv):
         spatial, weight_conv, bias_conv = ctx.saved_tensors
-        grad_spatial, grad_weight_conv, grad_bias_conv = snnlib.fire_conv_bp(
-            spatial, grad_conv, weight_conv, ctx.stride, ctx.padding, (1, 1), 1, conv_benchmark,
-            False, True, (0, 1, 3, 4), alpha, thresh, beta, interval)
-        if ctx.if_bias_conv:
-            return grad_spatial, grad_weight_conv, grad_bias_conv, None, None, None
-        return grad_spatial, grad_weight_conv, None, None, None, None
+        g_spatial, g_weight_conv, g_bias_conv = snnlib.fire_conv_bp(
+            spatial, grad_conv, weight_conv, ctx.stride, ctx.padding, _DILATION, _GROUPS,
+            conv_benchmark, False, True, _DIM_CONV, alpha, thresh, beta, interval)
+        return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv, leading=(g_spatial,))
 
 
+class ConvFunc(torch.autograd.Function):
+    """conv = conv2d(spatial) per time step (no fire)."""
+
+    @staticmethod
+    def forward(ctx, spatial, weight_conv, bias_conv, stride, padding, if_bias_conv):
+        ctx.save_for_backward(spatial, weight_conv, bias_conv)
+        ctx.stride, ctx.padding, ctx.if_bias_conv = stride, padding, if_bias_conv
+        return snnlib.conv_fp(spatial, weight_conv, bias_conv, stride, padding, _DILATION, _GROUPS,
+                              conv_benchmark, False)
+
+    @staticmethod
+    def backward(ctx, grad_conv):
+        spatial, weight_conv, bias_conv = ctx.saved_tensors
+        g_spatial, g_weight_conv, g_bias_conv = snnlib.conv_bp(
+            spatial, grad_conv, weight_conv, ctx.stride, ctx.padding, _DILATION, _GROUPS,
+            conv_benchmark, False, True, _DIM_CONV)
+        return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv, leading=(g_spatial,))
+
+
+fire_func = FireFunc.apply
+bn_func = BnFunc.apply
+bn_fire_func = BnFireFunc.apply
+bn_fire_fc_func = BnFireFcFunc.apply
+fire_fc_func = FireFcFunc.apply
+fc_func = FcFunc.apply
+bn_fire_conv_func = BnFireConvFunc.apply
 fire_conv_func = FireConvFunc.apply
+conv_func = ConvFunc.apply

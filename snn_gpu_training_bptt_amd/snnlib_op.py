@@ -1,12 +1,17 @@
-"""Layer modules built on the fire operator.
+"""Layer modules of the snnlib interface (single GPU).
 
-``Fire`` has the reference's surface (snnlib/example/snnlib_op.py:11-16): no constructor
-arguments, no parameters or buffers, ``forward(x) = fire_func(x)`` on a tensor shaped
-``[T, B, C, H, W]`` or ``[T, B, C]``, returning 0.0 / 1.0 spikes of the same shape and dtype.
-``BnFire`` (snnlib/example/snnlib_op.py:53-84) applies a batch norm inside the recurrence.
-``FireFc`` (snnlib/example/snnlib_op.py:131-139) and ``FireConv`` (:195-210) feed those spikes to a
-fully connected / 3x3-style convolution layer; constructor arguments, parameter names and
-initialisation are the reference's.
+Class names, constructor arguments, parameter names and initialisation are the reference's
+(snnlib/example/snnlib_op.py): ``Fire`` :11-16, ``Bn`` :19-50, ``BnFire`` :53-84, ``BnFireFc`` :87-128,
+``FireFc`` :131-139, ``Fc`` :141-149, ``BnFireConv`` :152-192, ``FireConv`` :195-210, ``Conv`` :214-228.
+Inputs are ``[T, B, C, H, W]`` or ``[T, B, C]`` tensors; each module forwards to the matching
+``snnlib_func.<name>_func``.  The ``*Dist`` modules (:231-405, synchronised batch norm over several
+GPUs) are not provided.
+
+Batch-norm behaviour shared by the ``Bn*`` modules, as in the reference: ``train_bn`` (not
+``nn.Module.training``) selects batch statistics (``torch.var_mean(..., unbiased=False)`` over
+``dim_bn``) or the running ones; the running statistics are ``nn.Parameter`` objects that are
+*replaced* on every training-mode call (momentum 0.1, variance corrected by n/(n-1), n = elements
+per channel of the first input seen).
 """
 import math
 
@@ -14,6 +19,51 @@ import torch
 import torch.nn as nn
 
 from . import snnlib_func as sf
+
+
+class _BatchStatistics(nn.Module):
+    """Affine parameters and running statistics of a per-channel batch norm over ``channels``."""
+
+    def _init_batch_norm(self, channels, dim_bn, eps_bn):
+        self.dim_bn = dim_bn
+        self.eps_bn = eps_bn
+        self._bn_channels = channels
+        self.weight_bn = nn.Parameter(torch.ones(channels))
+        self.bias_bn = nn.Parameter(torch.zeros(channels))
+        self.running_var = nn.Parameter(torch.ones(channels))
+        self.running_mean = nn.Parameter(torch.zeros(channels))
+        self.factor = None
+        self.train_bn = True
+
+    def _statistics(self, x):
+        """(var, mean) to normalise ``x`` with; updates the running pair in training mode."""
+        if self.factor is None:
+            per_channel = x.numel() / self._bn_channels
+            self.factor = per_channel / (per_channel - 1)
+            self.running_var = self.running_var.to(x.device)
+            self.running_mean = self.running_mean.to(x.device)
+        if not self.train_bn:
+            return self.running_var, self.running_mean
+        var, mean = torch.var_mean(x, dim=self.dim_bn, unbiased=False)
+        self.running_var = nn.Parameter(self.running_var * 0.9 + var * (0.1 * self.factor))
+        self.running_mean = nn.Parameter(self.running_mean * 0.9 + mean * 0.1)
+        return var, mean
+
+
+def _fc_parameters(module, cin, cout, like_linear):
+    if like_linear:   # nn.Linear's default initialisation
+        fc = nn.Linear(cin, cout, bias=True)
+        module.weight_fc, module.bias_fc = nn.Parameter(fc.weight), nn.Parameter(fc.bias)
+    else:             # N(0, 0.75/sqrt(cin)) weights, zero bias
+        module.weight_fc = nn.Parameter(nn.init.normal_(torch.zeros(cout, cin), 0, 0.75 / math.sqrt(cin)))
+        module.bias_fc = nn.Parameter(torch.zeros(cout))
+
+
+def _conv_attributes(module, cin, stride, padding, if_bias_conv):
+    module.cin = cin
+    module.stride = stride
+    module.padding = padding
+    module.if_bias_conv = if_bias_conv
 
 
 class Fire(nn.Module):
@@ -24,62 +74,84 @@ class Fire(nn.Module):
         return sf.fire_func(x)
 
 
-class BnFire(nn.Module):
-    """Batch norm folded into the fire recurrence (snnlib/example/snnlib_op.py:53-84).
+class Bn(_BatchStatistics):
+    def __init__(self, cin, dim_bn, eps_bn=1e-5):
+        super(Bn, self).__init__()
+        self.cin = cin
+        self._init_batch_norm(cin, dim_bn, eps_bn)
 
-    ``dim_bn`` names the axes the statistics run over: ``(0, 1)`` for ``[T, B, C]`` inputs,
-    ``(0, 1, 3, 4)`` for ``[T, B, C, H, W]``.  As in the reference, the running statistics are held
-    as ``nn.Parameter`` objects that are *replaced* on every training-mode call (momentum 0.1, the
-    variance corrected by n/(n-1)), and ``train_bn`` -- not ``nn.Module.training`` -- selects between
-    batch and running statistics.
-    """
+    def forward(self, x):
+        var, mean = self._statistics(x)
+        return sf.bn_func(x, self.weight_bn, self.bias_bn, var, mean, self.dim_bn, self.eps_bn)
 
+
+class BnFire(_BatchStatistics):
     def __init__(self, cin, dim_bn, eps_bn=1e-5):
         super(BnFire, self).__init__()
         self.cin = cin
-        self.dim_bn = dim_bn
-        self.eps_bn = eps_bn
-        self.weight_bn = nn.Parameter(torch.ones(cin))
-        self.bias_bn = nn.Parameter(torch.zeros(cin))
-        self.running_var = nn.Parameter(torch.ones(cin))
-        self.running_mean = nn.Parameter(torch.zeros(cin))
-        self.factor = None
-        self.train_bn = True
+        self._init_batch_norm(cin, dim_bn, eps_bn)
 
     def forward(self, x):
-        if self.factor is None:
-            factor = x.numel() / self.cin
-            self.factor = factor / (factor - 1)
-            self.running_var = self.running_var.to(x.device)
-            self.running_mean = self.running_mean.to(x.device)
-
-        if self.train_bn:
-            var, mean = torch.var_mean(x, dim=self.dim_bn, unbiased=False)
-            self.running_var = nn.Parameter(self.running_var * 0.9 + var * (0.1 * self.factor))
-            self.running_mean = nn.Parameter(self.running_mean * 0.9 + mean * 0.1)
-        else:
-            var, mean = self.running_var, self.running_mean
-
+        var, mean = self._statistics(x)
         return sf.bn_fire_func(x, self.weight_bn, self.bias_bn, var, mean, self.dim_bn, self.eps_bn)
+
+
+class BnFireFc(_BatchStatistics):
+    """``cin_bn`` is the channel count of the batch norm when the input is still an image
+    (``[T, B, cin_bn, H, W]`` with ``cin = cin_bn*H*W`` features for the linear layer)."""
+
+    def __init__(self, cin, cout, dim_bn, eps_bn=1e-5, cin_bn=None):
+        super(BnFireFc, self).__init__()
+        self.cin = cin
+        self.cin_bn = cin if cin_bn is None else cin_bn
+        self._init_batch_norm(self.cin_bn, dim_bn, eps_bn)
+        _fc_parameters(self, cin, cout, like_linear=True)
+
+    def forward(self, x):
+        var, mean = self._statistics(x)
+        return sf.bn_fire_fc_func(x, self.weight_bn, self.bias_bn, var, mean, self.dim_bn, self.eps_bn,
+                                  self.weight_fc, self.bias_fc)
 
 
 class FireFc(nn.Module):
     def __init__(self, cin, cout):
         super(FireFc, self).__init__()
-        self.weight_fc = nn.Parameter(nn.init.normal_(torch.zeros(cout, cin), 0, 0.75 / math.sqrt(cin)))
-        self.bias_fc = nn.Parameter(torch.zeros(cout))
+        _fc_parameters(self, cin, cout, like_linear=False)
 
     def forward(self, x):
         return sf.fire_fc_func(x, self.weight_fc, self.bias_fc)
 
 
+class Fc(nn.Module):
+    def __init__(self, cin, cout):
+        super(Fc, self).__init__()
+        _fc_parameters(self, cin, cout, like_linear=False)
+
+    def forward(self, x):
+        return sf.fc_func(x, self.weight_fc, self.bias_fc)
+
+
+class BnFireConv(_BatchStatistics):
+    def __init__(self, cin, cout, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), eps_bn=1e-5,
+                 if_bias_conv=True):
+        super(BnFireConv, self).__init__()
+        _conv_attributes(self, cin, stride, padding, if_bias_conv)
+        self._init_batch_norm(cin, (0, 1, 3, 4), eps_bn)
+        conv = nn.Conv2d(cin, cout, kernel_size, stride, padding)
+        self.weight_conv = nn.Parameter(conv.weight)
+        self.bias_conv = nn.Parameter(conv.bias)
+
+    def forward(self, x):
+        var, mean = self._statistics(x)
+        return sf.bn_fire_conv_func(x, self.weight_bn, self.bias_bn, var, mean, self.eps_bn,
+                                    self.weight_conv, self.bias_conv, self.stride, self.padding,
+                                    self.if_bias_conv)
+
+
 class FireConv(nn.Module):
     def __init__(self, cin, cout, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), if_bias_conv=True):
         super(FireConv, self).__init__()
-        self.cin = cin
-        self.stride = stride
-        self.padding = padding
-        self.if_bias_conv = if_bias_conv
+        _conv_attributes(self, cin, stride, padding, if_bias_conv)
         conv = nn.Conv2d(cin, cout, kernel_size, stride, padding)
         self.weight_conv = nn.Parameter(conv.weight)
         self.bias_conv = nn.Parameter(conv.bias)
@@ -87,3 +159,16 @@ class FireConv(nn.Module):
     def forward(self, x):
         return sf.fire_conv_func(x, self.weight_conv, self.bias_conv, self.stride, self.padding,
                                  self.if_bias_conv)
+
+
+class Conv(nn.Module):
+    def __init__(self, cin, cout, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), if_bias_conv=True):
+        super(Conv, self).__init__()
+        _conv_attributes(self, cin, stride, padding, if_bias_conv)
+        self.weight_conv = nn.Parameter(nn.init.normal_(
+            torch.zeros(cout, cin, kernel_size[0], kernel_size[1]), 0, 0.75 / math.sqrt(cin)))
+        self.bias_conv = nn.Parameter(torch.zeros(cout))
+
+    def forward(self, x):
+        return sf.conv_func(x, self.weight_conv, self.bias_conv, self.stride, self.padding,
+                            self.if_bias_conv)
