@@ -4,6 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg5_bf16|cfg1]
                     [--no-cpu-baseline]
     python bench.py --workload train_step [--steps K] [--warmup W]     (context figure, see below)
+    python bench.py --workload bn_fire    [--steps K] [--warmup W]     (next-row op, see below)
 
 One "step" is one forward (spikes from the input current) plus one backward (input gradient from
 the saved input current and the spike gradient) over one synthetic batch that is already resident
@@ -27,6 +28,11 @@ pre-allocated outputs.  The default workload is the headline configuration
 spiking CNN on CIFAR-shaped random data (conv / linear / pooling on PyTorch-ROCm, the four LIF layers
 through ``snnlib_op.Fire``) and reports the end-to-end step time and the share of it spent in the
 fire kernels, measured with events around the ``snnlib.fire_s_fp`` / ``snnlib.fire_bp`` calls.
+
+``--workload bn_fire`` times the batch-norm + fire op (``snnlif_bn_fire_s_fp`` / ``snnlif_bn_fire_bp``)
+at the headline shape through the C ABI: 8 B per neuron-step forward, 20 B backward (two sweeps over
+x and the spike gradient, one write of the input gradient), checked against the CPU oracle on a
+sample of channels.
 """
 import argparse
 import json
@@ -200,12 +206,86 @@ def run_train_step(args):
     }), flush=True)
 
 
+def run_bn_fire(args):
+    import numpy as np
+    import torch
+    from snn_gpu_training_bptt_amd import lif_cabi
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no ROCm GPU visible")
+    lif_cabi.load()
+    dev = torch.device("cuda:0")
+    shape = (8, 64, 128, 32, 32)
+    T, B, C, HW = shape[0], shape[1], shape[2], shape[3] * shape[4]
+    ns = T * B * C * HW
+    eps = 1e-5
+    gen = torch.Generator(device=dev).manual_seed(SEED)
+    x = 0.5 + torch.randn(shape, generator=gen, device=dev)
+    g = torch.randn(shape, generator=gen, device=dev)
+    weight = 0.5 + torch.rand(C, generator=gen, device=dev)
+    bias = 0.2 * torch.randn(C, generator=gen, device=dev)
+    var, mean = torch.var_mean(x, dim=(0, 1, 3, 4), unbiased=False)
+    ivar, spike = torch.empty_like(var), torch.empty_like(x)
+    gx, gw, gb = torch.empty_like(x), torch.empty_like(weight), torch.empty_like(weight)
+    ws = torch.empty(lif_cabi.bn_fire_bp_workspace_bytes(lif_cabi.DTYPE_F32, T, B, C, HW),
+                     dtype=torch.uint8, device=dev)
+
+    def fwd():
+        lif_cabi.bn_fire_s_fp_into(x, weight, bias, var, mean, ivar, spike, eps, ALPHA, THRESH)
+
+    def bwd():
+        lif_cabi.bn_fire_bp_into(x, weight, bias, ivar, mean, g, gx, gw, gb, ALPHA, THRESH, BETA,
+                                 INTERVAL, ws)
+
+    for _ in range(args.warmup):
+        fwd()
+        bwd()
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for k in range(args.steps):
+        ev[k][0].record()
+        fwd()
+        ev[k][1].record()
+        bwd()
+        ev[k][2].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+
+    # parity on a sample of channels (channels are independent given their statistics)
+    from oracle import c_oracle
+    pick = [0, 1, C // 2, C - 1]
+    take = lambda t: t[:, :8, pick].contiguous().cpu().numpy()
+    p = lambda t: t[pick].cpu().numpy()
+    ivar_o, _, spike_o = c_oracle.bn_fire_forward(take(x), p(weight), p(bias), p(var), p(mean), eps, ALPHA, THRESH)
+    result = {
+        "metric": "BnFire fwd+bwd neuron-steps/s (next-row op, not the headline metric)",
+        "value": ns * args.steps / wall, "unit": "neuron-steps/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3, "higher_is_better": True,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"bn_fire: batch-norm + LIF fire fwd+bwd, [T,B,C,H,W]={list(shape)} float32, "
+                               f"batch statistics, eps={eps}, alpha={ALPHA} thresh={THRESH} beta={BETA} interval={INTERVAL}"},
+        "roofline": {"kernel": "lif_bn_backward_partial_kernel + bn_channel_reduce/finalize + lif_bn_backward_input_kernel",
+                     "bound": "hbm", "algorithmic_bytes_per_launch": 20 * ns, "avg_launch_ms": bwd_ms,
+                     "achieved": 20 * ns / (bwd_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": 20 * ns / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "fwd": {"algorithmic_bytes_per_launch": 8 * ns, "avg_launch_ms": fwd_ms,
+                             "achieved": 8 * ns / (fwd_ms * 1e-3) / 1e9,
+                             "frac": 8 * ns / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
+        "parity": {"sampled_spikes_bit_exact": bool(np.array_equal(take(spike), spike_o)),
+                   "sampled_ivar_bit_exact": bool(np.array_equal(p(ivar), ivar_o))},
+    }
+    print(json.dumps(result), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step"])
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step", "bn_fire"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain device copies of the input tensor (known size: one "
@@ -223,6 +303,9 @@ def main():
         if args.warmup == 20:
             args.warmup = 3
         return run_train_step(args)
+
+    if args.workload == "bn_fire":
+        return run_bn_fire(args)
 
     import torch
     from snn_gpu_training_bptt_amd import lif_cabi

@@ -58,29 +58,43 @@ int bn_backward_window(const float* x, const float* weight, const float* bias, c
     constexpr bool can_be_inexact = TW > 8;
     const bool exact = !can_be_inexact || (T == TW);
 
+    // Wavefronts are channel-uniform when every aligned group of 64 neurons stays inside one
+    // (batch entry, channel) plane.
+    const bool wave = (HW % 64) == 0;
+    int rc;
+#define SNNLIF_BN_PARTIAL(EXACT_, WAVE_)                                                          \
+    hipLaunchKernelGGL((lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_>), grid, block, 0, stream, \
+                       x, g, weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha,     \
+                       thresh, beta, interval)
     if (exact) {
-        hipLaunchKernelGGL((lif_bn_backward_partial_kernel<TW, true>), grid, block, 0, stream, x, g,
-                           weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha, thresh,
-                           beta, interval);
+        if (wave) SNNLIF_BN_PARTIAL(true, true); else SNNLIF_BN_PARTIAL(true, false);
     } else if constexpr (can_be_inexact) {
-        hipLaunchKernelGGL((lif_bn_backward_partial_kernel<TW, false>), grid, block, 0, stream, x, g,
-                           weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha, thresh,
-                           beta, interval);
+        if (wave) SNNLIF_BN_PARTIAL(false, true); else SNNLIF_BN_PARTIAL(false, false);
     }
-    int rc = launch_status();
+#undef SNNLIF_BN_PARTIAL
+    rc = launch_status();
     if (rc != SNNLIF_OK) return rc;
 
-    const int64_t bs = (B + S - 1) / S;
-    hipLaunchKernelGGL(bn_channel_reduce_kernel, dim3(static_cast<unsigned>(C), S),
-                       dim3(kReduceBlock), 0, stream, part_gy, part_gyx, split, B, C, HW, bs, S);
-    rc = launch_status();
-    if (rc != SNNLIF_OK) return rc;
-    hipLaunchKernelGGL(bn_channel_finalize_kernel,
-                       dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
-                       dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias, coef, C,
-                       S, static_cast<float>(T * B * HW));
-    rc = launch_status();
-    if (rc != SNNLIF_OK) return rc;
+    const float count = static_cast<float>(T * B * HW);
+    if (wave) {
+        hipLaunchKernelGGL(bn_channel_reduce_finalize_kernel, dim3(static_cast<unsigned>(C)),
+                           dim3(kReduceBlock), 0, stream, part_gy, part_gyx, weight, grad_weight,
+                           grad_bias, coef, B, C, HW / 64, count);
+        rc = launch_status();
+        if (rc != SNNLIF_OK) return rc;
+    } else {
+        const int64_t bs = (B + S - 1) / S;
+        hipLaunchKernelGGL(bn_channel_reduce_kernel, dim3(static_cast<unsigned>(C), S),
+                           dim3(kReduceBlock), 0, stream, part_gy, part_gyx, split, B, C, HW, bs, S);
+        rc = launch_status();
+        if (rc != SNNLIF_OK) return rc;
+        hipLaunchKernelGGL(bn_channel_finalize_kernel,
+                           dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
+                           dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias,
+                           coef, C, S, count);
+        rc = launch_status();
+        if (rc != SNNLIF_OK) return rc;
+    }
 
     if (exact) {
         hipLaunchKernelGGL((lif_bn_backward_input_kernel<TW, true>), grid, block, 0, stream, x, g,

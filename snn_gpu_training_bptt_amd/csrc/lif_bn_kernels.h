@@ -17,14 +17,16 @@
 // Mapping.  Same lanes as the plain fire kernels (one neuron per lane, time in registers).  The
 // backward needs per-channel sums over everything before any input gradient can be formed, so it
 // is two sweeps over (x, g) with a reduction between them:
-//   1. lif_bn_backward_partial_kernel: reverse chain per neuron, sums over its T steps -> two
-//      floats per neuron (1/T of a tensor, not a tensor);
-//   2. bn_channel_reduce_kernel / bn_channel_finalize_kernel: per-channel sums of those partials
-//      (wavefront shuffles, then LDS across the waves of a workgroup; the only place in this library
-//      where lanes cooperate), in a fixed order -> bit-reproducible results;
+//   1. lif_bn_backward_partial_kernel: reverse chain per neuron, sums over its T steps, and -- when
+//      a wavefront's 64 neurons share a channel (HW % 64 == 0) -- over the wavefront by shuffles:
+//      two floats per 64 neurons (per neuron otherwise);
+//   2. bn_channel_reduce_finalize_kernel (or bn_channel_reduce_kernel + bn_channel_finalize_kernel
+//      for per-neuron partials): per-channel sums of those partials (wavefront shuffles, then LDS
+//      across the waves of a workgroup; the only place in this library where lanes cooperate), in
+//      an order fixed by the launch geometry -> bit-reproducible results;
 //   3. lif_bn_backward_input_kernel: the chain again (x and g re-read: 8 B per neuron-step, the
 //      same as storing and re-loading gy would cost) and the input gradient.
-// HBM traffic: forward 8 B, backward 20 B (+ 16/T B) per neuron-step; the reference moves 8 and 36.
+// HBM traffic: forward 8 B, backward 20 B (+ at most 16/T B) per neuron-step; the reference moves 8 and 36.
 #ifndef SNNLIF_LIF_BN_KERNELS_H
 #define SNNLIF_LIF_BN_KERNELS_H
 
@@ -149,8 +151,17 @@ __device__ __forceinline__ void bn_reverse_chain(const float* __restrict__ x,
     }
 }
 
-// Sweep 1: per-neuron sums over time of gy and gy * xhat.
-template <int TW, bool EXACT>
+// Sum over the 64 lanes of a wavefront; lane 0 holds the result.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
+    return v;
+}
+
+// Sweep 1: sums over time of gy and gy * xhat, per neuron (WAVE = false) or, when every aligned
+// group of 64 neurons lies inside one channel plane (HW % 64 == 0), already summed over the
+// wavefront: one pair of floats per 64 neurons (WAVE = true; part_* then hold N/64 entries).
+template <int TW, bool EXACT, bool WAVE>
 __global__ void __launch_bounds__(kBwdBlock)
 lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restrict__ g,
                                const float* __restrict__ weight, const float* __restrict__ bias,
@@ -173,8 +184,17 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
                                         acc_gy += gy;
                                         acc_gyx += gy * xhat;
                                     });
-        part_gy[col] = acc_gy;
-        part_gyx[col] = acc_gyx;
+        if (WAVE) {
+            acc_gy = wave_sum(acc_gy);
+            acc_gyx = wave_sum(acc_gyx);
+            if ((threadIdx.x & 63) == 0) {
+                part_gy[col >> 6] = acc_gy;
+                part_gyx[col >> 6] = acc_gyx;
+            }
+        } else {
+            part_gy[col] = acc_gy;
+            part_gyx[col] = acc_gyx;
+        }
     }
 }
 
@@ -212,12 +232,6 @@ lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restric
 // (consecutive addresses), so the sum order is fixed by the geometry alone.
 // split = {gy[S][C], gyx[S][C]}.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
-    return v;
-}
-
 __global__ void __launch_bounds__(kReduceBlock)
 bn_channel_reduce_kernel(const float* __restrict__ part_gy, const float* __restrict__ part_gyx,
                          float* __restrict__ split, int64_t B, int64_t C, int64_t HW, int64_t bs,
@@ -263,6 +277,48 @@ bn_channel_reduce_kernel(const float* __restrict__ part_gy, const float* __restr
         }
         split[static_cast<int64_t>(s) * C + c] = ta;
         split[static_cast<int64_t>(S) * C + static_cast<int64_t>(s) * C + c] = tax;
+    }
+}
+
+// Whole reduction of one channel in one workgroup, for partials that are few (the wave-summed
+// form): sums the B*G entries of channel c (G entries per batch entry), then writes the parameter
+// gradients and the two coefficients of the input-gradient sweep.
+__global__ void __launch_bounds__(kReduceBlock)
+bn_channel_reduce_finalize_kernel(const float* __restrict__ part_gy,
+                                  const float* __restrict__ part_gyx,
+                                  const float* __restrict__ weight, float* __restrict__ grad_weight,
+                                  float* __restrict__ grad_bias, float* __restrict__ coef,
+                                  int64_t B, int64_t C, int64_t G, float count) {
+    const int c = blockIdx.x;
+    const int64_t n = B * G;
+    float a = 0.f, ax = 0.f;
+    for (int64_t e = threadIdx.x; e < n; e += kReduceBlock) {
+        const int64_t b = e / G, i = e % G;
+        const int64_t at = (b * C + c) * G + i;
+        a += part_gy[at];
+        ax += part_gyx[at];
+    }
+    __shared__ float lds[2][kReduceBlock / 64];
+    a = wave_sum(a);
+    ax = wave_sum(ax);
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    if (lane == 0) {
+        lds[0][wave] = a;
+        lds[1][wave] = ax;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float ta = 0.f, tax = 0.f;
+#pragma unroll
+        for (int w = 0; w < kReduceBlock / 64; ++w) {
+            ta += lds[0][w];
+            tax += lds[1][w];
+        }
+        grad_bias[c] = ta;
+        grad_weight[c] = tax;
+        const float wgt = weight[c];
+        coef[c] = (ta * wgt) / count;
+        coef[C + c] = (tax * wgt) / count;
     }
 }
 
