@@ -56,6 +56,11 @@ WORKLOADS = {
     "cfg5": ((16, 128, 512, 16, 16), 0.5, 1.0, "float32"),
     "cfg5_bf16": ((16, 128, 512, 16, 16), 0.5, 1.0, "bfloat16"),
 }
+# HBM bytes per launch of the backward kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
+# this file (each counter scaled by its reading for a plain device copy of the same tensor:
+# --copy-calibration); the summary with the commands is profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt.
+# Counters cannot be read from inside this process, so workloads without a profiled figure report null.
+MEASURED_TRAFFIC_BYTES = {"cfg2": 805276475}
 METRIC = "LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T=8,B=64,C=128,32x32"
 
 
@@ -404,7 +409,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": bwd_gbps / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "algorithmic_bytes_per_launch": bytes_bwd,
             "avg_launch_ms": bwd_ms,
             "fwd": {"kernel": "lif_forward_kernel", "algorithmic_bytes_per_launch": bytes_fwd,
