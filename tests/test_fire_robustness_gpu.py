@@ -1,0 +1,122 @@
+"""Robustness of the fire kernels beyond the benchmark shapes: tensors whose element index does not
+fit 32 bits (the reference indexes with ``int``: snnlib/cuda/snn_kernel_fp.cu:45, :60-63), capture into
+a HIP graph with replays, and concurrent launches on two streams."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import ALPHA, BETA, INTERVAL, THRESH
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from snn_gpu_training_bptt_amd import lif_cabi
+    lif_cabi.load()
+    return lif_cabi
+
+
+def test_element_index_beyond_32_bits(cabi):
+    """T=3 rows of 2**31 + 4096 neurons: the last row starts past element 2**32."""
+    from oracle import c_oracle
+    T, N = 3, (1 << 31) + 4096
+    need = 4 * T * N * 4
+    free, _ = torch.cuda.mem_get_info()
+    if free < need + (8 << 30):
+        pytest.skip(f"needs {need >> 30} GiB of device memory")
+    gen = torch.Generator(device="cuda").manual_seed(77)
+    x = torch.empty((T, 1, N), device="cuda")
+    g = torch.empty((T, 1, N), device="cuda")
+    for t in range(T):          # row-wise: keeps the generator's temporaries small
+        x[t].normal_(0.5, 1.0, generator=gen)
+        g[t].normal_(0.0, 1.0, generator=gen)
+    spike = torch.empty_like(x)
+    gx = torch.empty_like(x)
+    cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+    cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+    torch.cuda.synchronize()
+    # neurons at both ends, around the 2**31 boundary and a random sample
+    idx = torch.cat([torch.arange(0, 2048), torch.arange((1 << 31) - 1024, (1 << 31) + 1024),
+                     torch.arange(N - 2048, N),
+                     torch.randint(0, N, (50_000,), generator=torch.Generator().manual_seed(3))]).cuda()
+    take = lambda t: t.view(T, N)[:, idx].cpu().numpy().reshape(T, 1, -1)
+    _, spike_o = c_oracle.fire_forward(take(x), ALPHA, THRESH)
+    gx_o = c_oracle.fire_backward(take(x), take(g), ALPHA, THRESH, BETA, INTERVAL)
+    assert np.array_equal(take(spike), spike_o)
+    assert np.array_equal(take(gx), gx_o)
+    del x, g, spike, gx
+    torch.cuda.empty_cache()
+
+
+def test_hip_graph_capture_and_replay(cabi):
+    """Forward + backward captured once, replayed with fresh inputs and eager work in between: every
+    replay must equal the eager result (the entry points allocate nothing and record no memsets)."""
+    from oracle import c_oracle
+    shape = (8, 4, 64, 16, 16)
+    gen = torch.Generator().manual_seed(78)
+    x = torch.empty(shape, device="cuda")
+    g = torch.empty(shape, device="cuda")
+    spike = torch.empty_like(x)
+    gx = torch.empty_like(x)
+    x.copy_(0.5 + torch.randn(shape, generator=gen))
+    g.copy_(torch.randn(shape, generator=gen))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):          # warm-up on the capture stream, as torch recommends
+        cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+        cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+        cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+
+    for rep in range(4):
+        x_cpu = 0.5 + torch.randn(shape, generator=gen)
+        g_cpu = torch.randn(shape, generator=gen)
+        x.copy_(x_cpu)
+        g.copy_(g_cpu)
+        spike.fill_(-1.0)
+        gx.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        _, spike_o = c_oracle.fire_forward(x_cpu.numpy(), ALPHA, THRESH)
+        gx_o = c_oracle.fire_backward(x_cpu.numpy(), g_cpu.numpy(), ALPHA, THRESH, BETA, INTERVAL)
+        assert np.array_equal(spike.cpu().numpy(), spike_o), f"replay {rep}: spikes"
+        assert np.array_equal(gx.cpu().numpy(), gx_o), f"replay {rep}: gradients"
+        # eager work between replays
+        eager = torch.empty_like(x)
+        cabi.fire_s_fp_into(x, eager, ALPHA, THRESH)
+        assert torch.equal(eager, spike)
+
+
+def test_two_streams_concurrently(cabi):
+    from oracle import c_oracle
+    shape = (8, 8, 64, 32, 32)
+    gen = torch.Generator().manual_seed(79)
+    data = []
+    for _ in range(2):
+        x_cpu = 0.5 + torch.randn(shape, generator=gen)
+        g_cpu = torch.randn(shape, generator=gen)
+        data.append((x_cpu, g_cpu, x_cpu.cuda(), g_cpu.cuda()))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = []
+    for (x_cpu, g_cpu, x, g), st in zip(data, streams):
+        with torch.cuda.stream(st):
+            spike, gx = torch.empty_like(x), torch.empty_like(x)
+            for _ in range(3):          # several rounds so the two streams overlap
+                cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+                cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+            outs.append((spike, gx))
+    for st in streams:
+        st.synchronize()
+    for (x_cpu, g_cpu, _, _), (spike, gx) in zip(data, outs):
+        _, spike_o = c_oracle.fire_forward(x_cpu.numpy(), ALPHA, THRESH)
+        gx_o = c_oracle.fire_backward(x_cpu.numpy(), g_cpu.numpy(), ALPHA, THRESH, BETA, INTERVAL)
+        assert np.array_equal(spike.cpu().numpy(), spike_o)
+        assert np.array_equal(gx.cpu().numpy(), gx_o)
