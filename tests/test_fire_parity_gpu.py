@@ -159,3 +159,31 @@ def test_misaligned_views_take_narrow_lanes(cabi, oracle):
     gx_o = oracle.fire_backward(x.numpy(), g.numpy(), ALPHA, THRESH, BETA, INTERVAL)
     assert np.array_equal(spike.cpu().numpy(), spike_o)
     assert np.array_equal(gx.cpu().numpy(), gx_o)
+
+
+def test_special_values_follow_ieee_like_the_oracle(cabi, oracle):
+    """Denormals (must not be flushed), signed zeros, infinities and NaNs in the input current and in
+    the spike gradient: the kernels must produce the oracle's values, NaNs in the same places."""
+    T, N = 6, 512
+    gen = torch.Generator().manual_seed(4321)
+    x = 0.5 + torch.randn((T, 1, N), generator=gen)
+    g = torch.randn((T, 1, N), generator=gen)
+    specials = torch.tensor([1e-40, -1e-40, 1.4e-45, 0.0, -0.0, float("inf"), -float("inf"),
+                             float("nan"), 3.0e38, -3.0e38, 0.5, 1.0, 1.17549435e-38])
+    for k, v in enumerate(specials):
+        x[k % T, 0, 7 * k] = v            # one special per neuron, at varying time steps
+        g[(k + 2) % T, 0, 7 * k + 100] = v
+    x[:, 0, 300:364] *= 1e-39             # whole neurons in the denormal range
+    g[:, 0, 364:428] *= 1e-41
+    alpha, thresh, beta, interval = 0.5, 0.0, 1.0, 1.0e38   # wide window so denormal paths carry gradient
+    outs = run_gpu(cabi, x, g, alpha, thresh, beta, interval)
+    mem, spike_a, spike_b, gx = (o.numpy() for o in outs)
+    mem_o, spike_o = oracle.fire_forward(x.numpy(), alpha, thresh)
+    gx_o = oracle.fire_backward(x.numpy(), g.numpy(), alpha, thresh, beta, interval)
+    assert np.array_equal(spike_a, spike_o) and np.array_equal(spike_b, spike_o)
+    assert np.array_equal(np.isnan(mem), np.isnan(mem_o))
+    assert np.array_equal(mem[~np.isnan(mem)], mem_o[~np.isnan(mem_o)])
+    assert np.array_equal(np.isnan(gx), np.isnan(gx_o))
+    assert np.array_equal(gx[~np.isnan(gx)], gx_o[~np.isnan(gx_o)])
+    # the denormal neurons really exercised denormal arithmetic
+    assert (np.abs(mem_o[:, 0, 300:364]) < 1.2e-38).all() and (mem_o[:, 0, 300:364] != 0).any()
