@@ -187,3 +187,36 @@ def test_special_values_follow_ieee_like_the_oracle(cabi, oracle):
     assert np.array_equal(gx[~np.isnan(gx)], gx_o[~np.isnan(gx_o)])
     # the denormal neurons really exercised denormal arithmetic
     assert (np.abs(mem_o[:, 0, 300:364]) < 1.2e-38).all() and (mem_o[:, 0, 300:364] != 0).any()
+
+
+@pytest.mark.parametrize("shape", [(8, 3, 255), (5, 1, 1), (16, 2, 4097), (33, 3, 77), (12, 4, 64, 4, 4)])
+def test_bf16_storage_parity_including_odd_sizes(cabi, oracle, shape):
+    """bf16 storage, fp32 arithmetic: two values per lane when N is even and the bases are 4-byte
+    aligned, one otherwise.  Expected = the fp32 oracle on the bf16-rounded inputs, outputs rounded
+    once to bf16 (spikes are exact either way)."""
+    x32, g32 = make_inputs(shape, 0.5, 1.0, seed=2468)
+    x, g = x32.bfloat16(), g32.bfloat16()
+    mem, spike_a, spike_b, gx = run_gpu(cabi, x, g)
+    mem_o, spike_o = oracle.fire_forward(x.float().numpy(), ALPHA, THRESH)
+    gx_o = oracle.fire_backward(x.float().numpy(), g.float().numpy(), ALPHA, THRESH, BETA, INTERVAL)
+    assert np.array_equal(spike_a.float().numpy(), spike_o)
+    assert np.array_equal(spike_b.float().numpy(), spike_o)
+    assert torch.equal(mem, torch.from_numpy(mem_o).bfloat16())
+    assert torch.equal(gx, torch.from_numpy(gx_o).bfloat16())
+
+
+def test_bf16_misaligned_base_takes_single_lanes(cabi, oracle):
+    T, N = 8, 1024
+    x32, g32 = make_inputs((T, 1, N), 0.5, 1.0, seed=1357)
+    x, g = x32.bfloat16(), g32.bfloat16()
+    off = 1  # one bf16: 2-byte aligned only
+    view = lambda: torch.empty(T * N + off, dtype=torch.bfloat16, device="cuda")[off:].view(T, 1, N)
+    xd, gd, spike, gx = view().copy_(x), view().copy_(g), view(), view()
+    assert xd.data_ptr() % 4 == 2
+    cabi.fire_s_fp_into(xd, spike, ALPHA, THRESH)
+    cabi.fire_bp_into(xd, gd, gx, ALPHA, THRESH, BETA, INTERVAL)
+    torch.cuda.synchronize()
+    _, spike_o = oracle.fire_forward(x.float().numpy(), ALPHA, THRESH)
+    gx_o = oracle.fire_backward(x.float().numpy(), g.float().numpy(), ALPHA, THRESH, BETA, INTERVAL)
+    assert np.array_equal(spike.float().cpu().numpy(), spike_o)
+    assert torch.equal(gx.cpu(), torch.from_numpy(gx_o).bfloat16())
