@@ -12,9 +12,13 @@
  *   - Tensors are dense row-major [T, N]: T time steps, N = B*C*H*W (or B*C) neurons; element
  *     (t, n) sits at index t*N + n (reference indexing: snnlib/cuda/snn_kernel_fp.cu:45 with
  *     b*CHW + i folded into n -- neurons are independent, so the batch axis needs no loop).
+ *     The batch-norm entry points need the channel of a neuron and therefore take the neuron axis
+ *     as B, C, HW (N = B*C*HW, neuron (b, c, k) at (b*C + c)*HW + k); per-channel vectors are [C].
  *   - All pointers are DEVICE pointers on the current HIP device.  Inputs are only read; outputs
  *     are fully overwritten.  Nothing is allocated, nothing is kept between calls, so calls are
- *     thread-safe and may be issued on any stream.
+ *     thread-safe and may be issued on any stream (also under HIP graph capture: only kernel
+ *     launches are enqueued).  Scratch memory, where an entry point needs any, is the caller's
+ *     `workspace` argument.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only enqueue
  *     work; they never synchronise.
  *   - `dtype` selects the storage type of every tensor argument (see SNNLIF_DTYPE_*).  Arithmetic
