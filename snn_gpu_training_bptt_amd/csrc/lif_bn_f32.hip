@@ -58,12 +58,14 @@ int bn_backward_window(const float* x, const float* weight, const float* bias, c
     constexpr bool can_be_inexact = TW > 8;
     const bool exact = !can_be_inexact || (T == TW);
 
-    // Wavefronts are channel-uniform when every aligned group of 64 neurons stays inside one
-    // (batch entry, channel) plane.
-    const bool wave = (HW % 64) == 0;
+    // Planes with few positions (fully connected shapes) would leave most lanes of a plane-aligned
+    // wavefront idle; they keep one lane per neuron and per-neuron partials.
+    const bool wave = HW >= 32;
+    const int64_t G = (HW + 63) / 64;
+    const dim3 grid_partial(wave ? grid_for(B * C * G * 64, kBwdBlock) : grid_for(N, kBwdBlock));
     int rc;
 #define SNNLIF_BN_PARTIAL(EXACT_, WAVE_)                                                          \
-    hipLaunchKernelGGL((lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_>), grid, block, 0, stream, \
+    hipLaunchKernelGGL((lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_>), grid_partial, block, 0, stream, \
                        x, g, weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha,     \
                        thresh, beta, interval)
     if (exact) {
@@ -79,7 +81,7 @@ int bn_backward_window(const float* x, const float* weight, const float* bias, c
     if (wave) {
         hipLaunchKernelGGL(bn_channel_reduce_finalize_kernel, dim3(static_cast<unsigned>(C)),
                            dim3(kReduceBlock), 0, stream, part_gy, part_gyx, weight, grad_weight,
-                           grad_bias, coef, B, C, HW / 64, count);
+                           grad_bias, coef, B, C, G, count);
         rc = launch_status();
         if (rc != SNNLIF_OK) return rc;
     } else {

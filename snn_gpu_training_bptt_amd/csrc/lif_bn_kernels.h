@@ -17,9 +17,9 @@
 // Mapping.  Same lanes as the plain fire kernels (one neuron per lane, time in registers).  The
 // backward needs per-channel sums over everything before any input gradient can be formed, so it
 // is two sweeps over (x, g) with a reduction between them:
-//   1. lif_bn_backward_partial_kernel: reverse chain per neuron, sums over its T steps, and -- when
-//      a wavefront's 64 neurons share a channel (HW % 64 == 0) -- over the wavefront by shuffles:
-//      two floats per 64 neurons (per neuron otherwise);
+//   1. lif_bn_backward_partial_kernel: reverse chain per neuron, sums over its T steps, and -- for
+//      planes of at least 32 positions, over which wavefronts are laid so that all 64 lanes share a
+//      channel -- over the wavefront by shuffles: two floats per wavefront (per neuron otherwise);
 //   2. bn_channel_reduce_finalize_kernel (or bn_channel_reduce_kernel + bn_channel_finalize_kernel
 //      for per-neuron partials): per-channel sums of those partials (wavefront shuffles, then LDS
 //      across the waves of a workgroup; the only place in this library where lanes cooperate), in
@@ -158,9 +158,12 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// Sweep 1: sums over time of gy and gy * xhat, per neuron (WAVE = false) or, when every aligned
-// group of 64 neurons lies inside one channel plane (HW % 64 == 0), already summed over the
-// wavefront: one pair of floats per 64 neurons (WAVE = true; part_* then hold N/64 entries).
+// Sweep 1: sums over time of gy and gy * xhat.
+// WAVE = false: one lane per neuron in storage order, one pair of floats per neuron.
+// WAVE = true: wavefronts are laid over the (batch entry, channel) planes -- G = ceil(HW/64)
+// wavefronts per plane, the last one partly idle when HW is not a multiple of 64 -- so all lanes of
+// a wavefront share a channel and their sums are folded by shuffles: one pair of floats per
+// wavefront, part_* indexed [plane][chunk] (B*C*G entries).
 template <int TW, bool EXACT, bool WAVE>
 __global__ void __launch_bounds__(kBwdBlock)
 lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restrict__ g,
@@ -171,27 +174,49 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
                                float beta, float interval) {
     const bool small = N <= 0xffffffffll;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
-    for (int64_t col = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; col < N;
-         col += stride) {
-        const int c = channel_of(col, C, HW, small);
-        const float m = mean[c], iv = ivar[c];
-        const float scale = weight[c] * iv;
-        const float b = bias[c];
-        float acc_gy = 0.f, acc_gyx = 0.f;
-        bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval,
-                                    [&](int, float gy, float xt) {
-                                        const float xhat = (xt - m) * iv;
-                                        acc_gy += gy;
-                                        acc_gyx += gy * xhat;
-                                    });
-        if (WAVE) {
+    if (WAVE) {
+        const int64_t G = (HW + 63) / 64;
+        const int64_t lanes = (N / HW) * G * 64;  // padded lane space: planes * G wavefronts
+        for (int64_t pc = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; pc < lanes;
+             pc += stride) {
+            const int64_t wave = pc >> 6;
+            const int64_t plane = wave / G;
+            const int64_t k = (wave - plane * G) * 64 + (pc & 63);  // position inside the plane
+            const int c = static_cast<int>(plane % C);
+            float acc_gy = 0.f, acc_gyx = 0.f;
+            if (k < HW) {
+                const int64_t col = plane * HW + k;
+                const float m = mean[c], iv = ivar[c];
+                const float scale = weight[c] * iv;
+                const float b = bias[c];
+                bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
+                                            interval, [&](int, float gy, float xt) {
+                                                const float xhat = (xt - m) * iv;
+                                                acc_gy += gy;
+                                                acc_gyx += gy * xhat;
+                                            });
+            }
             acc_gy = wave_sum(acc_gy);
             acc_gyx = wave_sum(acc_gyx);
-            if ((threadIdx.x & 63) == 0) {
-                part_gy[col >> 6] = acc_gy;
-                part_gyx[col >> 6] = acc_gyx;
+            if ((pc & 63) == 0) {
+                part_gy[wave] = acc_gy;
+                part_gyx[wave] = acc_gyx;
             }
-        } else {
+        }
+    } else {
+        for (int64_t col = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; col < N;
+             col += stride) {
+            const int c = channel_of(col, C, HW, small);
+            const float m = mean[c], iv = ivar[c];
+            const float scale = weight[c] * iv;
+            const float b = bias[c];
+            float acc_gy = 0.f, acc_gyx = 0.f;
+            bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval,
+                                        [&](int, float gy, float xt) {
+                                            const float xhat = (xt - m) * iv;
+                                            acc_gy += gy;
+                                            acc_gyx += gy * xhat;
+                                        });
             part_gy[col] = acc_gy;
             part_gyx[col] = acc_gyx;
         }

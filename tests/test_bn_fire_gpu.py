@@ -48,7 +48,10 @@ SHAPES = [
     (6, 2, 8),                # the reference test's fc shape
     (6, 2, 8, 8, 8),          # the reference test's conv shape
     (8, 16, 32, 16, 16),      # HW = 256
-    (4, 5, 7, 7, 7),          # HW = 49, odd everything
+    (4, 5, 7, 7, 7),          # HW = 49: one partly idle wavefront per plane
+    (6, 3, 6, 14, 14),        # HW = 196: four wavefronts per plane, the last with 4 active lanes
+    (5, 2, 3, 4, 8),          # HW = 32: the smallest plane-aligned case
+    (5, 2, 9, 31),            # HW = 31: just below it, one lane per neuron
     (13, 3, 20, 5, 3),        # window without an instantiation of its own
     (32, 2, 16, 4, 4),
     (8, 64, 1024),            # fully connected, many channels
