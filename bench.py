@@ -423,6 +423,12 @@ def main():
 
     if not args.no_cpu_baseline:
         best, threads, (s_ref, gx_ref) = cpu_baseline(torch, x_cpu, g_cpu)
+        # per-core figure: one thread on the first eighth of the batch
+        b8 = max(1, shape[1] // 8)
+        torch.set_num_threads(1)
+        best_1t, _, _ = cpu_baseline(torch, x_cpu[:, :b8].contiguous(), g_cpu[:, :b8].contiguous(), repeats=2)
+        torch.set_num_threads(threads)
+        ns_1t = n_steps_total // shape[1] * b8
         total_s, fwd_s, bwd_s = best
         s_gpu = spike.float().cpu()
         gx_gpu = gx.float().cpu()
@@ -441,6 +447,8 @@ def main():
             "fwd_s": fwd_s,
             "bwd_s": bwd_s,
             "host_cpus": os.cpu_count(),
+            "one_thread": {"value": ns_1t / best_1t[0], "unit": "neuron-steps/s", "cores": 1,
+                           "sample": f"batch entries [0, {b8}) of the same tensor, best of 2"},
         }
         result["parity"] = {
             "spikes_bit_exact": bool(torch.equal(s_gpu, s_ref)),
