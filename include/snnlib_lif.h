@@ -52,9 +52,12 @@ extern "C" {
 #define SNNLIF_ERR_ALIGN      -4 /* a pointer is not aligned to its element size */
 #define SNNLIF_ERR_UNSUPPORTED -5 /* valid arguments this entry point does not implement (see its comment) */
 
-/* Largest T for which the backward keeps the recomputed membrane potential in registers and
- * therefore needs no workspace. */
+/* Largest T for which the backward keeps the whole recomputed membrane potential in registers
+ * (one kernel, 12 bytes per neuron-step in fp32). */
 #define SNNLIF_BP_FUSED_MAX_T 32
+/* Largest T for which snnlif_fire_bp needs no workspace: up to here longer windows are processed
+ * in register-sized segments whose boundary potentials live in LDS (16 bytes per neuron-step). */
+#define SNNLIF_BP_NO_WORKSPACE_MAX_T 1024
 
 /* ABI version of the loaded library (== SNNLIF_ABI_VERSION it was built with). */
 int snnlif_abi_version(void);
@@ -87,7 +90,7 @@ int snnlif_fire_us_fp(const void* spatial, void* mem, void* spike, int dtype, in
 
 /*
  * Bytes of device workspace snnlif_fire_bp needs for this shape: 0 when
- * T <= SNNLIF_BP_FUSED_MAX_T (membrane potential recomputed into registers), otherwise
+ * T <= SNNLIF_BP_NO_WORKSPACE_MAX_T (membrane potential recomputed on chip), otherwise
  * T*N*sizeof(arithmetic type) for the recomputed membrane potential (the reference always
  * allocates this tensor: `mem`, snnlib/cuda/snn_kernel_bp.cu:154).  Returns 0 for invalid arguments.
  */

@@ -71,7 +71,7 @@ int snnlif_fire_s_fp(const void* spatial, void* spike, int dtype, int64_t T, int
 size_t snnlif_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t N) {
     const size_t es = arith_size(dtype);
     if (es == 0 || shape_error(T, N) != SNNLIF_OK) return 0;
-    if (T <= SNNLIF_BP_FUSED_MAX_T) return 0;
+    if (T <= SNNLIF_BP_NO_WORKSPACE_MAX_T) return 0;
     return static_cast<size_t>(T) * static_cast<size_t>(N) * es;
 }
 

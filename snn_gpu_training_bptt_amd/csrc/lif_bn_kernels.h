@@ -165,7 +165,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // a wavefront share a channel and their sums are folded by shuffles: one pair of floats per
 // wavefront, part_* indexed [plane][chunk] (B*C*G entries).
 template <int TW, bool EXACT, bool WAVE>
-__global__ void __launch_bounds__(kBwdBlock)
+__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
 lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restrict__ g,
                                const float* __restrict__ weight, const float* __restrict__ bias,
                                const float* __restrict__ ivar, const float* __restrict__ mean,
@@ -225,7 +225,7 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
 
 // Sweep 2: input gradient.  coef = {gxhat[C], gxhatx[C]}.
 template <int TW, bool EXACT>
-__global__ void __launch_bounds__(kBwdBlock)
+__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
 lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restrict__ g,
                              const float* __restrict__ weight, const float* __restrict__ bias,
                              const float* __restrict__ ivar, const float* __restrict__ mean,

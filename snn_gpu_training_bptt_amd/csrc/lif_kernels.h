@@ -41,8 +41,10 @@
 //     element-wise CPU/GPU ops do, which makes spikes, potentials and gradients bit-identical to
 //     the per-op rounded reference arithmetic.
 //
-// Longer windows (T > 32) use the same forward kernel to write u to a caller-provided workspace
-// and a streaming reverse kernel that reads it back.
+// Longer windows (32 < T <= 1024) are cut into 32-step segments: one forward pass leaves the
+// membrane potential at the segment boundaries in LDS, then each segment is recomputed into registers
+// and swept in reverse, last segment first (x is read twice, nothing else changes).  Beyond that the
+// forward kernel writes u to a caller-provided workspace and a streaming reverse kernel reads it back.
 #ifndef SNNLIF_LIF_KERNELS_H
 #define SNNLIF_LIF_KERNELS_H
 
@@ -84,7 +86,24 @@
 #define SNNLIF_BWD_GCHUNK 8
 #endif
 
+// Upper bound on resident wavefronts per SIMD of a kernel (the compiler spends the freed register
+// budget; the hardware then cannot co-schedule more).
+#define SNNLIF_WAVES_PER_SIMD(n) __attribute__((amdgpu_waves_per_eu(1, (n))))
+
 namespace snnlif {
+
+// Wavefronts per SIMD the backward kernels allow themselves for a register window of `rows` time
+// steps.  A wavefront keeps 2*rows row requests in flight; past roughly 100 of them per SIMD the
+// streams of different wavefronts start to evict each other's DRAM pages, and measured bandwidth
+// drops (by 4 % at 16 rows and 9 % at 32 rows with all 8 wavefronts resident; windows of up to 8
+// rows are best left uncapped).  SNNLIF_BWD_MAX_WAVES overrides.
+constexpr int backward_waves(int rows) {
+#ifdef SNNLIF_BWD_MAX_WAVES
+    return SNNLIF_BWD_MAX_WAVES;
+#else
+    return rows <= 8 ? 8 : (rows <= 12 ? 5 : 4);
+#endif
+}
 
 constexpr int kLaneBytes = SNNLIF_LANE_BYTES;
 constexpr int lane_vec(size_t elem_bytes) {
@@ -265,111 +284,209 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fused backward for a window of at most TW rows: recompute u[0..T-1] into registers, then sweep t
-// downwards.  EXACT = true: T == TW, straight-line code.  EXACT = false: T < TW; rows t >= T are
-// not fetched (zeros stand in for them), the recomputation runs over all TW rows (rows past T only
-// produce values nobody reads) and the reverse sweep skips them.
+// One register-resident backward window of at most TW rows, for the neuron(s) at column `col`.
+// Row pointers x, g, gx are those of the window's first row.  On entry uc / sc hold the membrane
+// potential and spike of the step before the window (zeros at t = 0) and gu the gradient carried
+// in from the step after it (zero at the end of time); on exit gu is the gradient of the window's
+// first step, ready for the window before.
+// EXACT = true: `rows` == TW, straight-line code.  EXACT = false: rows < TW; rows t >= `rows` are
+// not fetched (zeros stand in for them), the recomputation runs over all TW rows (rows past the end
+// only produce values nobody reads) and the reverse sweep skips them.
 // Gradient rows are fetched in groups of at most GC, the newest time steps first; the fetch of the
 // next (earlier) group is issued before the current group is consumed.
 // ---------------------------------------------------------------------------------------------
 template <typename S, int V, int TW, bool EXACT>
-__global__ void __launch_bounds__(kBwdBlock)
-lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
-                          int T, int64_t N, int64_t nvec, typename Arith<S>::type alpha,
-                          typename Arith<S>::type thresh, typename Arith<S>::type beta,
-                          typename Arith<S>::type interval) {
+__device__ __forceinline__ void backward_window(const S* __restrict__ x, const S* __restrict__ g,
+                                                S* __restrict__ gx, int rows, int64_t N,
+                                                int64_t col, typename Arith<S>::type (&uc)[V],
+                                                typename Arith<S>::type (&sc)[V],
+                                                typename Arith<S>::type (&gu)[V],
+                                                typename Arith<S>::type alpha,
+                                                typename Arith<S>::type thresh,
+                                                typename Arith<S>::type beta,
+                                                typename Arith<S>::type interval) {
     using C = typename Arith<S>::type;
     constexpr int GC = (TW < SNNLIF_BWD_GCHUNK) ? TW : SNNLIF_BWD_GCHUNK;
     constexpr int NG = (TW + GC - 1) / GC;  // groups; group 0 holds the newest rows
     // group q covers rows [lo(q), hi(q)) with hi(q) = TW - q*GC and lo(q) = max(0, hi(q) - GC)
 
+    Pack<S, V> xin[TW];
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+        if (EXACT) {
+            xin[t] = load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
+        } else {
+            xin[t] = zero_pack<S, V>();
+            if (t < rows) xin[t] = load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
+        }
+    }
+    Pack<S, V> gbuf[2][GC];
+#pragma unroll
+    for (int t = TW - 1; t >= ((TW - GC) > 0 ? (TW - GC) : 0); --t) {
+        const int k = t - ((TW - GC) > 0 ? (TW - GC) : 0);
+        if (EXACT) {
+            gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+        } else {
+            gbuf[0][k] = zero_pack<S, V>();
+            if (t < rows) gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+        }
+    }
+
+    C u[TW][V];
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            lif_step<C>(uc[j], sc[j], Arith<S>::load(xin[t].e[j]), alpha, thresh);
+            u[t][j] = uc[j];
+        }
+    }
+
+#pragma unroll
+    for (int q = 0; q < NG; ++q) {
+        const int hi = TW - q * GC;
+        const int lo = (hi - GC) > 0 ? (hi - GC) : 0;
+        if (q + 1 < NG) {
+            const int nhi = lo;
+            const int nlo = (nhi - GC) > 0 ? (nhi - GC) : 0;
+#pragma unroll
+            for (int t = nhi - 1; t >= nlo; --t) {
+                if (EXACT) {
+                    gbuf[(q + 1) & 1][t - nlo] =
+                        load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+                } else {
+                    gbuf[(q + 1) & 1][t - nlo] = zero_pack<S, V>();
+                    if (t < rows)
+                        gbuf[(q + 1) & 1][t - nlo] =
+                            load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = hi - 1; t >= lo; --t) {
+            if (EXACT || t < rows) {
+                Pack<S, V> out;
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    lif_reverse_step<C>(gu[j], u[t][j], Arith<S>::load(gbuf[q & 1][t - lo].e[j]),
+                                        alpha, thresh, beta, interval);
+                    out.e[j] = Arith<S>::store(gu[j]);
+                }
+                store_pack<S, V>(gx + static_cast<int64_t>(t) * N + col, out);
+            }
+        }
+    }
+}
+
+// Column a lane works on: the backward walks the neuron axis from its end (see the file header).
+__device__ __forceinline__ int64_t backward_column(int64_t v, int64_t nvec, int V) {
+#if SNNLIF_BWD_DESCENDING
+    return (nvec - 1 - v) * V;
+#else
+    return v * V;
+#endif
+}
+
+// ---------------------------------------------------------------------------------------------
+// Fused backward for T <= TW: the whole time axis is one register window.
+// ---------------------------------------------------------------------------------------------
+template <typename S, int V, int TW, bool EXACT>
+__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
+lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
+                          int T, int64_t N, int64_t nvec, typename Arith<S>::type alpha,
+                          typename Arith<S>::type thresh, typename Arith<S>::type beta,
+                          typename Arith<S>::type interval) {
+    using C = typename Arith<S>::type;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
     for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < nvec;
          v += stride) {
-#if SNNLIF_BWD_DESCENDING
-        const int64_t col = (nvec - 1 - v) * V;
-#else
-        const int64_t col = v * V;
-#endif
-
-        Pack<S, V> xin[TW];
+        const int64_t col = backward_column(v, nvec, V);
+        C uc[V], sc[V], gu[V];
 #pragma unroll
-        for (int t = 0; t < TW; ++t) {
-            if (EXACT) {
-                xin[t] = load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
-            } else {
-                xin[t] = zero_pack<S, V>();
-                if (t < T) xin[t] = load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
-            }
+        for (int j = 0; j < V; ++j) {
+            uc[j] = C(0);
+            sc[j] = C(0);
+            gu[j] = C(0);
         }
-        Pack<S, V> gbuf[2][GC];
+        backward_window<S, V, TW, EXACT>(x, g, gx, T, N, col, uc, sc, gu, alpha, thresh, beta,
+                                         interval);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Segmented backward for windows longer than one register window (kSegment steps).  Two phases per
+// lane, no scratch memory in HBM:
+//   1. run the recurrence forward over all but the last segment and keep the membrane potential at
+//      every segment boundary in LDS (one value per neuron and segment, in a slot only this lane
+//      touches: no synchronisation; the spike flag at a boundary is u > thresh);
+//   2. from the last segment to the first, recompute that segment's u into registers from its
+//      boundary value and sweep it in reverse, carrying the gradient across segments.
+// x is read twice (12 + 4 = 16 bytes per neuron-step in fp32); the second read of the last
+// segments usually still hits the caches.  Dynamic LDS: ceil(T/kSegment) * kBwdBlock * V values.
+// ---------------------------------------------------------------------------------------------
+constexpr int kSegment = 32;
+
+template <typename S, int V>
+__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(kSegment))
+lif_backward_segmented_kernel(const S* __restrict__ x, const S* __restrict__ g,
+                              S* __restrict__ gx, int T, int64_t N, int64_t nvec,
+                              typename Arith<S>::type alpha, typename Arith<S>::type thresh,
+                              typename Arith<S>::type beta, typename Arith<S>::type interval) {
+    using C = typename Arith<S>::type;
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    C* boundary = reinterpret_cast<C*>(lds_raw);  // [segment][lane][V]
+    const int nseg = (T + kSegment - 1) / kSegment;
+    constexpr int ROWS = 8;  // rows requested at a time in phase 1
+    static_assert(kSegment % ROWS == 0, "a segment is a whole number of phase-1 groups");
+
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < nvec;
+         v += stride) {
+        const int64_t col = backward_column(v, nvec, V);
+        C uc[V], sc[V], gu[V];
 #pragma unroll
-        for (int t = TW - 1; t >= ((TW - GC) > 0 ? (TW - GC) : 0); --t) {
-            const int k = t - ((TW - GC) > 0 ? (TW - GC) : 0);
-            if (EXACT) {
-                gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
-            } else {
-                gbuf[0][k] = zero_pack<S, V>();
-                if (t < T) gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
-            }
+        for (int j = 0; j < V; ++j) {
+            uc[j] = C(0);
+            sc[j] = C(0);
+            gu[j] = C(0);
         }
 
-        C u[TW][V];
+        // phase 1: all full segments before the last one
+        for (int seg = 0; seg + 1 < nseg; ++seg) {
+            for (int t0 = seg * kSegment; t0 < (seg + 1) * kSegment; t0 += ROWS) {
+                Pack<S, V> rows[ROWS];
+#pragma unroll
+                for (int k = 0; k < ROWS; ++k)
+                    rows[k] = load_pack<S, V, false>(x + static_cast<int64_t>(t0 + k) * N + col);
+#pragma unroll
+                for (int k = 0; k < ROWS; ++k) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j)
+                        lif_step<C>(uc[j], sc[j], Arith<S>::load(rows[k].e[j]), alpha, thresh);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < V; ++j)
+                boundary[(static_cast<int64_t>(seg + 1) * kBwdBlock + threadIdx.x) * V + j] = uc[j];
+        }
+
+        // phase 2: the last (possibly partial) segment first; uc / sc already hold its boundary
         {
-            C uc[V], sc[V];
+            const int t0 = (nseg - 1) * kSegment;
+            const int64_t off = static_cast<int64_t>(t0) * N;
+            backward_window<S, V, kSegment, false>(x + off, g + off, gx + off, T - t0, N, col, uc, sc,
+                                                   gu, alpha, thresh, beta, interval);
+        }
+        for (int seg = nseg - 2; seg >= 0; --seg) {
 #pragma unroll
             for (int j = 0; j < V; ++j) {
-                uc[j] = C(0);
-                sc[j] = C(0);
+                uc[j] = seg == 0 ? C(0)
+                                 : boundary[(static_cast<int64_t>(seg) * kBwdBlock + threadIdx.x) * V + j];
+                sc[j] = (seg != 0 && uc[j] > thresh) ? C(1) : C(0);
             }
-#pragma unroll
-            for (int t = 0; t < TW; ++t) {
-#pragma unroll
-                for (int j = 0; j < V; ++j) {
-                    lif_step<C>(uc[j], sc[j], Arith<S>::load(xin[t].e[j]), alpha, thresh);
-                    u[t][j] = uc[j];
-                }
-            }
-        }
-
-        C gu[V];
-#pragma unroll
-        for (int j = 0; j < V; ++j) gu[j] = C(0);
-
-#pragma unroll
-        for (int q = 0; q < NG; ++q) {
-            const int hi = TW - q * GC;
-            const int lo = (hi - GC) > 0 ? (hi - GC) : 0;
-            if (q + 1 < NG) {
-                const int nhi = lo;
-                const int nlo = (nhi - GC) > 0 ? (nhi - GC) : 0;
-#pragma unroll
-                for (int t = nhi - 1; t >= nlo; --t) {
-                    if (EXACT) {
-                        gbuf[(q + 1) & 1][t - nlo] =
-                            load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
-                    } else {
-                        gbuf[(q + 1) & 1][t - nlo] = zero_pack<S, V>();
-                        if (t < T)
-                            gbuf[(q + 1) & 1][t - nlo] =
-                                load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
-                    }
-                }
-            }
-#pragma unroll
-            for (int t = hi - 1; t >= lo; --t) {
-                if (EXACT || t < T) {
-                    Pack<S, V> out;
-#pragma unroll
-                    for (int j = 0; j < V; ++j) {
-                        lif_reverse_step<C>(gu[j], u[t][j],
-                                            Arith<S>::load(gbuf[q & 1][t - lo].e[j]), alpha, thresh,
-                                            beta, interval);
-                        out.e[j] = Arith<S>::store(gu[j]);
-                    }
-                    store_pack<S, V>(gx + static_cast<int64_t>(t) * N + col, out);
-                }
-            }
+            const int64_t off = static_cast<int64_t>(seg) * kSegment * N;
+            backward_window<S, V, kSegment, true>(x + off, g + off, gx + off, kSegment, N, col, uc, sc,
+                                                  gu, alpha, thresh, beta, interval);
         }
     }
 }
@@ -632,7 +749,26 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
 #undef SNNLIF_BWD_WINDOW
     static_assert(SNNLIF_BP_FUSED_MAX_T == 32, "windows above must cover the fused range");
 
-    // Long window: u -> workspace (arithmetic type), then the streaming reverse sweep.
+    // Longer windows, up to what the boundary values of a workgroup fit into 64 KiB of LDS for
+    // every storage type: segmented kernel, still no scratch memory in HBM.
+    if (T <= SNNLIF_BP_NO_WORKSPACE_MAX_T) {
+        constexpr int maxv = fused_max_vec<S, kSegment>();
+        const void* ptrs[3] = {x, g, gx};
+        const size_t elem[3] = {sizeof(S), sizeof(S), sizeof(S)};
+        const int v = pick_vec(maxv, N, ptrs, elem, 3);
+        return with_vec<maxv>(v, [&](auto vc) {
+            constexpr int V = decltype(vc)::value;
+            const int64_t nvec = N / V;
+            const int nseg = static_cast<int>((T + kSegment - 1) / kSegment);
+            const size_t lds = static_cast<size_t>(nseg) * kBwdBlock * V * sizeof(C);
+            hipLaunchKernelGGL((lif_backward_segmented_kernel<S, V>), dim3(grid_for(nvec, kBwdBlock)),
+                               dim3(kBwdBlock), lds, stream, x, g, gx, static_cast<int>(T), N, nvec,
+                               C(alpha), C(thresh), C(beta), C(interval));
+            return launch_status();
+        });
+    }
+
+    // Very long window: u -> workspace (arithmetic type), then the streaming reverse sweep.
     const size_t need = static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(C);
     if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
     if (!aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;

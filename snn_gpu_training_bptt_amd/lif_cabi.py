@@ -14,6 +14,7 @@ LIB_PATH = os.path.join(PKG_DIR, "lib", "libsnnlif_gfx950.so")
 DTYPE_F32, DTYPE_F64, DTYPE_BF16 = 0, 1, 2
 OK, ERR_ARG, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_UNSUPPORTED = 0, -1, -2, -3, -4, -5
 BP_FUSED_MAX_T = 32
+BP_NO_WORKSPACE_MAX_T = 1024
 
 # name -> (restype, argtypes); must list every symbol include/snnlib_lif.h declares.
 _vp, _i64, _f32, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_size_t

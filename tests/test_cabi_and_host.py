@@ -46,6 +46,7 @@ def test_constants_match_the_header():
     assert int(macros["SNNLIF_ERR_WORKSPACE"]) == lif_cabi.ERR_WORKSPACE
     assert int(macros["SNNLIF_ERR_ALIGN"]) == lif_cabi.ERR_ALIGN
     assert int(macros["SNNLIF_BP_FUSED_MAX_T"]) == lif_cabi.BP_FUSED_MAX_T
+    assert int(macros["SNNLIF_BP_NO_WORKSPACE_MAX_T"]) == lif_cabi.BP_NO_WORKSPACE_MAX_T
     lib = lif_cabi.load()
     assert lib.snnlif_abi_version() == int(macros["SNNLIF_ABI_VERSION"])
     assert lib.snnlif_target_arch() == b"gfx950"
@@ -57,10 +58,12 @@ def test_host_side_queries_need_no_gpu():
     f32, f64, bf16 = lif_cabi.DTYPE_F32, lif_cabi.DTYPE_F64, lif_cabi.DTYPE_BF16
     assert lif_cabi.fire_bp_workspace_bytes(f32, 8, 1 << 23) == 0
     assert lif_cabi.fire_bp_workspace_bytes(f32, 32, 100) == 0
-    assert lif_cabi.fire_bp_workspace_bytes(f32, 33, 100) == 33 * 100 * 4
-    assert lif_cabi.fire_bp_workspace_bytes(f64, 40, 10) == 40 * 10 * 8
-    assert lif_cabi.fire_bp_workspace_bytes(bf16, 40, 10) == 40 * 10 * 4   # fp32 arithmetic
-    assert lif_cabi.fire_bp_workspace_bytes(7, 40, 10) == 0
+    assert lif_cabi.fire_bp_workspace_bytes(f32, 33, 100) == 0            # segmented on chip
+    assert lif_cabi.fire_bp_workspace_bytes(f32, 1024, 100) == 0
+    assert lif_cabi.fire_bp_workspace_bytes(f32, 1025, 100) == 1025 * 100 * 4
+    assert lif_cabi.fire_bp_workspace_bytes(f64, 2000, 10) == 2000 * 10 * 8
+    assert lif_cabi.fire_bp_workspace_bytes(bf16, 2000, 10) == 2000 * 10 * 4   # fp32 arithmetic
+    assert lif_cabi.fire_bp_workspace_bytes(7, 2000, 10) == 0
     assert lif_cabi.fire_bp_workspace_bytes(f32, -1, 10) == 0
     for code in (0, -1, -2, -3, -4, -99):
         assert lif_cabi.strerror(code)

@@ -80,8 +80,12 @@ CASES = [
     ((16, 2, 32, 8, 8), 0.5, 1.0),      # T=16
     ((32, 2, 16, 16, 16), 0.3, 0.8),    # T=32 (configuration 3's window)
     ((29, 2, 300), 0.3, 0.8),           # T=29 inside the T<=32 window
-    ((33, 2, 16, 8, 8), 0.3, 0.8),      # first T on the workspace path
-    ((70, 3, 129), 0.3, 0.8),           # long window, odd N
+    ((33, 2, 16, 8, 8), 0.3, 0.8),      # first T beyond one register window: two segments
+    ((70, 3, 129), 0.3, 0.8),           # three segments, the last partial, odd N
+    ((64, 2, 500), 0.3, 0.8),           # exactly two full segments
+    ((257, 2, 130), 0.2, 0.7),          # nine segments
+    ((1024, 1, 192), 0.2, 0.7),         # the longest window kept on chip
+    ((1030, 1, 64), 0.2, 0.7),          # beyond it: membrane potential staged in the workspace
 ]
 
 
@@ -94,7 +98,7 @@ def test_fp32_parity(cabi, oracle, shape, mean, std):
 @pytest.mark.parametrize("T", list(range(1, 35)))
 def test_fp32_every_window_length(cabi, oracle, T):
     """Each window length up to 32 maps to its own or the next larger register window; 33 and 34
-    take the workspace path.  Full-width lanes (N % 4 == 0) and scalar lanes (odd N)."""
+    are cut into two segments.  Even and odd N."""
     for n_inner in (256, 77):
         x, g = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=1000 + T)
         assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
@@ -113,7 +117,7 @@ def test_fp32_parity_hyperparameters(cabi, oracle, alpha, thresh, beta, interval
                   alpha, thresh, beta, interval)
 
 
-@pytest.mark.parametrize("shape", [(8, 4, 16, 8, 8), (6, 3, 7), (33, 2, 10)])
+@pytest.mark.parametrize("shape", [(8, 4, 16, 8, 8), (6, 3, 7), (33, 2, 10), (100, 2, 33), (1100, 1, 16)])
 def test_fp64_parity(cabi, oracle, shape):
     x, g = make_inputs(shape, 0.5, 1.0, seed=99, dtype=torch.float64)
     assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
@@ -136,8 +140,8 @@ def test_argument_errors(cabi):
     assert lib.snnlif_fire_s_fp(x.data_ptr(), x.data_ptr(), 9, 4, 8, ALPHA, THRESH, None) == cabi.ERR_DTYPE
     assert lib.snnlif_fire_s_fp(x.data_ptr(), x.data_ptr(), 0, -1, 8, ALPHA, THRESH, None) == cabi.ERR_ARG
     assert lib.snnlif_fire_s_fp(x.data_ptr() + 2, x.data_ptr(), 0, 2, 4, ALPHA, THRESH, None) == cabi.ERR_ALIGN
-    big = torch.zeros(40, 8, device="cuda")
-    rc = lib.snnlif_fire_bp(big.data_ptr(), big.data_ptr(), big.data_ptr(), 0, 40, 8,
+    big = torch.zeros(1100, 8, device="cuda")
+    rc = lib.snnlif_fire_bp(big.data_ptr(), big.data_ptr(), big.data_ptr(), 0, 1100, 8,
                             ALPHA, THRESH, BETA, INTERVAL, None, 0, None)
     assert rc == cabi.ERR_WORKSPACE
     torch.cuda.synchronize()
@@ -189,7 +193,8 @@ def test_special_values_follow_ieee_like_the_oracle(cabi, oracle):
     assert (np.abs(mem_o[:, 0, 300:364]) < 1.2e-38).all() and (mem_o[:, 0, 300:364] != 0).any()
 
 
-@pytest.mark.parametrize("shape", [(8, 3, 255), (5, 1, 1), (16, 2, 4097), (33, 3, 77), (12, 4, 64, 4, 4)])
+@pytest.mark.parametrize("shape", [(8, 3, 255), (5, 1, 1), (16, 2, 4097), (33, 3, 77), (12, 4, 64, 4, 4),
+                                   (1024, 1, 128), (1040, 1, 30)])
 def test_bf16_storage_parity_including_odd_sizes(cabi, oracle, shape):
     """bf16 storage, fp32 arithmetic: two values per lane when N is even and the bases are 4-byte
     aligned, one otherwise.  Expected = the fp32 oracle on the bf16-rounded inputs, outputs rounded

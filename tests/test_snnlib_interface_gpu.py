@@ -106,12 +106,14 @@ def test_strided_input_and_expanded_gradient(mods):
     assert torch.equal(x.grad.cpu(), gx_ref)
 
 
-def test_long_window_uses_workspace_through_module(mods):
+@pytest.mark.parametrize("T", [40, 1100])
+def test_long_windows_through_module(mods, T):
+    """T = 40 is segmented on chip; T = 1100 makes the module allocate the membrane workspace."""
     _, _, gold = mods
     import snnlib
     gen = torch.Generator().manual_seed(14)
-    x_cpu = 0.3 + 0.8 * torch.randn((40, 2, 50), generator=gen)
-    g_cpu = torch.randn((40, 2, 50), generator=gen)
+    x_cpu = 0.3 + 0.8 * torch.randn((T, 2, 50), generator=gen)
+    g_cpu = torch.randn((T, 2, 50), generator=gen)
     _, _, gx_ref = gold.gold_fire_fwd_bwd(x_cpu, g_cpu, 0.25, 0.5, 1.0, 0.5)
     gx = snnlib.fire_bp(x_cpu.cuda(), g_cpu.cuda(), 0.25, 0.5, 1.0, 0.5)
     assert torch.equal(gx.cpu(), gx_ref)
