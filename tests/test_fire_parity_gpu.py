@@ -117,7 +117,7 @@ def test_fp32_parity_hyperparameters(cabi, oracle, alpha, thresh, beta, interval
                   alpha, thresh, beta, interval)
 
 
-@pytest.mark.parametrize("shape", [(8, 4, 16, 8, 8), (6, 3, 7), (33, 2, 10), (100, 2, 33), (1100, 1, 16)])
+@pytest.mark.parametrize("shape", [(8, 4, 16, 8, 8), (6, 3, 7), (33, 2, 10), (100, 2, 33), (1024, 1, 40), (1100, 1, 16)])
 def test_fp64_parity(cabi, oracle, shape):
     x, g = make_inputs(shape, 0.5, 1.0, seed=99, dtype=torch.float64)
     assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
