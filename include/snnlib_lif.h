@@ -70,6 +70,20 @@ const char* snnlif_target_arch(void);
 const char* snnlif_strerror(int code);
 
 /*
+ * Arms kernel-exact timing for the calling thread: the first kernel that the next snnlif_* entry
+ * point called from this thread launches gets the two events (hipEvent_t created with timing enabled,
+ * passed as void*; either may be NULL) attached to its dispatch -- `start_event` completes when that
+ * kernel begins, `stop_event` when it has finished -- so hipEventElapsedTime(start, stop) is the
+ * kernel's own duration, without the dispatch gaps an interval between two hipEventRecord markers
+ * contains.  The arming is consumed by that one launch; passing two NULLs disarms.  Entry points
+ * that launch one kernel (snnlif_fire_s_fp, snnlif_fire_us_fp, snnlif_fire_bp up to
+ * SNNLIF_BP_NO_WORKSPACE_MAX_T, snnlif_bn_fire_s_fp, snnlif_bn_fire_s_recompute) are timed whole; of
+ * the others only the first kernel is.  Not meant for use under HIP graph capture.  No counterpart in
+ * the reference (which has no timing hooks); for benchmarks and profilers built on this ABI.
+ */
+int snnlif_time_next_kernel(void* start_event, void* stop_event);
+
+/*
  * Fire forward: spikes only.
  *   u[t] = (alpha * u[t-1]) * (1 - s[t-1]) + x[t],   s[t] = u[t] > thresh,   u[-1] = s[-1] = 0
  *   spike[t] = s[t] as 0.0 / 1.0 in the storage dtype.

@@ -3,6 +3,10 @@
 #include "lif_bn.h"
 #include "lif_kernels.h"
 
+namespace snnlif {
+thread_local KernelTimer tl_kernel_timer;
+}  // namespace snnlif
+
 namespace {
 
 inline size_t arith_size(int dtype) {
@@ -28,6 +32,12 @@ extern "C" {
 int snnlif_abi_version(void) { return SNNLIF_ABI_VERSION; }
 
 const char* snnlif_target_arch(void) { return "gfx950"; }
+
+int snnlif_time_next_kernel(void* start_event, void* stop_event) {
+    snnlif::tl_kernel_timer.start = static_cast<hipEvent_t>(start_event);
+    snnlif::tl_kernel_timer.stop = static_cast<hipEvent_t>(stop_event);
+    return SNNLIF_OK;
+}
 
 const char* snnlif_strerror(int code) {
     switch (code) {

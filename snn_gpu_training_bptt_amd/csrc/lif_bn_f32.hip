@@ -14,13 +14,13 @@ int bn_forward_launch(const float* x, const float* weight, const float* bias, co
     const int Ti = static_cast<int>(T);
     constexpr int TC = SNNLIF_FWD_ROWS;
     if (T <= 4 && TC > 4) {
-        hipLaunchKernelGGL((lif_bn_forward_kernel<4, false, FROM_IVAR>), grid, block, 0, stream, x,
+        launch_kernel(lif_bn_forward_kernel<4, false, FROM_IVAR>, grid, block, 0, stream, x,
                            weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
     } else if (T <= TC) {
-        hipLaunchKernelGGL((lif_bn_forward_kernel<TC, false, FROM_IVAR>), grid, block, 0, stream, x,
+        launch_kernel(lif_bn_forward_kernel<TC, false, FROM_IVAR>, grid, block, 0, stream, x,
                            weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
     } else {
-        hipLaunchKernelGGL((lif_bn_forward_kernel<TC, true, FROM_IVAR>), grid, block, 0, stream, x,
+        launch_kernel(lif_bn_forward_kernel<TC, true, FROM_IVAR>, grid, block, 0, stream, x,
                            weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, eps, alpha, thresh);
     }
     return launch_status();
@@ -65,7 +65,7 @@ int bn_backward_window(const float* x, const float* weight, const float* bias, c
     const dim3 grid_partial(wave ? grid_for(B * C * G * 64, kBwdBlock) : grid_for(N, kBwdBlock));
     int rc;
 #define SNNLIF_BN_PARTIAL(EXACT_, WAVE_)                                                          \
-    hipLaunchKernelGGL((lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_>), grid_partial, block, 0, stream, \
+    launch_kernel(lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_>, grid_partial, block, 0, stream, \
                        x, g, weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha,     \
                        thresh, beta, interval)
     if (exact) {
@@ -79,18 +79,18 @@ int bn_backward_window(const float* x, const float* weight, const float* bias, c
 
     const float count = static_cast<float>(T * B * HW);
     if (wave) {
-        hipLaunchKernelGGL(bn_channel_reduce_finalize_kernel, dim3(static_cast<unsigned>(C)),
+        launch_kernel(bn_channel_reduce_finalize_kernel, dim3(static_cast<unsigned>(C)),
                            dim3(kReduceBlock), 0, stream, part_gy, part_gyx, weight, grad_weight,
                            grad_bias, coef, B, C, G, count);
         rc = launch_status();
         if (rc != SNNLIF_OK) return rc;
     } else {
         const int64_t bs = (B + S - 1) / S;
-        hipLaunchKernelGGL(bn_channel_reduce_kernel, dim3(static_cast<unsigned>(C), S),
+        launch_kernel(bn_channel_reduce_kernel, dim3(static_cast<unsigned>(C), S),
                            dim3(kReduceBlock), 0, stream, part_gy, part_gyx, split, B, C, HW, bs, S);
         rc = launch_status();
         if (rc != SNNLIF_OK) return rc;
-        hipLaunchKernelGGL(bn_channel_finalize_kernel,
+        launch_kernel(bn_channel_finalize_kernel,
                            dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
                            dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias,
                            coef, C, S, count);
@@ -99,11 +99,11 @@ int bn_backward_window(const float* x, const float* weight, const float* bias, c
     }
 
     if (exact) {
-        hipLaunchKernelGGL((lif_bn_backward_input_kernel<TW, true>), grid, block, 0, stream, x, g,
+        launch_kernel(lif_bn_backward_input_kernel<TW, true>, grid, block, 0, stream, x, g,
                            weight, bias, ivar, mean, coef, gx, Ti, N, C, HW, alpha, thresh, beta,
                            interval);
     } else if constexpr (can_be_inexact) {
-        hipLaunchKernelGGL((lif_bn_backward_input_kernel<TW, false>), grid, block, 0, stream, x, g,
+        launch_kernel(lif_bn_backward_input_kernel<TW, false>, grid, block, 0, stream, x, g,
                            weight, bias, ivar, mean, coef, gx, Ti, N, C, HW, alpha, thresh, beta,
                            interval);
     }

@@ -49,6 +49,7 @@
 #define SNNLIF_LIF_KERNELS_H
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstddef>
 #include <cstdint>
@@ -563,6 +564,28 @@ lif_backward_stream_kernel(const typename Arith<S>::type* __restrict__ mem,
 // Host side: vector-width selection and launches.
 // ---------------------------------------------------------------------------------------------
 
+// Events a caller armed with snnlif_time_next_kernel() for this thread: the next kernel launched
+// from this thread gets them attached to its dispatch (start = the kernel begins, stop = it has
+// finished), which times the kernel itself rather than the interval between two stream markers.
+struct KernelTimer {
+    hipEvent_t start = nullptr;
+    hipEvent_t stop = nullptr;
+};
+extern thread_local KernelTimer tl_kernel_timer;  // defined in lif_abi.hip
+
+template <typename Kernel, typename... Args>
+inline void launch_kernel(Kernel kernel, dim3 grid, dim3 block, size_t lds_bytes,
+                          hipStream_t stream, Args... args) {
+    KernelTimer timer = tl_kernel_timer;
+    if (timer.start != nullptr || timer.stop != nullptr) {
+        tl_kernel_timer = KernelTimer{};
+        hipExtLaunchKernelGGL(kernel, grid, block, static_cast<uint32_t>(lds_bytes), stream,
+                              timer.start, timer.stop, 0, args...);
+    } else {
+        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args...);
+    }
+}
+
 // Upper bound on blocks per launch; beyond it lanes take further columns in the grid-stride loop.
 constexpr int64_t kMaxGrid = int64_t(1) << 24;
 
@@ -618,13 +641,13 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
     const int Ti = static_cast<int>(T);
     constexpr int TC = SNNLIF_FWD_ROWS;
     if (T <= 4 && TC > 4) {
-        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, 4, false, WRITE_U, WRITE_S>), grid,
+        launch_kernel(lif_forward_kernel<S, M, V, 4, false, WRITE_U, WRITE_S>, grid,
                            block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
     } else if (T <= TC) {
-        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, TC, false, WRITE_U, WRITE_S>), grid,
+        launch_kernel(lif_forward_kernel<S, M, V, TC, false, WRITE_U, WRITE_S>, grid,
                            block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
     } else {
-        hipLaunchKernelGGL((lif_forward_kernel<S, M, V, TC, true, WRITE_U, WRITE_S>), grid,
+        launch_kernel(lif_forward_kernel<S, M, V, TC, true, WRITE_U, WRITE_S>, grid,
                            block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
     }
     return launch_status();
@@ -693,10 +716,10 @@ int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, f
         const dim3 grid(grid_for(nvec, kBwdBlock)), block(kBwdBlock);
         const int Ti = static_cast<int>(T);
         if (exact) {
-            hipLaunchKernelGGL((lif_backward_fused_kernel<S, V, TW, true>), grid, block, 0, stream,
+            launch_kernel(lif_backward_fused_kernel<S, V, TW, true>, grid, block, 0, stream,
                                x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval));
         } else if constexpr (can_be_inexact) {
-            hipLaunchKernelGGL((lif_backward_fused_kernel<S, V, TW, false>), grid, block, 0, stream,
+            launch_kernel(lif_backward_fused_kernel<S, V, TW, false>, grid, block, 0, stream,
                                x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval));
         }
         return launch_status();
@@ -709,7 +732,7 @@ int launch_backward_stream_v(const typename Arith<S>::type* mem, const S* g, S* 
                              hipStream_t stream) {
     using C = typename Arith<S>::type;
     const int64_t nvec = N / V;
-    hipLaunchKernelGGL((lif_backward_stream_kernel<S, V, 8>), dim3(grid_for(nvec, kBwdBlock)),
+    launch_kernel(lif_backward_stream_kernel<S, V, 8>, dim3(grid_for(nvec, kBwdBlock)),
                        dim3(kBwdBlock), 0, stream, mem, g, gx, static_cast<int>(T), N, nvec,
                        C(alpha), C(thresh), C(beta), C(interval));
     return launch_status();
@@ -761,7 +784,7 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
             const int64_t nvec = N / V;
             const int nseg = static_cast<int>((T + kSegment - 1) / kSegment);
             const size_t lds = static_cast<size_t>(nseg) * kBwdBlock * V * sizeof(C);
-            hipLaunchKernelGGL((lif_backward_segmented_kernel<S, V>), dim3(grid_for(nvec, kBwdBlock)),
+            launch_kernel(lif_backward_segmented_kernel<S, V>, dim3(grid_for(nvec, kBwdBlock)),
                                dim3(kBwdBlock), lds, stream, x, g, gx, static_cast<int>(T), N, nvec,
                                C(alpha), C(thresh), C(beta), C(interval));
             return launch_status();

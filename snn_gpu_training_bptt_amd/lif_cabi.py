@@ -22,6 +22,7 @@ SYMBOLS = {
     "snnlif_abi_version": (_int, []),
     "snnlif_target_arch": (ctypes.c_char_p, []),
     "snnlif_strerror": (ctypes.c_char_p, [_int]),
+    "snnlif_time_next_kernel": (_int, [_vp, _vp]),
     "snnlif_fire_s_fp": (_int, [_vp, _vp, _int, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_fire_us_fp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64]),
@@ -96,6 +97,15 @@ def _require_dense_gpu(*tensors):
             raise ValueError("device tensor required")
         if not t.is_contiguous():
             raise ValueError("dense (contiguous) tensor required")
+
+
+def time_next_kernel(start_event, stop_event):
+    """Attach two ``torch.cuda.Event(enable_timing=True)`` objects to the next kernel this thread
+    launches through the library (see ``snnlif_time_next_kernel``).  The events must already exist
+    on the device side, i.e. have been recorded at least once; ``None`` stands for no event."""
+    handle = lambda e: ctypes.c_void_p(None if e is None else e.cuda_event)
+    _check(load().snnlif_time_next_kernel(handle(start_event), handle(stop_event)),
+           "snnlif_time_next_kernel")
 
 
 def fire_s_fp_into(spatial, spike, alpha, thresh):

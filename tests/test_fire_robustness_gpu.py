@@ -120,3 +120,43 @@ def test_two_streams_concurrently(cabi):
         gx_o = c_oracle.fire_backward(x_cpu.numpy(), g_cpu.numpy(), ALPHA, THRESH, BETA, INTERVAL)
         assert np.array_equal(spike.cpu().numpy(), spike_o)
         assert np.array_equal(gx.cpu().numpy(), gx_o)
+
+
+def test_events_attached_to_the_next_kernel(cabi):
+    """snnlif_time_next_kernel: the armed events bracket exactly one launch, results are unchanged,
+    the arming is consumed, and the duration is no longer than the interval between two stream
+    markers around the same launch."""
+    from oracle import c_oracle
+    shape = (8, 16, 64, 32, 32)
+    gen = torch.Generator().manual_seed(83)
+    x_cpu = 0.5 + torch.randn(shape, generator=gen)
+    g_cpu = torch.randn(shape, generator=gen)
+    x, g = x_cpu.cuda(), g_cpu.cuda()
+    spike, gx = torch.empty_like(x), torch.empty_like(x)
+    for _ in range(3):
+        cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+    k0, k1, m0, m1, late = (torch.cuda.Event(enable_timing=True) for _ in range(5))
+    for e in (k0, k1, late):
+        e.record()
+    torch.cuda.synchronize()
+    gx.zero_()
+    m0.record()
+    cabi.time_next_kernel(k0, k1)
+    cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+    m1.record()
+    # not armed any more: this launch must leave k0 / k1 alone
+    cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+    late.record()
+    torch.cuda.synchronize()
+    kernel_ms, marker_ms = k0.elapsed_time(k1), m0.elapsed_time(m1)
+    assert 0.0 < kernel_ms <= marker_ms * 1.02, (kernel_ms, marker_ms)
+    assert k1.elapsed_time(late) > 0.0
+    gx_o = c_oracle.fire_backward(x_cpu.numpy(), g_cpu.numpy(), ALPHA, THRESH, BETA, INTERVAL)
+    _, spike_o = c_oracle.fire_forward(x_cpu.numpy(), ALPHA, THRESH)
+    assert np.array_equal(gx.cpu().numpy(), gx_o)
+    assert np.array_equal(spike.cpu().numpy(), spike_o)
+    # disarming with two NULLs is accepted
+    cabi.time_next_kernel(None, None)
+    cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+    torch.cuda.synchronize()
+    assert np.array_equal(spike.cpu().numpy(), spike_o)
