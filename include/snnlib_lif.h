@@ -174,6 +174,39 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
                       int64_t HW, float alpha, float thresh, float beta, float interval,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * The same backward in the two halves that a batch sharded over several GPUs runs on either side of
+ * an all-reduce (fp32 only, T <= SNNLIF_BP_FUSED_MAX_T, shapes and workspace as snnlif_bn_fire_bp;
+ * B is the local batch).
+ *
+ * snnlif_bn_fire_bp_dist1: the local parameter gradients and the local per-channel means
+ *   mean_gxhat[c]  = weight[c] * (sum gy)      / (T*B*HW)
+ *   mean_gxhatx[c] = weight[c] * (sum gy*xhat) / (T*B*HW)
+ * Replaces bn_fire_bp_cuda_dist1 (snnlib/cuda/snn_kernel_bp.cu:753-809), bound as
+ * snnlib.bn_fire_bp_dist1 (snnlib/cuda/snn.cpp:826) and run inside bn_fire_fc_bp_cuda_dist1 (:966-1061)
+ * and bn_fire_conv_bp_cuda_dist1 (:1265-1340).
+ *
+ * snnlif_bn_fire_bp_dist2: the input gradient from the two means averaged over all ranks,
+ *   grad_spatial = (gy*weight[c])*ivar[c] - ivar[c]*((xhat*grad_xhatx[c]) + grad_xhat[c])
+ * Needs no workspace.  Replaces bn_fire_bp_cuda_dist2 (snnlib/cuda/snn_kernel_bp.cu:811-854), bound
+ * as snnlib.bn_fire_bp_dist2 (snnlib/cuda/snn.cpp:827).
+ *
+ * dist1 followed by dist2 on the same arrays is snnlif_bn_fire_bp, bit for bit.  The all-reduce
+ * between them is the caller's.
+ */
+int snnlif_bn_fire_bp_dist1(const void* spatial, const void* weight, const void* bias,
+                            const void* ivar, const void* mean, const void* grad_spike,
+                            void* mean_gxhat, void* mean_gxhatx, void* grad_weight, void* grad_bias,
+                            int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
+                            float thresh, float beta, float interval, void* workspace,
+                            size_t workspace_bytes, void* stream);
+
+int snnlif_bn_fire_bp_dist2(const void* spatial, const void* weight, const void* bias,
+                            const void* ivar, const void* mean, const void* grad_spike,
+                            const void* grad_xhat, const void* grad_xhatx, void* grad_spatial,
+                            int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
+                            float thresh, float beta, float interval, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

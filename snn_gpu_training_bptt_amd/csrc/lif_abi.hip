@@ -191,4 +191,63 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
         static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
 }
 
+int snnlif_bn_fire_bp_dist1(const void* spatial, const void* weight, const void* bias,
+                            const void* ivar, const void* mean, const void* grad_spike,
+                            void* mean_gxhat, void* mean_gxhatx, void* grad_weight, void* grad_bias,
+                            int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
+                            float thresh, float beta, float interval, void* workspace,
+                            size_t workspace_bytes, void* stream) {
+    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
+    if (dtype != SNNLIF_DTYPE_F32) return SNNLIF_ERR_UNSUPPORTED;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    // an empty batch has no statistics to report: the channel arrays are left untouched
+    if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
+    if (T > SNNLIF_BP_FUSED_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
+    if (!spatial || !weight || !bias || !ivar || !mean || !grad_spike || !mean_gxhat ||
+        !mean_gxhatx || !grad_weight || !grad_bias)
+        return SNNLIF_ERR_ARG;
+    const void* ptrs[10] = {spatial, weight, bias, ivar, mean, grad_spike, mean_gxhat, mean_gxhatx,
+                            grad_weight, grad_bias};
+    for (const void* p : ptrs)
+        if (!snnlif::aligned_to(p, sizeof(float))) return SNNLIF_ERR_ALIGN;
+    const size_t need = snnlif::bn_backward_workspace_floats(B, C, HW) * sizeof(float);
+    if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
+    if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
+    return snnlif::bn_backward_stats_f32(
+        static_cast<const float*>(spatial), static_cast<const float*>(weight),
+        static_cast<const float*>(bias), static_cast<const float*>(ivar),
+        static_cast<const float*>(mean), static_cast<const float*>(grad_spike),
+        static_cast<float*>(grad_weight), static_cast<float*>(grad_bias),
+        static_cast<float*>(mean_gxhat), static_cast<float*>(mean_gxhatx), T, B, C, HW, alpha,
+        thresh, beta, interval, static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
+}
+
+int snnlif_bn_fire_bp_dist2(const void* spatial, const void* weight, const void* bias,
+                            const void* ivar, const void* mean, const void* grad_spike,
+                            const void* grad_xhat, const void* grad_xhatx, void* grad_spatial,
+                            int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
+                            float thresh, float beta, float interval, void* stream) {
+    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
+    if (dtype != SNNLIF_DTYPE_F32) return SNNLIF_ERR_UNSUPPORTED;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
+    if (T > SNNLIF_BP_FUSED_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
+    if (!spatial || !weight || !bias || !ivar || !mean || !grad_spike || !grad_xhat || !grad_xhatx ||
+        !grad_spatial)
+        return SNNLIF_ERR_ARG;
+    const void* ptrs[9] = {spatial, weight, bias, ivar, mean, grad_spike, grad_xhat, grad_xhatx,
+                           grad_spatial};
+    for (const void* p : ptrs)
+        if (!snnlif::aligned_to(p, sizeof(float))) return SNNLIF_ERR_ALIGN;
+    return snnlif::bn_backward_input_f32(
+        static_cast<const float*>(spatial), static_cast<const float*>(weight),
+        static_cast<const float*>(bias), static_cast<const float*>(ivar),
+        static_cast<const float*>(mean), static_cast<const float*>(grad_spike),
+        static_cast<const float*>(grad_xhat), static_cast<const float*>(grad_xhatx),
+        static_cast<float*>(grad_spatial), T, B, C, HW, alpha, thresh, beta, interval,
+        static_cast<hipStream_t>(stream));
+}
+
 }  // extern "C"

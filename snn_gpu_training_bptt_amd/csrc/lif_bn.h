@@ -34,6 +34,21 @@ int bn_forward_f32(const float* x, const float* weight, const float* bias, const
                    int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,
                    hipStream_t stream);
 
+// The backward in its two halves (what a batch sharded over several GPUs runs on either side of the
+// all-reduce of the two per-channel means): sweep 1 + channel reduction, then sweep 2.
+// bn_backward_f32 is the two back to back.
+int bn_backward_stats_f32(const float* x, const float* weight, const float* bias, const float* ivar,
+                          const float* mean, const float* g, float* grad_weight, float* grad_bias,
+                          float* mean_gxhat, float* mean_gxhatx, int64_t T, int64_t B, int64_t C,
+                          int64_t HW, float alpha, float thresh, float beta, float interval,
+                          float* workspace, hipStream_t stream);
+
+int bn_backward_input_f32(const float* x, const float* weight, const float* bias, const float* ivar,
+                          const float* mean, const float* g, const float* mean_gxhat,
+                          const float* mean_gxhatx, float* gx, int64_t T, int64_t B, int64_t C,
+                          int64_t HW, float alpha, float thresh, float beta, float interval,
+                          hipStream_t stream);
+
 int bn_backward_f32(const float* x, const float* weight, const float* bias, const float* ivar,
                     const float* mean, const float* g, float* gx, float* grad_weight,
                     float* grad_bias, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,

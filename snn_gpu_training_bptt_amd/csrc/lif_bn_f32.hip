@@ -41,19 +41,21 @@ int bn_forward_f32(const float* x, const float* weight, const float* bias, const
 
 namespace {
 
+// Sweep 1 + channel reduction for windows of at most TW steps: parameter gradients and the two
+// per-channel means the input-gradient sweep needs.
 template <int TW>
-int bn_backward_window(const float* x, const float* weight, const float* bias, const float* ivar,
-                       const float* mean, const float* g, float* gx, float* grad_weight,
-                       float* grad_bias, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
-                       float thresh, float beta, float interval, float* workspace,
-                       hipStream_t stream) {
+int bn_backward_stats_window(const float* x, const float* weight, const float* bias,
+                             const float* ivar, const float* mean, const float* g,
+                             float* grad_weight, float* grad_bias, float* mean_gxhat,
+                             float* mean_gxhatx, int64_t T, int64_t B, int64_t C, int64_t HW,
+                             float alpha, float thresh, float beta, float interval,
+                             float* workspace, hipStream_t stream) {
     const int64_t N = B * C * HW;
     const int S = bn_reduce_splits(B, C);
     float* part_gy = workspace;
     float* part_gyx = part_gy + N;
     float* split = part_gyx + N;
-    float* coef = split + static_cast<int64_t>(2) * S * C;
-    const dim3 grid(grid_for(N, kBwdBlock)), block(kBwdBlock);
+    const dim3 block(kBwdBlock);
     const int Ti = static_cast<int>(T);
     constexpr bool can_be_inexact = TW > 8;
     const bool exact = !can_be_inexact || (T == TW);
@@ -66,8 +68,8 @@ int bn_backward_window(const float* x, const float* weight, const float* bias, c
     int rc;
 #define SNNLIF_BN_PARTIAL(EXACT_, WAVE_)                                                          \
     launch_kernel(lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_>, grid_partial, block, 0, stream, \
-                       x, g, weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha,     \
-                       thresh, beta, interval)
+                  x, g, weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha, thresh,  \
+                  beta, interval)
     if (exact) {
         if (wave) SNNLIF_BN_PARTIAL(true, true); else SNNLIF_BN_PARTIAL(true, false);
     } else if constexpr (can_be_inexact) {
@@ -80,64 +82,94 @@ int bn_backward_window(const float* x, const float* weight, const float* bias, c
     const float count = static_cast<float>(T * B * HW);
     if (wave) {
         launch_kernel(bn_channel_reduce_finalize_kernel, dim3(static_cast<unsigned>(C)),
-                           dim3(kReduceBlock), 0, stream, part_gy, part_gyx, weight, grad_weight,
-                           grad_bias, coef, B, C, G, count);
-        rc = launch_status();
-        if (rc != SNNLIF_OK) return rc;
-    } else {
-        const int64_t bs = (B + S - 1) / S;
-        launch_kernel(bn_channel_reduce_kernel, dim3(static_cast<unsigned>(C), S),
-                           dim3(kReduceBlock), 0, stream, part_gy, part_gyx, split, B, C, HW, bs, S);
-        rc = launch_status();
-        if (rc != SNNLIF_OK) return rc;
-        launch_kernel(bn_channel_finalize_kernel,
-                           dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
-                           dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias,
-                           coef, C, S, count);
-        rc = launch_status();
-        if (rc != SNNLIF_OK) return rc;
+                      dim3(kReduceBlock), 0, stream, part_gy, part_gyx, weight, grad_weight,
+                      grad_bias, mean_gxhat, mean_gxhatx, B, C, G, count);
+        return launch_status();
     }
+    const int64_t bs = (B + S - 1) / S;
+    launch_kernel(bn_channel_reduce_kernel, dim3(static_cast<unsigned>(C), S), dim3(kReduceBlock),
+                  0, stream, part_gy, part_gyx, split, B, C, HW, bs, S);
+    rc = launch_status();
+    if (rc != SNNLIF_OK) return rc;
+    launch_kernel(bn_channel_finalize_kernel,
+                  dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
+                  dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias, mean_gxhat,
+                  mean_gxhatx, C, S, count);
+    return launch_status();
+}
 
+// Sweep 2 for windows of at most TW steps.
+template <int TW>
+int bn_backward_input_window(const float* x, const float* weight, const float* bias,
+                             const float* ivar, const float* mean, const float* g,
+                             const float* mean_gxhat, const float* mean_gxhatx, float* gx, int64_t T,
+                             int64_t B, int64_t C, int64_t HW, float alpha, float thresh, float beta,
+                             float interval, hipStream_t stream) {
+    const int64_t N = B * C * HW;
+    const dim3 grid(grid_for(N, kBwdBlock)), block(kBwdBlock);
+    const int Ti = static_cast<int>(T);
+    constexpr bool can_be_inexact = TW > 8;
+    const bool exact = !can_be_inexact || (T == TW);
     if (exact) {
-        launch_kernel(lif_bn_backward_input_kernel<TW, true>, grid, block, 0, stream, x, g,
-                           weight, bias, ivar, mean, coef, gx, Ti, N, C, HW, alpha, thresh, beta,
-                           interval);
+        launch_kernel(lif_bn_backward_input_kernel<TW, true>, grid, block, 0, stream, x, g, weight,
+                      bias, ivar, mean, mean_gxhat, mean_gxhatx, gx, Ti, N, C, HW, alpha, thresh,
+                      beta, interval);
     } else if constexpr (can_be_inexact) {
-        launch_kernel(lif_bn_backward_input_kernel<TW, false>, grid, block, 0, stream, x, g,
-                           weight, bias, ivar, mean, coef, gx, Ti, N, C, HW, alpha, thresh, beta,
-                           interval);
+        launch_kernel(lif_bn_backward_input_kernel<TW, false>, grid, block, 0, stream, x, g, weight,
+                      bias, ivar, mean, mean_gxhat, mean_gxhatx, gx, Ti, N, C, HW, alpha, thresh,
+                      beta, interval);
     }
     return launch_status();
 }
 
 }  // namespace
 
+// Window lengths with a kernel instance of their own; any other T <= 32 runs in the next one up.
+#define SNNLIF_BN_WINDOWS(X) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(10) X(12) X(16) X(20) X(24) X(28) X(32)
+
+int bn_backward_stats_f32(const float* x, const float* weight, const float* bias, const float* ivar,
+                          const float* mean, const float* g, float* grad_weight, float* grad_bias,
+                          float* mean_gxhat, float* mean_gxhatx, int64_t T, int64_t B, int64_t C,
+                          int64_t HW, float alpha, float thresh, float beta, float interval,
+                          float* workspace, hipStream_t stream) {
+#define SNNLIF_BN_WINDOW(TW)                                                                      \
+    if (T <= TW)                                                                                  \
+        return bn_backward_stats_window<TW>(x, weight, bias, ivar, mean, g, grad_weight, grad_bias, \
+                                            mean_gxhat, mean_gxhatx, T, B, C, HW, alpha, thresh,   \
+                                            beta, interval, workspace, stream);
+    SNNLIF_BN_WINDOWS(SNNLIF_BN_WINDOW)
+#undef SNNLIF_BN_WINDOW
+    return SNNLIF_ERR_UNSUPPORTED;
+}
+
+int bn_backward_input_f32(const float* x, const float* weight, const float* bias, const float* ivar,
+                          const float* mean, const float* g, const float* mean_gxhat,
+                          const float* mean_gxhatx, float* gx, int64_t T, int64_t B, int64_t C,
+                          int64_t HW, float alpha, float thresh, float beta, float interval,
+                          hipStream_t stream) {
+#define SNNLIF_BN_WINDOW(TW)                                                                      \
+    if (T <= TW)                                                                                  \
+        return bn_backward_input_window<TW>(x, weight, bias, ivar, mean, g, mean_gxhat,           \
+                                            mean_gxhatx, gx, T, B, C, HW, alpha, thresh, beta,    \
+                                            interval, stream);
+    SNNLIF_BN_WINDOWS(SNNLIF_BN_WINDOW)
+#undef SNNLIF_BN_WINDOW
+    return SNNLIF_ERR_UNSUPPORTED;
+}
+
 int bn_backward_f32(const float* x, const float* weight, const float* bias, const float* ivar,
                     const float* mean, const float* g, float* gx, float* grad_weight,
                     float* grad_bias, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
                     float thresh, float beta, float interval, float* workspace,
                     hipStream_t stream) {
-#define SNNLIF_BN_WINDOW(TW)                                                                      \
-    if (T <= TW)                                                                                  \
-        return bn_backward_window<TW>(x, weight, bias, ivar, mean, g, gx, grad_weight, grad_bias, \
-                                      T, B, C, HW, alpha, thresh, beta, interval, workspace, stream);
-    SNNLIF_BN_WINDOW(1)
-    SNNLIF_BN_WINDOW(2)
-    SNNLIF_BN_WINDOW(3)
-    SNNLIF_BN_WINDOW(4)
-    SNNLIF_BN_WINDOW(5)
-    SNNLIF_BN_WINDOW(6)
-    SNNLIF_BN_WINDOW(7)
-    SNNLIF_BN_WINDOW(8)
-    SNNLIF_BN_WINDOW(10)
-    SNNLIF_BN_WINDOW(12)
-    SNNLIF_BN_WINDOW(16)
-    SNNLIF_BN_WINDOW(20)
-    SNNLIF_BN_WINDOW(24)
-    SNNLIF_BN_WINDOW(28)
-    SNNLIF_BN_WINDOW(32)
-#undef SNNLIF_BN_WINDOW
-    return SNNLIF_ERR_UNSUPPORTED;
+    // the two per-channel means live at the end of the workspace between the sweeps
+    float* coef = workspace + bn_backward_workspace_floats(B, C, HW) - 2 * C;
+    const int rc = bn_backward_stats_f32(x, weight, bias, ivar, mean, g, grad_weight, grad_bias,
+                                         coef, coef + C, T, B, C, HW, alpha, thresh, beta, interval,
+                                         workspace, stream);
+    if (rc != SNNLIF_OK) return rc;
+    return bn_backward_input_f32(x, weight, bias, ivar, mean, g, coef, coef + C, gx, T, B, C, HW,
+                                 alpha, thresh, beta, interval, stream);
 }
 
 }  // namespace snnlif

@@ -223,13 +223,15 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
     }
 }
 
-// Sweep 2: input gradient.  coef = {gxhat[C], gxhatx[C]}.
+// Sweep 2: input gradient.  mean_gxhat[C], mean_gxhatx[C]: the per-channel means that sweep 1 and
+// the channel reduction produced (averaged over the ranks first when the batch is sharded).
 template <int TW, bool EXACT>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
 lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restrict__ g,
                              const float* __restrict__ weight, const float* __restrict__ bias,
                              const float* __restrict__ ivar, const float* __restrict__ mean,
-                             const float* __restrict__ coef, float* __restrict__ gx, int T,
+                             const float* __restrict__ mean_gxhat,
+                             const float* __restrict__ mean_gxhatx, float* __restrict__ gx, int T,
                              int64_t N, int64_t C, int64_t HW, float alpha, float thresh, float beta,
                              float interval) {
     const bool small = N <= 0xffffffffll;
@@ -241,7 +243,7 @@ lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restric
         const float m = mean[c], iv = ivar[c], wgt = weight[c];
         const float scale = wgt * iv;
         const float b = bias[c];
-        const float gxhat = coef[c], gxhatx = coef[C + c];
+        const float gxhat = mean_gxhat[c], gxhatx = mean_gxhatx[c];
         bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval,
                                     [&](int t, float gy, float xt) {
                                         Pack<float, 1> out;
@@ -312,8 +314,9 @@ __global__ void __launch_bounds__(kReduceBlock)
 bn_channel_reduce_finalize_kernel(const float* __restrict__ part_gy,
                                   const float* __restrict__ part_gyx,
                                   const float* __restrict__ weight, float* __restrict__ grad_weight,
-                                  float* __restrict__ grad_bias, float* __restrict__ coef,
-                                  int64_t B, int64_t C, int64_t G, float count) {
+                                  float* __restrict__ grad_bias, float* __restrict__ mean_gxhat,
+                                  float* __restrict__ mean_gxhatx, int64_t B, int64_t C, int64_t G,
+                                  float count) {
     const int c = blockIdx.x;
     const int64_t n = B * G;
     float a = 0.f, ax = 0.f;
@@ -342,8 +345,8 @@ bn_channel_reduce_finalize_kernel(const float* __restrict__ part_gy,
         grad_bias[c] = ta;
         grad_weight[c] = tax;
         const float wgt = weight[c];
-        coef[c] = (ta * wgt) / count;
-        coef[C + c] = (tax * wgt) / count;
+        mean_gxhat[c] = (ta * wgt) / count;
+        mean_gxhatx[c] = (tax * wgt) / count;
     }
 }
 
@@ -352,7 +355,8 @@ bn_channel_reduce_finalize_kernel(const float* __restrict__ part_gy,
 __global__ void __launch_bounds__(kReduceBlock)
 bn_channel_finalize_kernel(const float* __restrict__ split, const float* __restrict__ weight,
                            float* __restrict__ grad_weight, float* __restrict__ grad_bias,
-                           float* __restrict__ coef, int64_t C, int S, float count) {
+                           float* __restrict__ mean_gxhat, float* __restrict__ mean_gxhatx,
+                           int64_t C, int S, float count) {
     const int64_t c = static_cast<int64_t>(blockIdx.x) * kReduceBlock + threadIdx.x;
     if (c >= C) return;
     float a = 0.f, ax = 0.f;
@@ -363,8 +367,8 @@ bn_channel_finalize_kernel(const float* __restrict__ split, const float* __restr
     grad_bias[c] = a;
     grad_weight[c] = ax;
     const float wgt = weight[c];
-    coef[c] = (a * wgt) / count;
-    coef[C + c] = (ax * wgt) / count;
+    mean_gxhat[c] = (a * wgt) / count;
+    mean_gxhatx[c] = (ax * wgt) / count;
 }
 
 }  // namespace snnlif

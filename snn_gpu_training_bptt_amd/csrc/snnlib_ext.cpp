@@ -337,6 +337,61 @@ std::vector<Tensor> bn_fire_bp(Tensor spatial, Tensor weight_bn, Tensor bias_bn,
     return {grad_spatial, grad_weight.view_as(weight_bn), grad_bias.view_as(weight_bn)};
 }
 
+// The two halves of bn_fire_bp that a batch sharded over several GPUs runs before and after the
+// all-reduce of the per-channel means (snnlib/cuda/snn_kernel_bp.cu:753-854).
+std::vector<Tensor> bn_fire_bp_dist1(Tensor spatial, Tensor weight_bn, Tensor bias_bn, Tensor ivar,
+                                     Tensor mean, IntList dim_bn, Tensor grad_spike, float alpha,
+                                     float thresh, float beta, float interval) {
+    (void)dim_bn;
+    const char* op = "bn_fire_bp_dist1";
+    const BnOperands o = bn_operands(spatial, weight_bn, bias_bn, ivar, mean, op, "ivar");
+    check_input(grad_spike, op, "grad_spike");
+    check_like(grad_spike, spatial, op, "grad_spike");
+    check_same_shape(spatial, grad_spike, op, "spatial", "grad_spike");
+    const DeviceGuard guard(spatial.device());
+    Tensor g = grad_spike.contiguous();
+    // zeros: an empty local batch contributes nothing to the all-reduce
+    Tensor mean_gxhat = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
+    Tensor mean_gxhatx = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
+    Tensor grad_weight = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
+    Tensor grad_bias = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
+    const size_t ws_bytes =
+        snnlif_bn_fire_bp_workspace_bytes(SNNLIF_DTYPE_F32, o.d.T, o.d.B, o.d.C, o.d.HW);
+    Tensor workspace =
+        torch::empty({static_cast<int64_t>(ws_bytes)}, o.x.options().dtype(at::kByte));
+    check_rc(snnlif_bn_fire_bp_dist1(o.x.data_ptr(), o.weight.data_ptr(), o.bias.data_ptr(),
+                                     o.stat.data_ptr(), o.mean.data_ptr(), g.data_ptr(),
+                                     mean_gxhat.data_ptr(), mean_gxhatx.data_ptr(),
+                                     grad_weight.data_ptr(), grad_bias.data_ptr(), SNNLIF_DTYPE_F32,
+                                     o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh, beta, interval,
+                                     ws_bytes ? workspace.data_ptr() : nullptr, ws_bytes,
+                                     current_stream()),
+             op);
+    return {mean_gxhat, mean_gxhatx, grad_weight.view_as(weight_bn), grad_bias.view_as(weight_bn)};
+}
+
+Tensor bn_fire_bp_dist2(Tensor spatial, Tensor weight_bn, Tensor bias_bn, Tensor ivar, Tensor mean,
+                        Tensor grad_spike, Tensor grad_xhat, Tensor grad_xhatx, float alpha,
+                        float thresh, float beta, float interval) {
+    const char* op = "bn_fire_bp_dist2";
+    const BnOperands o = bn_operands(spatial, weight_bn, bias_bn, ivar, mean, op, "ivar");
+    check_input(grad_spike, op, "grad_spike");
+    check_like(grad_spike, spatial, op, "grad_spike");
+    check_same_shape(spatial, grad_spike, op, "spatial", "grad_spike");
+    Tensor gxhat = channel_param(grad_xhat, o.x, o.d.C, op, "grad_xhat");
+    Tensor gxhatx = channel_param(grad_xhatx, o.x, o.d.C, op, "grad_xhatx");
+    const DeviceGuard guard(spatial.device());
+    Tensor g = grad_spike.contiguous();
+    Tensor grad_spatial = torch::empty_like(o.x, at::MemoryFormat::Contiguous);
+    check_rc(snnlif_bn_fire_bp_dist2(o.x.data_ptr(), o.weight.data_ptr(), o.bias.data_ptr(),
+                                     o.stat.data_ptr(), o.mean.data_ptr(), g.data_ptr(),
+                                     gxhat.data_ptr(), gxhatx.data_ptr(), grad_spatial.data_ptr(),
+                                     SNNLIF_DTYPE_F32, o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh,
+                                     beta, interval, current_stream()),
+             op);
+    return grad_spatial;
+}
+
 // ---- layers without fire (ATen only) ------------------------------------------------------------
 
 std::vector<Tensor> bn_fp(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor var, Tensor mean,
@@ -372,6 +427,59 @@ std::vector<Tensor> bn_bp(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor 
         /*running_mean=*/c10::nullopt, /*running_var=*/c10::nullopt, /*save_mean=*/m,
         /*save_invstd=*/iv, /*train=*/true, /*eps=*/0.0, {true, true, true});
     return {std::get<0>(grads).view(x_bn.sizes()), std::get<1>(grads), std::get<2>(grads)};
+}
+
+// The two halves of bn_bp for a sharded batch (snnlib/cuda/snn_kernel_bp.cu:348-425): local
+// parameter gradients and per-channel means, then the input gradient from the averaged means.
+std::vector<Tensor> bn_bp_dist1(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor ivar,
+                                Tensor mean, IntList dim_bn, Tensor grad_y_bn) {
+    (void)bias_bn;
+    (void)dim_bn;
+    const char* op = "bn_bp_dist1";
+    check_input(x_bn, op, "x_bn");
+    check_like(grad_y_bn, x_bn, op, "grad_y_bn");
+    check_same_shape(x_bn, grad_y_bn, op, "x_bn", "grad_y_bn");
+    const BnDims d = bn_dims_of(x_bn, op);
+    Tensor w = channel_param(weight_bn, x_bn, d.C, op, "weight_bn");
+    Tensor iv = channel_param(ivar, x_bn, d.C, op, "ivar");
+    Tensor m = channel_param(mean, x_bn, d.C, op, "mean");
+    const DeviceGuard guard(x_bn.device());
+    if (x_bn.numel() == 0) {
+        Tensor z = torch::zeros_like(w);
+        return {z, z.clone(), z.clone(), z.clone()};
+    }
+    // one pass: sum gy and sum gy*(x - mean) per channel, and the parameter gradients from them
+    auto sums = at::batch_norm_backward_reduce(fold_time(grad_y_bn.contiguous()),
+                                               fold_time(x_bn.contiguous()), m, iv, w,
+                                               /*input_g=*/true, /*weight_g=*/true, /*bias_g=*/true);
+    const Tensor& grad_weight = std::get<2>(sums);
+    const Tensor& grad_bias = std::get<3>(sums);
+    const double count = static_cast<double>(d.T) * d.B * d.HW;
+    return {(grad_bias * w) / count, (grad_weight * w) / count, grad_weight, grad_bias};
+}
+
+Tensor bn_bp_dist2(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor ivar, Tensor mean,
+                   IntList dim_bn, Tensor grad_y_bn, Tensor grad_xhat, Tensor grad_xhatx) {
+    (void)bias_bn;
+    (void)dim_bn;
+    const char* op = "bn_bp_dist2";
+    check_input(x_bn, op, "x_bn");
+    check_like(grad_y_bn, x_bn, op, "grad_y_bn");
+    check_same_shape(x_bn, grad_y_bn, op, "x_bn", "grad_y_bn");
+    const BnDims d = bn_dims_of(x_bn, op);
+    const DeviceGuard guard(x_bn.device());
+    // per-channel vectors shaped to broadcast over [T, B, C, ...]
+    std::vector<int64_t> shape(static_cast<size_t>(x_bn.dim()), 1);
+    shape[2] = d.C;
+    auto per_channel = [&](const Tensor& p, const char* name) {
+        return channel_param(p, x_bn, d.C, op, name).view(shape);
+    };
+    Tensor w = per_channel(weight_bn, "weight_bn"), iv = per_channel(ivar, "ivar");
+    Tensor m = per_channel(mean, "mean");
+    Tensor gxhat = per_channel(grad_xhat, "grad_xhat"), gxhatx = per_channel(grad_xhatx, "grad_xhatx");
+    // grad_x = gy*w*ivar - ivar*(xhat*grad_xhatx + grad_xhat),  xhat = (x - mean)*ivar
+    Tensor xhat = (x_bn - m) * iv;
+    return (grad_y_bn * w) * iv - iv * (xhat * gxhatx + gxhat);
 }
 
 Tensor fc_fp(Tensor spatial, Tensor weight_fc, Tensor bias_fc) {
@@ -540,6 +648,48 @@ std::vector<Tensor> bn_fire_conv_bp(Tensor spatial, Tensor weight_bn, Tensor bia
     return {bn[0], bn[1], bn[2], dense[1], dense[2]};
 }
 
+// Sharded-batch form of bn_fire_fc_bp / bn_fire_conv_bp: everything up to the all-reduce, with the
+// gradient of the spikes handed back for bn_fire_bp_dist2
+// (snnlib/cuda/snn_kernel_bp.cu:966-1061, 1265-1340).
+std::vector<Tensor> bn_fire_fc_bp_dist1(Tensor spatial, Tensor weight_bn, Tensor bias_bn,
+                                        Tensor ivar, Tensor mean, IntList dim_bn, Tensor grad_fc,
+                                        Tensor weight_fc, Tensor bias_fc, IntList dim_fc, float alpha,
+                                        float thresh, float beta, float interval) {
+    (void)bias_fc;
+    const char* op = "bn_fire_fc_bp_dist1";
+    check_input(spatial, op, "spatial");
+    check_like(weight_fc, spatial, op, "weight_fc");
+    check_like(grad_fc, spatial, op, "grad_fc");
+    check_fc_weight(spatial, weight_fc, op);
+    Tensor spike = bn_fire_spikes_from_ivar(spatial, weight_bn, bias_bn, ivar, mean, alpha, thresh, op);
+    const DeviceGuard guard(spatial.device());
+    auto dense = linear_backward_folded(spike, grad_fc, weight_fc, dim_fc, op);
+    auto bn = bn_fire_bp_dist1(spatial, weight_bn, bias_bn, ivar, mean, dim_bn, dense[0], alpha,
+                               thresh, beta, interval);
+    return {dense[0], bn[0], bn[1], bn[2], bn[3], dense[1], dense[2]};
+}
+
+std::vector<Tensor> bn_fire_conv_bp_dist1(Tensor spatial, Tensor weight_bn, Tensor bias_bn,
+                                          Tensor ivar, Tensor mean, IntList dim_bn, Tensor grad_conv,
+                                          Tensor weight_conv, IntList stride, IntList padding,
+                                          IntList dilation, int64_t groups, bool /*benchmark*/,
+                                          bool /*deterministic*/, bool /*allow_tf32*/,
+                                          IntList dim_conv, float alpha, float thresh, float beta,
+                                          float interval) {
+    const char* op = "bn_fire_conv_bp_dist1";
+    check_input(spatial, op, "spatial");
+    check_image(spatial, op);
+    check_like(weight_conv, spatial, op, "weight_conv");
+    check_like(grad_conv, spatial, op, "grad_conv");
+    Tensor spike = bn_fire_spikes_from_ivar(spatial, weight_bn, bias_bn, ivar, mean, alpha, thresh, op);
+    const DeviceGuard guard(spatial.device());
+    auto dense = conv_backward_folded(spike, grad_conv, weight_conv, stride, padding, dilation,
+                                      groups, dim_conv, op);
+    auto bn = bn_fire_bp_dist1(spatial, weight_bn, bias_bn, ivar, mean, dim_bn, dense[0], alpha,
+                               thresh, beta, interval);
+    return {dense[0], bn[0], bn[1], bn[2], bn[3], dense[1], dense[2]};
+}
+
 }  // namespace
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -572,4 +722,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("bn_fire_conv_bp", &bn_fire_conv_bp, "bn fire conv backward");
     m.def("fire_conv_bp", &fire_conv_bp, "fire conv backward");
     m.def("conv_bp", &conv_bp, "conv backward");
+
+    m.def("bn_bp_dist1", &bn_bp_dist1, "bn backward, sharded batch: before the all-reduce");
+    m.def("bn_bp_dist2", &bn_bp_dist2, "bn backward, sharded batch: after the all-reduce");
+    m.def("bn_fire_bp_dist1", &bn_fire_bp_dist1, "bn fire backward, sharded batch: before the all-reduce");
+    m.def("bn_fire_bp_dist2", &bn_fire_bp_dist2, "bn fire backward, sharded batch: after the all-reduce");
+    m.def("bn_fire_fc_bp_dist1", &bn_fire_fc_bp_dist1, "bn fire fc backward, sharded batch: before the all-reduce");
+    m.def("bn_fire_conv_bp_dist1", &bn_fire_conv_bp_dist1, "bn fire conv backward, sharded batch: before the all-reduce");
 }

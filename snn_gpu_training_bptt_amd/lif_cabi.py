@@ -31,6 +31,8 @@ SYMBOLS = {
     "snnlif_bn_fire_s_recompute": (_int, [_vp] * 6 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_bn_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "snnlif_bn_fire_bp": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
+    "snnlif_bn_fire_bp_dist1": (_int, [_vp] * 10 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
+    "snnlif_bn_fire_bp_dist2": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp]),
 }
 
 _lib = None
@@ -197,3 +199,37 @@ def bn_fire_bp_into(spatial, weight, bias, ivar, mean, grad_spike, grad_spatial,
                                   _stream_handle(spatial))
     _check(rc, "snnlif_bn_fire_bp")
     return grad_spatial, grad_weight, grad_bias
+
+
+def bn_fire_bp_dist1_into(spatial, weight, bias, ivar, mean, grad_spike, mean_gxhat, mean_gxhatx,
+                          grad_weight, grad_bias, alpha, thresh, beta, interval, workspace):
+    """``snnlif_bn_fire_bp_dist1`` on fp32 device tensors: the half of the backward before the
+    all-reduce of a sharded batch."""
+    _require_dense_gpu(spatial, weight, bias, ivar, mean, grad_spike, mean_gxhat, mean_gxhatx,
+                       grad_weight, grad_bias, workspace)
+    T, B, C, HW = _bn_dims(spatial)
+    rc = load().snnlif_bn_fire_bp_dist1(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                        ivar.data_ptr(), mean.data_ptr(), grad_spike.data_ptr(),
+                                        mean_gxhat.data_ptr(), mean_gxhatx.data_ptr(),
+                                        grad_weight.data_ptr(), grad_bias.data_ptr(),
+                                        _torch_dtype_code(spatial), T, B, C, HW, alpha, thresh, beta,
+                                        interval, workspace.data_ptr(),
+                                        workspace.numel() * workspace.element_size(),
+                                        _stream_handle(spatial))
+    _check(rc, "snnlif_bn_fire_bp_dist1")
+    return mean_gxhat, mean_gxhatx, grad_weight, grad_bias
+
+
+def bn_fire_bp_dist2_into(spatial, weight, bias, ivar, mean, grad_spike, grad_xhat, grad_xhatx,
+                          grad_spatial, alpha, thresh, beta, interval):
+    """``snnlif_bn_fire_bp_dist2`` on fp32 device tensors: the half after the all-reduce."""
+    _require_dense_gpu(spatial, weight, bias, ivar, mean, grad_spike, grad_xhat, grad_xhatx,
+                       grad_spatial)
+    T, B, C, HW = _bn_dims(spatial)
+    rc = load().snnlif_bn_fire_bp_dist2(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                        ivar.data_ptr(), mean.data_ptr(), grad_spike.data_ptr(),
+                                        grad_xhat.data_ptr(), grad_xhatx.data_ptr(),
+                                        grad_spatial.data_ptr(), _torch_dtype_code(spatial), T, B, C,
+                                        HW, alpha, thresh, beta, interval, _stream_handle(spatial))
+    _check(rc, "snnlif_bn_fire_bp_dist2")
+    return grad_spatial

@@ -4,8 +4,9 @@ Same surface as the reference's ``snnlib_func.py`` for every single-GPU layer
 (snnlib/example/snnlib_func.py:10-17 module-level settings; ``BnFunc`` :42-59, ``BnFireFunc`` :67-85,
 ``BnFireFcFunc`` :91-110, ``FireFcFunc`` :116-132, ``FcFunc`` :138-154, ``BnFireConvFunc`` :162-191,
 ``FireConvFunc`` :197-223, ``ConvFunc`` :229-253, ``FireFunc`` :22-36, each with its
-``<name>_func = <Class>.apply`` alias).  The multi-GPU ``*Dist`` functions (:261-379) are not
-provided.
+``<name>_func = <Class>.apply`` alias), and for the sharded-batch forms ``BnDistFunc`` :261-288,
+``BnFireFcDistFunc`` :297-327, ``BnFireConvDistFunc`` :336-377, whose backward runs the native op in
+two halves with ``torch.distributed.all_reduce`` of two ``[C]`` vectors between them.
 
 Contract shared by all of them, as in the reference: a forward saves only its *inputs* (plus the
 per-channel inverse standard deviation a batch-norm forward returns) -- never spikes or membrane
@@ -66,8 +67,8 @@ class BnFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_y_bn):
-        x_bn, weight_bn, bias_bn, ivar, mean = ctx.saved_tensors
-        return _pad(snnlib.bn_bp(x_bn, weight_bn, bias_bn, ivar, mean, ctx.dim_bn, grad_y_bn), 7)
+        # saved: x_bn, weight_bn, bias_bn, ivar, mean
+        return _pad(snnlib.bn_bp(*ctx.saved_tensors, ctx.dim_bn, grad_y_bn), 7)
 
 
 class BnFireFunc(torch.autograd.Function):
@@ -82,8 +83,8 @@ class BnFireFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_spike):
-        spatial, weight_bn, bias_bn, ivar, mean = ctx.saved_tensors
-        return _pad(snnlib.bn_fire_bp(spatial, weight_bn, bias_bn, ivar, mean, ctx.dim_bn, grad_spike,
+        # saved: spatial, weight_bn, bias_bn, ivar, mean
+        return _pad(snnlib.bn_fire_bp(*ctx.saved_tensors, ctx.dim_bn, grad_spike,
                                       alpha, thresh, beta, interval), 7)
 
 
@@ -100,11 +101,11 @@ class BnFireFcFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_fc):
-        spatial, weight_bn, bias_bn, ivar, mean, weight_fc, bias_fc = ctx.saved_tensors
-        g_spatial, g_weight_bn, g_bias_bn, g_weight_fc, g_bias_fc = snnlib.bn_fire_fc_bp(
-            spatial, weight_bn, bias_bn, ivar, mean, ctx.dim_bn, grad_fc, weight_fc, bias_fc, _DIM_FC,
-            alpha, thresh, beta, interval)
-        return g_spatial, g_weight_bn, g_bias_bn, None, None, None, None, g_weight_fc, g_bias_fc
+        *bn_saved, weight_fc, bias_fc = ctx.saved_tensors
+        grads = snnlib.bn_fire_fc_bp(*bn_saved, ctx.dim_bn, grad_fc, weight_fc, bias_fc, _DIM_FC,
+                                     alpha, thresh, beta, interval)
+        # spatial and the two batch-norm parameters, then var / mean / dim_bn / eps_bn, then the fc pair
+        return (*grads[:3], None, None, None, None, *grads[3:])
 
 
 class FireFcFunc(torch.autograd.Function):
@@ -117,8 +118,8 @@ class FireFcFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_fc):
-        spatial, weight_fc, bias_fc = ctx.saved_tensors
-        return tuple(snnlib.fire_fc_bp(spatial, grad_fc, weight_fc, bias_fc, _DIM_FC,
+        spatial, *fc_params = ctx.saved_tensors
+        return tuple(snnlib.fire_fc_bp(spatial, grad_fc, *fc_params, _DIM_FC,
                                        alpha, thresh, beta, interval))
 
 
@@ -132,8 +133,8 @@ class FcFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_fc):
-        spatial, weight_fc, bias_fc = ctx.saved_tensors
-        return tuple(snnlib.fc_bp(spatial, grad_fc, weight_fc, bias_fc, _DIM_FC))
+        spatial, *fc_params = ctx.saved_tensors
+        return tuple(snnlib.fc_bp(spatial, grad_fc, *fc_params, _DIM_FC))
 
 
 def _conv_grads(ctx, g_spatial, g_weight, g_bias, leading=()):
@@ -157,11 +158,10 @@ class BnFireConvFunc(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, grad_conv):
-        spatial, weight_bn, bias_bn, ivar, mean, weight_conv, bias_conv = ctx.saved_tensors
+        *bn_saved, weight_conv, _ = ctx.saved_tensors
         g_spatial, g_weight_bn, g_bias_bn, g_weight_conv, g_bias_conv = snnlib.bn_fire_conv_bp(
-            spatial, weight_bn, bias_bn, ivar, mean, _DIM_CONV, grad_conv, weight_conv,
-            ctx.stride, ctx.padding, _DILATION, _GROUPS, conv_benchmark, False, True, _DIM_CONV,
-            alpha, thresh, beta, interval)
+            *bn_saved, _DIM_CONV, grad_conv, weight_conv, ctx.stride, ctx.padding, _DILATION, _GROUPS,
+            conv_benchmark, False, True, _DIM_CONV, alpha, thresh, beta, interval)
         return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv,
                            leading=(g_spatial, g_weight_bn, g_bias_bn, None, None, None))
 
@@ -204,6 +204,79 @@ class ConvFunc(torch.autograd.Function):
         return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv, leading=(g_spatial,))
 
 
+def _mean_over_ranks(local_xhat, local_xhatx, reduce_op):
+    """All-reduce the two per-channel means of a sharded batch and average them.
+    ``reduce_op`` is the reference's triple ``[ReduceOp, process_group, world_size]``."""
+    kinds, group, world_size = reduce_op
+    torch.distributed.all_reduce(local_xhat, kinds.SUM, group)
+    torch.distributed.all_reduce(local_xhatx, kinds.SUM, group)
+    return local_xhat / world_size, local_xhatx / world_size
+
+
+class BnDistFunc(BnFunc):
+    """``BnFunc`` for a batch sharded over the ranks of a process group; one more argument, the
+    ``[ReduceOp, process_group, world_size]`` triple, follows ``BnFunc``'s."""
+
+    @staticmethod
+    def forward(ctx, *args):
+        ctx.reduce_op = args[-1]
+        return BnFunc.forward(ctx, *args[:-1])
+
+    @staticmethod
+    def backward(ctx, grad_y_bn):
+        saved = ctx.saved_tensors          # x_bn, weight_bn, bias_bn, ivar, mean
+        local_xhat, local_xhatx, g_weight_bn, g_bias_bn = snnlib.bn_bp_dist1(
+            *saved, ctx.dim_bn, grad_y_bn)
+        g_x_bn = snnlib.bn_bp_dist2(*saved, ctx.dim_bn, grad_y_bn,
+                                    *_mean_over_ranks(local_xhat, local_xhatx, ctx.reduce_op))
+        return _pad((g_x_bn, g_weight_bn, g_bias_bn), 8)
+
+
+def _sharded_bn_fire_input_grad(ctx, bn_saved, g_spike, local_xhat, local_xhatx):
+    """Second half of a sharded bn + fire backward: average the means, then the input gradient."""
+    g_xhat, g_xhatx = _mean_over_ranks(local_xhat, local_xhatx, ctx.reduce_op)
+    return snnlib.bn_fire_bp_dist2(*bn_saved, g_spike, g_xhat, g_xhatx, alpha, thresh, beta, interval)
+
+
+class BnFireFcDistFunc(BnFireFcFunc):
+    """``BnFireFcFunc`` for a sharded batch (same arguments plus the reduce triple)."""
+
+    @staticmethod
+    def forward(ctx, *args):
+        ctx.reduce_op = args[-1]
+        return BnFireFcFunc.forward(ctx, *args[:-1])
+
+    @staticmethod
+    def backward(ctx, grad_fc):
+        *bn_saved, weight_fc, bias_fc = ctx.saved_tensors
+        g_spike, local_xhat, local_xhatx, *param_grads = snnlib.bn_fire_fc_bp_dist1(
+            *bn_saved, ctx.dim_bn, grad_fc, weight_fc, bias_fc, _DIM_FC, alpha, thresh, beta, interval)
+        g_weight_bn, g_bias_bn, g_weight_fc, g_bias_fc = param_grads
+        g_spatial = _sharded_bn_fire_input_grad(ctx, bn_saved, g_spike, local_xhat, local_xhatx)
+        return (g_spatial, g_weight_bn, g_bias_bn, None, None, None, None, g_weight_fc, g_bias_fc,
+                None)
+
+
+class BnFireConvDistFunc(BnFireConvFunc):
+    """``BnFireConvFunc`` for a sharded batch (same arguments plus the reduce triple)."""
+
+    @staticmethod
+    def forward(ctx, *args):
+        ctx.reduce_op = args[-1]
+        return BnFireConvFunc.forward(ctx, *args[:-1])
+
+    @staticmethod
+    def backward(ctx, grad_conv):
+        *bn_saved, weight_conv, _ = ctx.saved_tensors
+        g_spike, local_xhat, local_xhatx, *param_grads = snnlib.bn_fire_conv_bp_dist1(
+            *bn_saved, _DIM_CONV, grad_conv, weight_conv, ctx.stride, ctx.padding, _DILATION, _GROUPS,
+            conv_benchmark, False, True, _DIM_CONV, alpha, thresh, beta, interval)
+        g_weight_bn, g_bias_bn, g_weight_conv, g_bias_conv = param_grads
+        g_spatial = _sharded_bn_fire_input_grad(ctx, bn_saved, g_spike, local_xhat, local_xhatx)
+        return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv,
+                           leading=(g_spatial, g_weight_bn, g_bias_bn, None, None, None)) + (None,)
+
+
 fire_func = FireFunc.apply
 bn_func = BnFunc.apply
 bn_fire_func = BnFireFunc.apply
@@ -213,3 +286,6 @@ fc_func = FcFunc.apply
 bn_fire_conv_func = BnFireConvFunc.apply
 fire_conv_func = FireConvFunc.apply
 conv_func = ConvFunc.apply
+bn_dist_func = BnDistFunc.apply
+bn_fire_fc_dist_func = BnFireFcDistFunc.apply
+bn_fire_conv_dist_func = BnFireConvDistFunc.apply

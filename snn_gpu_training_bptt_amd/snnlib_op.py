@@ -4,8 +4,10 @@ Class names, constructor arguments, parameter names and initialisation are the r
 (snnlib/example/snnlib_op.py): ``Fire`` :11-16, ``Bn`` :19-50, ``BnFire`` :53-84, ``BnFireFc`` :87-128,
 ``FireFc`` :131-139, ``Fc`` :141-149, ``BnFireConv`` :152-192, ``FireConv`` :195-210, ``Conv`` :214-228.
 Inputs are ``[T, B, C, H, W]`` or ``[T, B, C]`` tensors; each module forwards to the matching
-``snnlib_func.<name>_func``.  The ``*Dist`` modules (:231-405, synchronised batch norm over several
-GPUs) are not provided.
+``snnlib_func.<name>_func``.  ``BnDist`` :231-281, ``BnFireFcDist`` :284-344 and ``BnFireConvDist``
+:347-405 are the same layers for a batch sharded over the ranks of ``torch.distributed``'s default
+process group (one rank per GPU): the batch statistics and, in the backward, two per-channel means
+are all-reduced, so every rank normalises with the statistics of the whole batch.
 
 Batch-norm behaviour shared by the ``Bn*`` modules, as in the reference: ``train_bn`` (not
 ``nn.Module.training``) selects batch statistics (``torch.var_mean(..., unbiased=False)`` over
@@ -48,6 +50,40 @@ class _BatchStatistics(nn.Module):
         self.running_var = nn.Parameter(self.running_var * 0.9 + var * (0.1 * self.factor))
         self.running_mean = nn.Parameter(self.running_mean * 0.9 + mean * 0.1)
         return var, mean
+
+
+class _ShardedBatchStatistics(_BatchStatistics):
+    """Batch statistics of a batch that is sharded over the default process group: each rank
+    contributes E[x] and E[x^2] of its shard (shards of equal size), var = E[x^2] - E[x]^2.
+    Running statistics move with momentum 0.05."""
+
+    def _init_batch_norm(self, channels, dim_bn, eps_bn):
+        super()._init_batch_norm(channels, dim_bn, eps_bn)
+        self.ReduceOp = torch.distributed.ReduceOp
+
+    def _statistics(self, x):
+        if self.factor is None:
+            per_channel = x.numel() / self._bn_channels
+            self.factor = per_channel / (per_channel - 1)
+            self.running_var = nn.Parameter(self.running_var.to(x.device))
+            self.running_mean = nn.Parameter(self.running_mean.to(x.device))
+            self.process_group = torch.distributed.group.WORLD
+            self.world_size = torch.distributed.get_world_size(self.process_group)
+        if not self.train_bn:
+            return self.running_var, self.running_mean
+        first = torch.mean(x, dim=self.dim_bn)
+        second = torch.mean(x ** 2, dim=self.dim_bn)
+        torch.distributed.all_reduce(first, self.ReduceOp.SUM, self.process_group)
+        torch.distributed.all_reduce(second, self.ReduceOp.SUM, self.process_group)
+        mean = first / self.world_size
+        var = second / self.world_size - mean ** 2
+        self.running_var = nn.Parameter(self.running_var * 0.95 + var * (0.05 * self.factor))
+        self.running_mean = nn.Parameter(self.running_mean * 0.95 + mean * 0.05)
+        return var, mean
+
+    def _reduce_op(self):
+        """What the ``*_dist_func`` functions take as their last argument."""
+        return [self.ReduceOp, self.process_group, self.world_size]
 
 
 def _fc_parameters(module, cin, cout, like_linear):
@@ -172,3 +208,46 @@ class Conv(nn.Module):
     def forward(self, x):
         return sf.conv_func(x, self.weight_conv, self.bias_conv, self.stride, self.padding,
                             self.if_bias_conv)
+
+
+class BnDist(_ShardedBatchStatistics):
+    def __init__(self, cin, dim_bn, eps_bn=1e-5):
+        super(BnDist, self).__init__()
+        self.cin = cin
+        self._init_batch_norm(cin, dim_bn, eps_bn)
+
+    def forward(self, x):
+        var, mean = self._statistics(x)
+        return sf.bn_dist_func(x, self.weight_bn, self.bias_bn, var, mean, self.dim_bn, self.eps_bn,
+                               self._reduce_op())
+
+
+class BnFireFcDist(_ShardedBatchStatistics):
+    def __init__(self, cin, cout, dim_bn, eps_bn=1e-5, cin_bn=None):
+        super(BnFireFcDist, self).__init__()
+        self.cin = cin
+        self.cin_bn = cin if cin_bn is None else cin_bn
+        self._init_batch_norm(self.cin_bn, dim_bn, eps_bn)
+        _fc_parameters(self, cin, cout, like_linear=True)
+
+    def forward(self, x):
+        var, mean = self._statistics(x)
+        return sf.bn_fire_fc_dist_func(x, self.weight_bn, self.bias_bn, var, mean, self.dim_bn,
+                                       self.eps_bn, self.weight_fc, self.bias_fc, self._reduce_op())
+
+
+class BnFireConvDist(_ShardedBatchStatistics):
+    def __init__(self, cin, cout, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1), eps_bn=1e-5,
+                 if_bias_conv=True):
+        super(BnFireConvDist, self).__init__()
+        _conv_attributes(self, cin, stride, padding, if_bias_conv)
+        self._init_batch_norm(cin, (0, 1, 3, 4), eps_bn)
+        conv = nn.Conv2d(cin, cout, kernel_size, stride, padding)
+        self.weight_conv = nn.Parameter(conv.weight)
+        self.bias_conv = nn.Parameter(conv.bias)
+
+    def forward(self, x):
+        var, mean = self._statistics(x)
+        return sf.bn_fire_conv_dist_func(x, self.weight_bn, self.bias_bn, var, mean, self.eps_bn,
+                                         self.weight_conv, self.bias_conv, self.stride, self.padding,
+                                         self.if_bias_conv, self._reduce_op())

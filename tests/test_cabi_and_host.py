@@ -104,6 +104,17 @@ def test_python_interface_mirrors_the_reference():
     assert (sf.alpha, sf.beta, sf.interval, sf.thresh, sf.time_step) == (0.25, 1.0, 0.5, 0.25, 6)
     assert issubclass(sf.FireFunc, torch.autograd.Function)
     assert sf.fire_func == sf.FireFunc.apply
+    # every layer and autograd function of the reference's two files, the sharded-batch ones included
+    for name in ("Fire", "Bn", "BnFire", "BnFireFc", "FireFc", "Fc", "BnFireConv", "FireConv", "Conv",
+                 "BnDist", "BnFireFcDist", "BnFireConvDist"):
+        assert issubclass(getattr(sop, name), torch.nn.Module), name
+    for name in ("fire", "bn", "bn_fire", "bn_fire_fc", "fire_fc", "fc", "bn_fire_conv", "fire_conv", "conv",
+                 "bn_dist", "bn_fire_fc_dist", "bn_fire_conv_dist"):
+        cls = getattr(sf, "".join(w.capitalize() for w in name.split("_")) + "Func")
+        assert issubclass(cls, torch.autograd.Function) and callable(getattr(sf, name + "_func")), name
+    for name in ("bn_bp_dist1", "bn_bp_dist2", "bn_fire_bp_dist1", "bn_fire_bp_dist2",
+                 "bn_fire_fc_bp_dist1", "bn_fire_conv_bp_dist1"):     # snnlib/cuda/snn.cpp:824-829
+        assert callable(getattr(sf.snnlib, name)), name
     fire = sop.Fire()
     assert isinstance(fire, torch.nn.Module)
     assert list(fire.parameters()) == [] and list(fire.buffers()) == []
