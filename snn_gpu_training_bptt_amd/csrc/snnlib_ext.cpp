@@ -1,8 +1,8 @@
 // Python extension module `snnlib` for PyTorch-ROCm: the operator boundary the autograd functions
 // of snnlib_func.py call (reference: snnlib/example/snnlib_func.py:22-253).
 //
-// Every single-GPU entry of the reference's binding table (snnlib/cuda/snn.cpp:798-822) is provided
-// with the same name and positional signature:
+// Every entry of the reference's binding table (snnlib/cuda/snn.cpp:798-829) is provided with the
+// same name and positional signature:
 //
 //   fire_s_fp(spatial, alpha, thresh) -> spike                                      snn.cpp:11-17
 //   fire_bp(spatial, grad_spike, alpha, thresh, beta, interval) -> grad_spatial     snn.cpp:270-279
@@ -16,8 +16,12 @@
 //   bn_fire_fc_fp / bn_fire_fc_bp, bn_fire_conv_fp / bn_fire_conv_bp                snn.cpp:85-101, 484-506, 162-188, 630-660
 //
 // plus fire_us_fp(spatial, alpha, thresh) -> (mem, spike), the public face of the reference's
-// internal fire_us_fp_kernel (snnlib/cuda/snn_kernel_bp.cu:54-93).  The *_dist1 / *_dist2 halves for
-// multi-GPU synchronised batch norm (snn.cpp:824-829) are not provided.
+// internal fire_us_fp_kernel (snnlib/cuda/snn_kernel_bp.cu:54-93), and the halves that a batch sharded
+// over several GPUs runs on either side of its all-reduce (the all-reduce itself is the caller's):
+//
+//   bn_bp_dist1 / bn_bp_dist2                                                       snn.cpp:317-355
+//   bn_fire_bp_dist1 / bn_fire_bp_dist2                                             snn.cpp:405-460
+//   bn_fire_fc_bp_dist1, bn_fire_conv_bp_dist1                                      snn.cpp:528-550, 687-716
 //
 // Division of labour: the fire recurrences (with or without the batch norm folded in) run on the
 // hand-written kernels behind the C ABI of libsnnlif_gfx950.so (include/snnlib_lif.h); linear,
