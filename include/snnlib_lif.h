@@ -157,7 +157,8 @@ int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const vo
 size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);
 
 /*
- * Batch-norm + fire backward (fp32 only; T <= SNNLIF_BP_FUSED_MAX_T, else SNNLIF_ERR_UNSUPPORTED).
+ * Batch-norm + fire backward (fp32 only; T <= SNNLIF_BP_NO_WORKSPACE_MAX_T, else
+ * SNNLIF_ERR_UNSUPPORTED; windows longer than SNNLIF_BP_FUSED_MAX_T read x twice per sweep).
  * With u recomputed from scale[c] = weight[c]*ivar[c], gy the fire reverse chain (see
  * snnlif_fire_bp), xhat = (x - mean[c])*ivar[c] and M = T*B*HW:
  *   grad_bias[c] = sum gy;   grad_weight[c] = sum gy*xhat
@@ -176,7 +177,7 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
 
 /*
  * The same backward in the two halves that a batch sharded over several GPUs runs on either side of
- * an all-reduce (fp32 only, T <= SNNLIF_BP_FUSED_MAX_T, shapes and workspace as snnlif_bn_fire_bp;
+ * an all-reduce (fp32 only, T <= SNNLIF_BP_NO_WORKSPACE_MAX_T, shapes and workspace as snnlif_bn_fire_bp;
  * B is the local batch).
  *
  * snnlif_bn_fire_bp_dist1: the local parameter gradients and the local per-channel means

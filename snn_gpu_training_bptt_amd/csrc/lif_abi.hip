@@ -172,7 +172,7 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
     const int se = bn_shape_error(T, B, C, HW);
     if (se != SNNLIF_OK) return se;
     if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
-    if (T > SNNLIF_BP_FUSED_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
+    if (T > SNNLIF_BP_NO_WORKSPACE_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
     if (!spatial || !weight || !bias || !ivar || !mean || !grad_spike || !grad_spatial ||
         !grad_weight || !grad_bias)
         return SNNLIF_ERR_ARG;
@@ -203,7 +203,7 @@ int snnlif_bn_fire_bp_dist1(const void* spatial, const void* weight, const void*
     if (se != SNNLIF_OK) return se;
     // an empty batch has no statistics to report: the channel arrays are left untouched
     if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
-    if (T > SNNLIF_BP_FUSED_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
+    if (T > SNNLIF_BP_NO_WORKSPACE_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
     if (!spatial || !weight || !bias || !ivar || !mean || !grad_spike || !mean_gxhat ||
         !mean_gxhatx || !grad_weight || !grad_bias)
         return SNNLIF_ERR_ARG;
@@ -233,7 +233,7 @@ int snnlif_bn_fire_bp_dist2(const void* spatial, const void* weight, const void*
     const int se = bn_shape_error(T, B, C, HW);
     if (se != SNNLIF_OK) return se;
     if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
-    if (T > SNNLIF_BP_FUSED_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
+    if (T > SNNLIF_BP_NO_WORKSPACE_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
     if (!spatial || !weight || !bias || !ivar || !mean || !grad_spike || !grad_xhat || !grad_xhatx ||
         !grad_spatial)
         return SNNLIF_ERR_ARG;

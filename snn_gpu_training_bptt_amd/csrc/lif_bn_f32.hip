@@ -41,9 +41,15 @@ int bn_forward_f32(const float* x, const float* weight, const float* bias, const
 
 namespace {
 
-// Sweep 1 + channel reduction for windows of at most TW steps: parameter gradients and the two
+// Dynamic LDS of the segmented sweeps: one boundary value per segment and lane.
+inline size_t bn_segment_lds_bytes(int64_t T) {
+    return static_cast<size_t>((T + kSegment - 1) / kSegment) * kBwdBlock * sizeof(float);
+}
+
+// Sweep 1 + channel reduction for windows of at most TW steps (SEGMENTED: of any length up to
+// SNNLIF_BP_NO_WORKSPACE_MAX_T, in segments of TW = kSegment steps): parameter gradients and the two
 // per-channel means the input-gradient sweep needs.
-template <int TW>
+template <int TW, bool SEGMENTED = false>
 int bn_backward_stats_window(const float* x, const float* weight, const float* bias,
                              const float* ivar, const float* mean, const float* g,
                              float* grad_weight, float* grad_bias, float* mean_gxhat,
@@ -58,7 +64,8 @@ int bn_backward_stats_window(const float* x, const float* weight, const float* b
     const dim3 block(kBwdBlock);
     const int Ti = static_cast<int>(T);
     constexpr bool can_be_inexact = TW > 8;
-    const bool exact = !can_be_inexact || (T == TW);
+    const bool exact = !SEGMENTED && (!can_be_inexact || (T == TW));
+    const size_t lds = SEGMENTED ? bn_segment_lds_bytes(T) : 0;
 
     // Planes with few positions (fully connected shapes) would leave most lanes of a plane-aligned
     // wavefront idle; they keep one lane per neuron and per-neuron partials.
@@ -67,10 +74,12 @@ int bn_backward_stats_window(const float* x, const float* weight, const float* b
     const dim3 grid_partial(wave ? grid_for(B * C * G * 64, kBwdBlock) : grid_for(N, kBwdBlock));
     int rc;
 #define SNNLIF_BN_PARTIAL(EXACT_, WAVE_)                                                          \
-    launch_kernel(lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_>, grid_partial, block, 0, stream, \
-                  x, g, weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW, alpha, thresh,  \
-                  beta, interval)
-    if (exact) {
+    launch_kernel(lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_, SEGMENTED>, grid_partial, block, \
+                  lds, stream, x, g, weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, HW,   \
+                  alpha, thresh, beta, interval)
+    if constexpr (SEGMENTED) {
+        if (wave) SNNLIF_BN_PARTIAL(false, true); else SNNLIF_BN_PARTIAL(false, false);
+    } else if (exact) {
         if (wave) SNNLIF_BN_PARTIAL(true, true); else SNNLIF_BN_PARTIAL(true, false);
     } else if constexpr (can_be_inexact) {
         if (wave) SNNLIF_BN_PARTIAL(false, true); else SNNLIF_BN_PARTIAL(false, false);
@@ -98,8 +107,8 @@ int bn_backward_stats_window(const float* x, const float* weight, const float* b
     return launch_status();
 }
 
-// Sweep 2 for windows of at most TW steps.
-template <int TW>
+// Sweep 2 for windows of at most TW steps (SEGMENTED: as above).
+template <int TW, bool SEGMENTED = false>
 int bn_backward_input_window(const float* x, const float* weight, const float* bias,
                              const float* ivar, const float* mean, const float* g,
                              const float* mean_gxhat, const float* mean_gxhatx, float* gx, int64_t T,
@@ -109,8 +118,12 @@ int bn_backward_input_window(const float* x, const float* weight, const float* b
     const dim3 grid(grid_for(N, kBwdBlock)), block(kBwdBlock);
     const int Ti = static_cast<int>(T);
     constexpr bool can_be_inexact = TW > 8;
-    const bool exact = !can_be_inexact || (T == TW);
-    if (exact) {
+    const bool exact = !SEGMENTED && (!can_be_inexact || (T == TW));
+    if constexpr (SEGMENTED) {
+        launch_kernel(lif_bn_backward_input_kernel<TW, false, true>, grid, block,
+                      bn_segment_lds_bytes(T), stream, x, g, weight, bias, ivar, mean, mean_gxhat,
+                      mean_gxhatx, gx, Ti, N, C, HW, alpha, thresh, beta, interval);
+    } else if (exact) {
         launch_kernel(lif_bn_backward_input_kernel<TW, true>, grid, block, 0, stream, x, g, weight,
                       bias, ivar, mean, mean_gxhat, mean_gxhatx, gx, Ti, N, C, HW, alpha, thresh,
                       beta, interval);
@@ -139,6 +152,11 @@ int bn_backward_stats_f32(const float* x, const float* weight, const float* bias
                                             beta, interval, workspace, stream);
     SNNLIF_BN_WINDOWS(SNNLIF_BN_WINDOW)
 #undef SNNLIF_BN_WINDOW
+    if (T <= SNNLIF_BP_NO_WORKSPACE_MAX_T)
+        return bn_backward_stats_window<kSegment, true>(x, weight, bias, ivar, mean, g, grad_weight,
+                                                        grad_bias, mean_gxhat, mean_gxhatx, T, B, C,
+                                                        HW, alpha, thresh, beta, interval, workspace,
+                                                        stream);
     return SNNLIF_ERR_UNSUPPORTED;
 }
 
@@ -154,6 +172,10 @@ int bn_backward_input_f32(const float* x, const float* weight, const float* bias
                                             interval, stream);
     SNNLIF_BN_WINDOWS(SNNLIF_BN_WINDOW)
 #undef SNNLIF_BN_WINDOW
+    if (T <= SNNLIF_BP_NO_WORKSPACE_MAX_T)
+        return bn_backward_input_window<kSegment, true>(x, weight, bias, ivar, mean, g, mean_gxhat,
+                                                        mean_gxhatx, gx, T, B, C, HW, alpha, thresh,
+                                                        beta, interval, stream);
     return SNNLIF_ERR_UNSUPPORTED;
 }
 

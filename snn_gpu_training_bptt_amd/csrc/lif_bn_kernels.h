@@ -26,7 +26,11 @@
 //      an order fixed by the launch geometry -> bit-reproducible results;
 //   3. lif_bn_backward_input_kernel: the chain again (x and g re-read: 8 B per neuron-step, the
 //      same as storing and re-loading gy would cost) and the input gradient.
-// HBM traffic: forward 8 B, backward 20 B (+ at most 16/T B) per neuron-step; the reference moves 8 and 36.
+// Windows of more than 32 steps (up to 1024) run both sweeps in 32-step segments with the membrane
+// potential at the segment boundaries kept in LDS (bn_reverse_segmented): x is then read twice per
+// sweep.
+// HBM traffic: forward 8 B, backward 20 B (+ at most 16/T B) per neuron-step up to 32 steps, 28 B
+// beyond; the reference moves 8 and 36.
 #ifndef SNNLIF_LIF_BN_KERNELS_H
 #define SNNLIF_LIF_BN_KERNELS_H
 
@@ -110,44 +114,116 @@ lif_bn_forward_kernel(const float* __restrict__ x, const float* __restrict__ wei
 }
 
 // ---------------------------------------------------------------------------------------------
-// Shared front half of both backward sweeps: load the window, recompute u, run the reverse chain.
-// Calls emit(t, gy, x_t) for t = T-1 .. 0.
+// Shared front half of both backward sweeps, for one register window of at most TW steps whose
+// first row the pointers x / g name: load the window, recompute u from the state (uc, sc) carried
+// in from the step before it, run the reverse chain from the gradient gu carried in from the step
+// after it.  Calls emit(t, gy, x_t) for t = rows-1 .. 0 (t counts from the window's first row).  On
+// exit uc / sc are the state after the window and gu the gradient at its first step.
 // ---------------------------------------------------------------------------------------------
+template <int TW, bool EXACT, typename Emit>
+__device__ __forceinline__ void bn_reverse_window(const float* __restrict__ x,
+                                                  const float* __restrict__ g, int rows, int64_t N,
+                                                  int64_t col, float m, float scale, float b,
+                                                  float& uc, float& sc, float& gu, float alpha,
+                                                  float thresh, float beta, float interval,
+                                                  Emit&& emit) {
+    float xin[TW], gin[TW], u[TW];
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+        xin[t] = 0.f;
+        if (EXACT || t < rows)
+            xin[t] = load_pack<float, 1, false>(x + static_cast<int64_t>(t) * N + col).e[0];
+    }
+#pragma unroll
+    for (int t = TW - 1; t >= 0; --t) {
+        gin[t] = 0.f;
+        if (EXACT || t < rows)
+            gin[t] = load_pack<float, 1, true>(g + static_cast<int64_t>(t) * N + col).e[0];
+    }
+#pragma unroll
+    for (int t = 0; t < TW; ++t) {
+        uc = (alpha * uc) * (1.f - sc) + (xin[t] - m) * scale + b;
+        sc = (uc > thresh) ? 1.f : 0.f;
+        u[t] = uc;
+    }
+#pragma unroll
+    for (int t = TW - 1; t >= 0; --t) {
+        if (EXACT || t < rows) {
+            lif_reverse_step<float>(gu, u[t], gin[t], alpha, thresh, beta, interval);
+            emit(t, gu, xin[t]);
+        }
+    }
+}
+
+// The whole time axis as one window (T <= TW).
 template <int TW, bool EXACT, typename Emit>
 __device__ __forceinline__ void bn_reverse_chain(const float* __restrict__ x,
                                                  const float* __restrict__ g, int T, int64_t N,
                                                  int64_t col, float m, float scale, float b,
                                                  float alpha, float thresh, float beta,
                                                  float interval, Emit&& emit) {
-    float xin[TW], gin[TW], u[TW];
+    float uc = 0.f, sc = 0.f, gu = 0.f;
+    bn_reverse_window<TW, EXACT>(x, g, T, N, col, m, scale, b, uc, sc, gu, alpha, thresh, beta,
+                                 interval, emit);
+}
+
+// Time axes longer than one register window, in segments of kSegment steps, the way
+// lif_backward_segmented_kernel does it: forward over all but the last segment keeping the membrane
+// potential at each boundary in this lane's own LDS slots (`boundary`: [segment][kBwdBlock] floats
+// of dynamic LDS), then the segments last to first.  emit gets the absolute time step.
+template <typename Emit>
+__device__ __forceinline__ void bn_reverse_segmented(const float* __restrict__ x,
+                                                     const float* __restrict__ g, int T, int64_t N,
+                                                     int64_t col, float m, float scale, float b,
+                                                     float alpha, float thresh, float beta,
+                                                     float interval, float* boundary, Emit&& emit) {
+    const int nseg = (T + kSegment - 1) / kSegment;
+    constexpr int ROWS = 8;
+    static_assert(kSegment % ROWS == 0, "a segment is a whole number of forward groups");
+    float uc = 0.f, sc = 0.f, gu = 0.f;
+    for (int seg = 0; seg + 1 < nseg; ++seg) {
+        for (int t0 = seg * kSegment; t0 < (seg + 1) * kSegment; t0 += ROWS) {
+            float rows[ROWS];
 #pragma unroll
-    for (int t = 0; t < TW; ++t) {
-        xin[t] = 0.f;
-        if (EXACT || t < T)
-            xin[t] = load_pack<float, 1, false>(x + static_cast<int64_t>(t) * N + col).e[0];
-    }
+            for (int k = 0; k < ROWS; ++k)
+                rows[k] = load_pack<float, 1, false>(x + static_cast<int64_t>(t0 + k) * N + col).e[0];
 #pragma unroll
-    for (int t = TW - 1; t >= 0; --t) {
-        gin[t] = 0.f;
-        if (EXACT || t < T)
-            gin[t] = load_pack<float, 1, true>(g + static_cast<int64_t>(t) * N + col).e[0];
+            for (int k = 0; k < ROWS; ++k) {
+                uc = (alpha * uc) * (1.f - sc) + (rows[k] - m) * scale + b;
+                sc = (uc > thresh) ? 1.f : 0.f;
+            }
+        }
+        boundary[(seg + 1) * kBwdBlock + threadIdx.x] = uc;
     }
     {
-        float uc = 0.f, sc = 0.f;
-#pragma unroll
-        for (int t = 0; t < TW; ++t) {
-            uc = (alpha * uc) * (1.f - sc) + (xin[t] - m) * scale + b;
-            sc = (uc > thresh) ? 1.f : 0.f;
-            u[t] = uc;
-        }
+        const int t0 = (nseg - 1) * kSegment;
+        const int64_t off = static_cast<int64_t>(t0) * N;
+        bn_reverse_window<kSegment, false>(x + off, g + off, T - t0, N, col, m, scale, b, uc, sc, gu,
+                                           alpha, thresh, beta, interval,
+                                           [&](int t, float gy, float xt) { emit(t0 + t, gy, xt); });
     }
-    float gu = 0.f;
-#pragma unroll
-    for (int t = TW - 1; t >= 0; --t) {
-        if (EXACT || t < T) {
-            lif_reverse_step<float>(gu, u[t], gin[t], alpha, thresh, beta, interval);
-            emit(t, gu, xin[t]);
-        }
+    for (int seg = nseg - 2; seg >= 0; --seg) {
+        uc = seg == 0 ? 0.f : boundary[seg * kBwdBlock + threadIdx.x];
+        sc = (seg != 0 && uc > thresh) ? 1.f : 0.f;
+        const int t0 = seg * kSegment;
+        const int64_t off = static_cast<int64_t>(t0) * N;
+        bn_reverse_window<kSegment, true>(x + off, g + off, kSegment, N, col, m, scale, b, uc, sc, gu,
+                                          alpha, thresh, beta, interval,
+                                          [&](int t, float gy, float xt) { emit(t0 + t, gy, xt); });
+    }
+}
+
+// Dispatch between the two: SEGMENTED kernels are instantiated with TW = kSegment.
+template <int TW, bool EXACT, bool SEGMENTED, typename Emit>
+__device__ __forceinline__ void bn_reverse(const float* __restrict__ x, const float* __restrict__ g,
+                                           int T, int64_t N, int64_t col, float m, float scale,
+                                           float b, float alpha, float thresh, float beta,
+                                           float interval, float* boundary, Emit&& emit) {
+    if constexpr (SEGMENTED) {
+        bn_reverse_segmented(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, boundary,
+                             emit);
+    } else {
+        bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, emit);
     }
 }
 
@@ -164,7 +240,7 @@ __device__ __forceinline__ float wave_sum(float v) {
 // wavefronts per plane, the last one partly idle when HW is not a multiple of 64 -- so all lanes of
 // a wavefront share a channel and their sums are folded by shuffles: one pair of floats per
 // wavefront, part_* indexed [plane][chunk] (B*C*G entries).
-template <int TW, bool EXACT, bool WAVE>
+template <int TW, bool EXACT, bool WAVE, bool SEGMENTED = false>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
 lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restrict__ g,
                                const float* __restrict__ weight, const float* __restrict__ bias,
@@ -172,6 +248,8 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
                                float* __restrict__ part_gy, float* __restrict__ part_gyx, int T,
                                int64_t N, int64_t C, int64_t HW, float alpha, float thresh,
                                float beta, float interval) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    float* boundary = reinterpret_cast<float*>(lds_raw);  // used by SEGMENTED only
     const bool small = N <= 0xffffffffll;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
     if (WAVE) {
@@ -189,12 +267,12 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
                 const float m = mean[c], iv = ivar[c];
                 const float scale = weight[c] * iv;
                 const float b = bias[c];
-                bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
-                                            interval, [&](int, float gy, float xt) {
-                                                const float xhat = (xt - m) * iv;
-                                                acc_gy += gy;
-                                                acc_gyx += gy * xhat;
-                                            });
+                bn_reverse<TW, EXACT, SEGMENTED>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
+                                                 interval, boundary, [&](int, float gy, float xt) {
+                                                     const float xhat = (xt - m) * iv;
+                                                     acc_gy += gy;
+                                                     acc_gyx += gy * xhat;
+                                                 });
             }
             acc_gy = wave_sum(acc_gy);
             acc_gyx = wave_sum(acc_gyx);
@@ -211,12 +289,12 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
             const float scale = weight[c] * iv;
             const float b = bias[c];
             float acc_gy = 0.f, acc_gyx = 0.f;
-            bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval,
-                                        [&](int, float gy, float xt) {
-                                            const float xhat = (xt - m) * iv;
-                                            acc_gy += gy;
-                                            acc_gyx += gy * xhat;
-                                        });
+            bn_reverse<TW, EXACT, SEGMENTED>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
+                                             interval, boundary, [&](int, float gy, float xt) {
+                                                 const float xhat = (xt - m) * iv;
+                                                 acc_gy += gy;
+                                                 acc_gyx += gy * xhat;
+                                             });
             part_gy[col] = acc_gy;
             part_gyx[col] = acc_gyx;
         }
@@ -225,7 +303,7 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
 
 // Sweep 2: input gradient.  mean_gxhat[C], mean_gxhatx[C]: the per-channel means that sweep 1 and
 // the channel reduction produced (averaged over the ranks first when the batch is sharded).
-template <int TW, bool EXACT>
+template <int TW, bool EXACT, bool SEGMENTED = false>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
 lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restrict__ g,
                              const float* __restrict__ weight, const float* __restrict__ bias,
@@ -234,6 +312,8 @@ lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restric
                              const float* __restrict__ mean_gxhatx, float* __restrict__ gx, int T,
                              int64_t N, int64_t C, int64_t HW, float alpha, float thresh, float beta,
                              float interval) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    float* boundary = reinterpret_cast<float*>(lds_raw);  // used by SEGMENTED only
     const bool small = N <= 0xffffffffll;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
     for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < N;
@@ -244,12 +324,13 @@ lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restric
         const float scale = wgt * iv;
         const float b = bias[c];
         const float gxhat = mean_gxhat[c], gxhatx = mean_gxhatx[c];
-        bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval,
-                                    [&](int t, float gy, float xt) {
-                                        Pack<float, 1> out;
-                                        out.e[0] = gy * wgt * iv - iv * ((xt - m) * iv * gxhatx + gxhat);
-                                        store_pack<float, 1>(gx + static_cast<int64_t>(t) * N + col, out);
-                                    });
+        bn_reverse<TW, EXACT, SEGMENTED>(
+            x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, boundary,
+            [&](int t, float gy, float xt) {
+                Pack<float, 1> out;
+                out.e[0] = gy * wgt * iv - iv * ((xt - m) * iv * gxhatx + gxhat);
+                store_pack<float, 1>(gx + static_cast<int64_t>(t) * N + col, out);
+            });
     }
 }
 

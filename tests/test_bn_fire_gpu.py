@@ -54,6 +54,11 @@ SHAPES = [
     (5, 2, 9, 31),            # HW = 31: just below it, one lane per neuron
     (13, 3, 20, 5, 3),        # window without an instantiation of its own
     (32, 2, 16, 4, 4),
+    (33, 2, 6, 8, 8),         # first window beyond the registers: two segments, the second of one step
+    (64, 2, 8, 4, 8),         # two full segments, plane-aligned wavefronts
+    (70, 2, 5, 31),           # three segments, one lane per neuron
+    (100, 3, 20),             # fully connected shape, four segments
+    (1024, 1, 4, 6, 6),       # the longest window: 32 segments of LDS boundary values
     (8, 64, 1024),            # fully connected, many channels
     (8, 32, 128, 32, 32),     # few channels, many positions: exercises the split reduction
 ]
@@ -163,9 +168,9 @@ def test_bn_fire_errors(cabi):
     with pytest.raises(RuntimeError, match="per channel"):
         snnlib.bn_fire_s_fp(x, p[:4], p, p, p, EPS, ALPHA, THRESH)
     lib = cabi.load()
-    big = torch.zeros(40, 2, 8, device="cuda")
+    big = torch.zeros(1025, 2, 8, device="cuda")      # longer than the segmented backward reaches
     rc = lib.snnlif_bn_fire_bp(big.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), big.data_ptr(),
-                               big.data_ptr(), p.data_ptr(), p.data_ptr(), 0, 40, 2, 8, 1, ALPHA, THRESH, BETA, INTERVAL,
+                               big.data_ptr(), p.data_ptr(), p.data_ptr(), 0, 1025, 2, 8, 1, ALPHA, THRESH, BETA, INTERVAL,
                                None, 0, None)
     assert rc == cabi.ERR_UNSUPPORTED
     rc = lib.snnlif_bn_fire_bp(x.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), x.data_ptr(),
