@@ -142,6 +142,13 @@ Tensor channel_param(const Tensor& p, const Tensor& like, int64_t C, const char*
     return p.contiguous();
 }
 
+// A freshly computed tensor under another shape, handed out as a tensor of its own rather than as
+// an autograd view: callers modify layer outputs in place (the residual `x += ...` of
+// snnlib/example/models.py:122-125), which autograd forbids on a view made inside a custom Function.
+Tensor reshaped_result(const Tensor& t, at::IntArrayRef sizes) {
+    return at::_unsafe_view(t, sizes);
+}
+
 // [T, B, ...] -> [T*B, ...], [T*B, prod(...)]
 Tensor fold_time(const Tensor& t) {
     IntList sizes = {t.size(0) * t.size(1)};
@@ -156,7 +163,8 @@ Tensor fold_time_flat(const Tensor& t) {
 // ---- dense halves (ATen: rocBLAS / MIOpen), time folded into the batch ---------------------------
 
 Tensor linear_folded(const Tensor& in, const Tensor& weight, const Tensor& bias) {
-    return at::linear(fold_time_flat(in), weight, bias).view({in.size(0), in.size(1), weight.size(0)});
+    return reshaped_result(at::linear(fold_time_flat(in), weight, bias),
+                           {in.size(0), in.size(1), weight.size(0)});
 }
 
 // -> {grad_in (shaped like `in`), grad_weight, grad_bias}
@@ -168,7 +176,7 @@ std::vector<Tensor> linear_backward_folded(const Tensor& in, const Tensor& grad_
                 "snnlib.", op, ": grad_fc must be [T, B, cout] = [", in.size(0), ", ", in.size(1),
                 ", ", weight.size(0), "], got ", grad_fc.sizes());
     Tensor g2 = fold_time_flat(grad_fc.contiguous());  // [T*B, cout]
-    Tensor grad_in = at::mm(g2, weight).view(in.sizes());
+    Tensor grad_in = reshaped_result(at::mm(g2, weight), in.sizes());
     Tensor grad_weight = at::mm(g2.t(), fold_time_flat(in));  // [cout, cin]
     return {grad_in, grad_weight, at::sum(grad_fc, dim_fc)};
 }
@@ -178,7 +186,7 @@ Tensor conv_folded(const Tensor& in, const Tensor& weight, const Tensor& bias,
                    int64_t groups) {
     Tensor conv = at::convolution(fold_time(in), weight, bias, stride, padding, dilation,
                                   /*transposed=*/false, /*output_padding=*/{0, 0}, groups);
-    return conv.view({in.size(0), in.size(1), conv.size(1), conv.size(2), conv.size(3)});
+    return reshaped_result(conv, {in.size(0), in.size(1), conv.size(1), conv.size(2), conv.size(3)});
 }
 
 // -> {grad_in (shaped like `in`), grad_weight, grad_bias}
@@ -194,7 +202,8 @@ std::vector<Tensor> conv_backward_folded(const Tensor& in, const Tensor& grad_co
         fold_time(grad_conv.contiguous()), fold_time(in), weight, /*bias_sizes=*/c10::nullopt,
         stride, padding, dilation, /*transposed=*/false, /*output_padding=*/{0, 0}, groups,
         /*output_mask=*/{true, true, false});
-    return {std::get<0>(grads).view(in.sizes()), std::get<1>(grads), at::sum(grad_conv, dim_conv)};
+    return {reshaped_result(std::get<0>(grads), in.sizes()), std::get<1>(grads),
+            at::sum(grad_conv, dim_conv)};
 }
 
 // ---- fire ---------------------------------------------------------------------------------------
@@ -338,7 +347,8 @@ std::vector<Tensor> bn_fire_bp(Tensor spatial, Tensor weight_bn, Tensor bias_bn,
                                interval, ws_bytes ? workspace.data_ptr() : nullptr, ws_bytes,
                                current_stream()),
              "bn_fire_bp");
-    return {grad_spatial, grad_weight.view_as(weight_bn), grad_bias.view_as(weight_bn)};
+    return {grad_spatial, reshaped_result(grad_weight, weight_bn.sizes()),
+            reshaped_result(grad_bias, weight_bn.sizes())};
 }
 
 // The two halves of bn_fire_bp that a batch sharded over several GPUs runs before and after the
@@ -371,7 +381,8 @@ std::vector<Tensor> bn_fire_bp_dist1(Tensor spatial, Tensor weight_bn, Tensor bi
                                      ws_bytes ? workspace.data_ptr() : nullptr, ws_bytes,
                                      current_stream()),
              op);
-    return {mean_gxhat, mean_gxhatx, grad_weight.view_as(weight_bn), grad_bias.view_as(weight_bn)};
+    return {mean_gxhat, mean_gxhatx, reshaped_result(grad_weight, weight_bn.sizes()),
+            reshaped_result(grad_bias, weight_bn.sizes())};
 }
 
 Tensor bn_fire_bp_dist2(Tensor spatial, Tensor weight_bn, Tensor bias_bn, Tensor ivar, Tensor mean,
@@ -410,7 +421,7 @@ std::vector<Tensor> bn_fp(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor 
     // y = (x - mean) * weight / sqrt(var + eps) + bias with the statistics the caller supplies
     Tensor y = at::batch_norm(fold_time(x_bn), w, b, m, v, /*training=*/false, /*momentum=*/0.0,
                               eps_bn, /*cudnn_enabled=*/true);
-    return {at::rsqrt(v + eps_bn), y.view(x_bn.sizes())};
+    return {at::rsqrt(v + eps_bn), reshaped_result(y, x_bn.sizes())};
 }
 
 std::vector<Tensor> bn_bp(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor ivar, Tensor mean,
@@ -430,7 +441,7 @@ std::vector<Tensor> bn_bp(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor 
         fold_time(grad_y_bn.contiguous()), fold_time(x_bn.contiguous()), w,
         /*running_mean=*/c10::nullopt, /*running_var=*/c10::nullopt, /*save_mean=*/m,
         /*save_invstd=*/iv, /*train=*/true, /*eps=*/0.0, {true, true, true});
-    return {std::get<0>(grads).view(x_bn.sizes()), std::get<1>(grads), std::get<2>(grads)};
+    return {reshaped_result(std::get<0>(grads), x_bn.sizes()), std::get<1>(grads), std::get<2>(grads)};
 }
 
 // The two halves of bn_bp for a sharded batch (snnlib/cuda/snn_kernel_bp.cu:348-425): local

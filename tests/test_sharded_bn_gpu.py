@@ -282,3 +282,72 @@ def test_dist_modules_with_one_rank(hyper, monkeypatch, kind):
     n = x.numel() / 8
     rel_close(layer.running_mean, 0.05 * mean, "running mean")
     rel_close(layer.running_var, 0.95 + var * (0.05 * n / (n - 1)), "running variance")
+
+
+def test_residual_and_alexnet_style_stacks_of_dist_layers_train(hyper, monkeypatch):
+    """The way the reference composes the sharded layers (snnlib/example/models.py:63-105 Alexnet_BN_DIST,
+    :107-127 ResidualDist, in-place residual add included), scaled down, with one rank."""
+    from snn_gpu_training_bptt_amd import snnlib_op as sop
+    OneRank().install(monkeypatch)
+    torch.manual_seed(50)
+    T, B = 4, 8
+
+    class Residual(torch.nn.Module):
+        def __init__(self, cin, cout, stride, downsample):
+            super().__init__()
+            self.conv1 = sop.FireConv(cin, cout, kernel_size=(3, 3), stride=stride, padding=(1, 1))
+            self.conv2 = sop.BnFireConvDist(cout, cout, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1))
+            self.bn2 = sop.BnDist(cout, dim_bn=(0, 1, 3, 4))
+            self.downsample = downsample
+
+        def forward(self, inp):
+            x = self.bn2(self.conv2(self.conv1(inp)))
+            x += self.downsample(inp) if self.downsample is not None else inp
+            return x
+
+    class Net(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.pre_conv = sop.Conv(3, 8, kernel_size=(3, 3), stride=(1, 1), padding=(1, 1))
+            self.pre_bn = sop.BnDist(8, dim_bn=(0, 1, 3, 4))
+            down = torch.nn.Sequential(sop.FireConv(8, 16, kernel_size=(1, 1), stride=(2, 2), padding=(0, 0)),
+                                       sop.BnDist(16, (0, 1, 3, 4)))
+            self.block1 = Residual(8, 16, (2, 2), down)
+            self.block2 = Residual(16, 16, (1, 1), None)
+            self.conv = sop.BnFireConvDist(16, 16, stride=(2, 2))
+            self.fc1 = sop.BnFireFcDist(4 * 4 * 16, 32, dim_bn=(0, 1, 3, 4), cin_bn=16)
+            self.fc2 = sop.BnFireFcDist(32, 32, dim_bn=(0, 1))
+            self.fire = sop.Fire()
+            self.fc3 = torch.nn.Linear(32, 10)
+
+        def forward(self, images):
+            x = torch.stack([images] * T, dim=0)
+            x = self.pre_bn(self.pre_conv(x))
+            x = self.block2(self.block1(x))
+            x = self.fc2(self.fc1(self.conv(x)))
+            return self.fc3(self.fire(x).mean(dim=0))
+
+    net = Net().cuda()
+    images = torch.rand(B, 3, 16, 16).cuda()
+    labels = torch.randint(0, 10, (B,)).cuda()
+    trainable = [p for n, p in net.named_parameters() if "running" not in n]
+    opt = torch.optim.SGD(trainable, lr=0.05)
+    crit = torch.nn.CrossEntropyLoss()
+    losses = []
+    for _ in range(12):
+        opt.zero_grad(set_to_none=True)
+        loss = crit(net(images), labels)
+        loss.backward()
+        for n, p in net.named_parameters():
+            if "running" not in n:
+                assert p.grad is not None and torch.isfinite(p.grad).all(), n
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert losses[-1] < losses[0], losses
+    # inference with the running statistics
+    for m in net.modules():
+        if hasattr(m, "train_bn"):
+            m.train_bn = False
+    with torch.no_grad():
+        out = net(images)
+    assert out.shape == (B, 10) and torch.isfinite(out).all()
