@@ -707,8 +707,8 @@ int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, f
     const size_t elem[3] = {sizeof(S), sizeof(S), sizeof(S)};
     const int v = pick_vec(maxv, N, ptrs, elem, 3);
     // Every window of at most 8 rows has an instantiation of its own, so only the longer ones
-    // are ever entered with T < TW.
-    constexpr bool can_be_inexact = TW > 8;
+    // are ever entered with T < TW; windows beyond the fused range are entered with T == TW only.
+    constexpr bool can_be_inexact = TW > 8 && TW <= SNNLIF_BP_FUSED_MAX_T;
     const bool exact = !can_be_inexact || (T == TW);
     return with_vec<maxv>(v, [&](auto vc) {
         constexpr int V = decltype(vc)::value;
@@ -771,6 +771,18 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
     SNNLIF_BWD_WINDOW(32)
 #undef SNNLIF_BWD_WINDOW
     static_assert(SNNLIF_BP_FUSED_MAX_T == 32, "windows above must cover the fused range");
+
+    // A few longer windows still fit the register file whole (u alone takes T VGPRs per lane) and
+    // then move 12 bytes per neuron-step instead of the segmented kernel's 16 -- but only in
+    // straight-line form: zero-filling a 48-row window for T = 33 is slower than two segments.
+#define SNNLIF_BWD_WIDE_WINDOW(TW)                                                               \
+    if (T == TW)                                                                                 \
+        return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, stream);
+    SNNLIF_BWD_WIDE_WINDOW(40)
+    SNNLIF_BWD_WIDE_WINDOW(48)
+    SNNLIF_BWD_WIDE_WINDOW(56)
+    SNNLIF_BWD_WIDE_WINDOW(64)
+#undef SNNLIF_BWD_WIDE_WINDOW
 
     // Longer windows, up to what the boundary values of a workgroup fit into 64 KiB of LDS for
     // every storage type: segmented kernel, still no scratch memory in HBM.

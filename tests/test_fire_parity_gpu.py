@@ -104,6 +104,16 @@ def test_fp32_every_window_length(cabi, oracle, T):
         assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
 
 
+@pytest.mark.parametrize("T", [40, 48, 56, 64, 41, 47, 63, 65])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_windows_between_32_and_64(cabi, oracle, T, dtype):
+    """40, 48, 56 and 64 steps run as one register window, their neighbours in two or three
+    segments; both must give the oracle's bits.  Even and odd N."""
+    for n_inner in (256, 77):
+        x, g = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=2000 + T, dtype=dtype)
+        assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
+
+
 @pytest.mark.parametrize("alpha,thresh,beta,interval", [
     (0.3, 0.5, 1.0, 0.5),      # decay that is not a power of two: exposes any FMA contraction
     (0.25, 0.25, 1.0, 0.5),    # the reference's default threshold (snnlib_func.py:14)
@@ -194,7 +204,7 @@ def test_special_values_follow_ieee_like_the_oracle(cabi, oracle):
 
 
 @pytest.mark.parametrize("shape", [(8, 3, 255), (5, 1, 1), (16, 2, 4097), (33, 3, 77), (12, 4, 64, 4, 4),
-                                   (1024, 1, 128), (1040, 1, 30)])
+                                   (48, 2, 130), (64, 2, 77), (64, 3, 256), (1024, 1, 128), (1040, 1, 30)])
 def test_bf16_storage_parity_including_odd_sizes(cabi, oracle, shape):
     """bf16 storage, fp32 arithmetic: two values per lane when N is even and the bases are 4-byte
     aligned, one otherwise.  Expected = the fp32 oracle on the bf16-rounded inputs, outputs rounded
