@@ -147,3 +147,52 @@ def test_bench_refuses_more_than_one_gpu():
                           capture_output=True, text=True)
     assert proc.returncode != 0
     assert "one GPU" in proc.stderr
+
+
+ROUTE_A = r"""
+import sys
+sys.path.insert(0, sys.argv[1])          # the directory that holds snnlib.so, nothing else of this build
+import torch
+import snnlib                            # what the reference's snnlib_func.py does (its line 8)
+assert "snn_gpu_training_bptt_amd" not in sys.modules
+names = ["fire_s_fp", "fire_bp", "bn_fire_s_fp", "bn_fire_bp", "bn_fp", "bn_bp", "fc_fp", "fc_bp", "conv_fp",
+         "conv_bp", "fire_fc_fp", "fire_fc_bp", "fire_conv_fp", "fire_conv_bp", "bn_fire_fc_fp", "bn_fire_fc_bp",
+         "bn_fire_conv_fp", "bn_fire_conv_bp", "bn_bp_dist1", "bn_bp_dist2", "bn_fire_bp_dist1",
+         "bn_fire_bp_dist2", "bn_fire_fc_bp_dist1", "bn_fire_conv_bp_dist1"]
+missing = [n for n in names if not callable(getattr(snnlib, n, None))]
+assert not missing, missing
+if len(sys.argv) > 2:                    # on a GPU: a user-side autograd function written against the module
+    class UserFire(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, x):
+            ctx.save_for_backward(x)
+            return snnlib.fire_s_fp(x, 0.25, 0.5)
+        @staticmethod
+        def backward(ctx, g):
+            (x,) = ctx.saved_tensors
+            return snnlib.fire_bp(x.contiguous(), g.contiguous(), 0.25, 0.5, 1.0, 0.5)
+    x = torch.full((3, 2, 4), 0.6, device="cuda", requires_grad=True)
+    s = UserFire.apply(x)
+    s.sum().backward()
+    # u = 0.6, 0.6, 0.6 (each step fires and resets): spikes all one, every step inside the window
+    assert bool((s == 1).all()) and x.grad.shape == x.shape and bool(torch.isfinite(x.grad).all())
+print("route-a-ok")
+"""
+
+
+def _run_route_a(*extra):
+    lib_dir = os.path.join(REPO, "snn_gpu_training_bptt_amd", "lib")
+    proc = subprocess.run([sys.executable, "-c", ROUTE_A, lib_dir, *extra], capture_output=True, text=True,
+                          cwd="/tmp", timeout=300)
+    assert proc.returncode == 0 and "route-a-ok" in proc.stdout, proc.stderr[-2000:]
+
+
+def test_module_binds_under_its_reference_name_from_the_lib_directory_alone():
+    """`import snnlib` with nothing but the directory of the two shared objects on the path, every
+    entry of the reference's binding table present (snnlib/cuda/snn.cpp:798-829)."""
+    _run_route_a()
+
+
+@pytest.mark.gpu
+def test_user_autograd_function_against_the_bare_module():
+    _run_route_a("gpu")
