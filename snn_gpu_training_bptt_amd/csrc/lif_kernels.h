@@ -41,7 +41,8 @@
 //     element-wise CPU/GPU ops do, which makes spikes, potentials and gradients bit-identical to
 //     the per-op rounded reference arithmetic.
 //
-// Longer windows (32 < T <= 1024) are cut into 32-step segments: one forward pass leaves the
+// Windows of exactly 40, 48, 56 or 64 steps still run as one register window.  Other longer windows
+// (32 < T <= 1024) are cut into 32-step segments: one forward pass leaves the
 // membrane potential at the segment boundaries in LDS, then each segment is recomputed into registers
 // and swept in reverse, last segment first (x is read twice, nothing else changes).  Beyond that the
 // forward kernel writes u to a caller-provided workspace and a streaming reverse kernel reads it back.
