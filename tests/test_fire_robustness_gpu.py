@@ -160,3 +160,58 @@ def test_events_attached_to_the_next_kernel(cabi):
     cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
     torch.cuda.synchronize()
     assert np.array_equal(spike.cpu().numpy(), spike_o)
+
+
+def test_layers_captured_with_torch_cuda_graph():
+    """A forward + backward through the PyTorch-facing layers (Fire, then BnFire with given statistics,
+    whose backward draws its workspace from the caching allocator) captured by torch.cuda.graph and
+    replayed with fresh inputs; every replay equals the eager result of the same layers."""
+    from snn_gpu_training_bptt_amd import snnlib_func as sf
+    saved = (sf.alpha, sf.thresh, sf.beta, sf.interval)
+    sf.alpha, sf.thresh, sf.beta, sf.interval = ALPHA, THRESH, BETA, INTERVAL
+    try:
+        shape = (6, 4, 16, 8, 8)
+        C = shape[2]
+        gen = torch.Generator().manual_seed(84)
+        w = (0.5 + torch.rand(C, generator=gen)).cuda().requires_grad_(True)
+        b = (0.2 * torch.randn(C, generator=gen)).cuda().requires_grad_(True)
+        var = (0.5 + torch.rand(C, generator=gen)).cuda()
+        mean = (0.1 * torch.randn(C, generator=gen)).cuda()
+        x = torch.zeros(shape, device="cuda", requires_grad=True)
+        gout = torch.zeros(shape, device="cuda")
+
+        def run():
+            spikes = sf.fire_func(x)
+            out = sf.bn_fire_func(spikes * 1.5 - 0.2, w, b, var, mean, (0, 1, 3, 4), 1e-5)
+            gx, gw, gb = torch.autograd.grad(out, (x, w, b), gout)
+            return out, gx, gw, gb
+
+        def load(seed):
+            g2 = torch.Generator().manual_seed(seed)
+            with torch.no_grad():
+                x.copy_(0.5 + torch.randn(shape, generator=g2))
+                gout.copy_(torch.randn(shape, generator=g2))
+
+        load(0)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                run()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static = run()
+        for seed in (1, 2, 3, 4):
+            load(seed)
+            graph.replay()
+            torch.cuda.synchronize()
+            got = [t.clone() for t in static]
+            want = run()                      # eager work between the replays
+            torch.cuda.synchronize()
+            for name, a, e in zip(("out", "grad x", "grad weight", "grad bias"), got, want):
+                assert torch.equal(a, e), f"replay with seed {seed}: {name}"
+    finally:
+        sf.alpha, sf.thresh, sf.beta, sf.interval = saved
