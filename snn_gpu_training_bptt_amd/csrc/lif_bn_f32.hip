@@ -10,7 +10,8 @@ int bn_forward_launch(const float* x, const float* weight, const float* bias, co
                       const float* mean, float* ivar, float* spike, int64_t T, int64_t B, int64_t C,
                       int64_t HW, float eps, float alpha, float thresh, hipStream_t stream) {
     const int64_t N = B * C * HW;
-    const dim3 grid(grid_for(N, kFwdBlock)), block(kFwdBlock);
+    const int threads = forward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(float));
+    const dim3 grid(grid_for(N, threads)), block(threads);
     const int Ti = static_cast<int>(T);
     constexpr int TC = SNNLIF_FWD_ROWS;
     if (T <= 4 && TC > 4) {
@@ -41,9 +42,13 @@ int bn_forward_f32(const float* x, const float* weight, const float* bias, const
 
 namespace {
 
+// Small workgroup of the two backward sweeps (see backward_block): the sweeps carry more state per
+// wavefront than the plain backward and single-wavefront groups cost them more than they gain.
+constexpr int kBnSmallBlock = 128;
+
 // Dynamic LDS of the segmented sweeps: one boundary value per segment and lane.
-inline size_t bn_segment_lds_bytes(int64_t T) {
-    return static_cast<size_t>((T + kSegment - 1) / kSegment) * kBwdBlock * sizeof(float);
+inline size_t bn_segment_lds_bytes(int64_t T, int threads) {
+    return static_cast<size_t>((T + kSegment - 1) / kSegment) * threads * sizeof(float);
 }
 
 // Sweep 1 + channel reduction for windows of at most TW steps (SEGMENTED: of any length up to
@@ -61,17 +66,18 @@ int bn_backward_stats_window(const float* x, const float* weight, const float* b
     float* part_gy = workspace;
     float* part_gyx = part_gy + N;
     float* split = part_gyx + N;
-    const dim3 block(kBwdBlock);
+    const int threads = backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(float), kBnSmallBlock);
+    const dim3 block(threads);
     const int Ti = static_cast<int>(T);
     constexpr bool can_be_inexact = TW > 8;
     const bool exact = !SEGMENTED && (!can_be_inexact || (T == TW));
-    const size_t lds = SEGMENTED ? bn_segment_lds_bytes(T) : 0;
+    const size_t lds = SEGMENTED ? bn_segment_lds_bytes(T, threads) : 0;
 
     // Planes with few positions (fully connected shapes) would leave most lanes of a plane-aligned
     // wavefront idle; they keep one lane per neuron and per-neuron partials.
     const bool wave = HW >= 32;
     const int64_t G = (HW + 63) / 64;
-    const dim3 grid_partial(wave ? grid_for(B * C * G * 64, kBwdBlock) : grid_for(N, kBwdBlock));
+    const dim3 grid_partial(wave ? grid_for(B * C * G * 64, threads) : grid_for(N, threads));
     int rc;
 #define SNNLIF_BN_PARTIAL(EXACT_, WAVE_)                                                          \
     launch_kernel(lif_bn_backward_partial_kernel<TW, EXACT_, WAVE_, SEGMENTED>, grid_partial, block, \
@@ -115,13 +121,14 @@ int bn_backward_input_window(const float* x, const float* weight, const float* b
                              int64_t B, int64_t C, int64_t HW, float alpha, float thresh, float beta,
                              float interval, hipStream_t stream) {
     const int64_t N = B * C * HW;
-    const dim3 grid(grid_for(N, kBwdBlock)), block(kBwdBlock);
+    const int threads = backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(float), kBnSmallBlock);
+    const dim3 grid(grid_for(N, threads)), block(threads);
     const int Ti = static_cast<int>(T);
     constexpr bool can_be_inexact = TW > 8;
     const bool exact = !SEGMENTED && (!can_be_inexact || (T == TW));
     if constexpr (SEGMENTED) {
         launch_kernel(lif_bn_backward_input_kernel<TW, false, true>, grid, block,
-                      bn_segment_lds_bytes(T), stream, x, g, weight, bias, ivar, mean, mean_gxhat,
+                      bn_segment_lds_bytes(T, threads), stream, x, g, weight, bias, ivar, mean, mean_gxhat,
                       mean_gxhatx, gx, Ti, N, C, HW, alpha, thresh, beta, interval);
     } else if (exact) {
         launch_kernel(lif_bn_backward_input_kernel<TW, true>, grid, block, 0, stream, x, g, weight,

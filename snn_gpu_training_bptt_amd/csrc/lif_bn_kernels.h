@@ -65,8 +65,8 @@ lif_bn_forward_kernel(const float* __restrict__ x, const float* __restrict__ wei
                       float* __restrict__ spike, int T, int64_t N, int64_t C, int64_t HW, float eps,
                       float alpha, float thresh) {
     const bool small = N <= 0xffffffffll;
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kFwdBlock;
-    for (int64_t col = static_cast<int64_t>(blockIdx.x) * kFwdBlock + threadIdx.x; col < N;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t col = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; col < N;
          col += stride) {
         const int c = channel_of(col, C, HW, small);
         const float m = mean[c];
@@ -169,7 +169,7 @@ __device__ __forceinline__ void bn_reverse_chain(const float* __restrict__ x,
 
 // Time axes longer than one register window, in segments of kSegment steps, the way
 // lif_backward_segmented_kernel does it: forward over all but the last segment keeping the membrane
-// potential at each boundary in this lane's own LDS slots (`boundary`: [segment][kBwdBlock] floats
+// potential at each boundary in this lane's own LDS slots (`boundary`: [segment][blockDim.x] floats
 // of dynamic LDS), then the segments last to first.  emit gets the absolute time step.
 template <typename Emit>
 __device__ __forceinline__ void bn_reverse_segmented(const float* __restrict__ x,
@@ -193,7 +193,7 @@ __device__ __forceinline__ void bn_reverse_segmented(const float* __restrict__ x
                 sc = (uc > thresh) ? 1.f : 0.f;
             }
         }
-        boundary[(seg + 1) * kBwdBlock + threadIdx.x] = uc;
+        boundary[(seg + 1) * blockDim.x + threadIdx.x] = uc;
     }
     {
         const int t0 = (nseg - 1) * kSegment;
@@ -203,7 +203,7 @@ __device__ __forceinline__ void bn_reverse_segmented(const float* __restrict__ x
                                            [&](int t, float gy, float xt) { emit(t0 + t, gy, xt); });
     }
     for (int seg = nseg - 2; seg >= 0; --seg) {
-        uc = seg == 0 ? 0.f : boundary[seg * kBwdBlock + threadIdx.x];
+        uc = seg == 0 ? 0.f : boundary[seg * blockDim.x + threadIdx.x];
         sc = (seg != 0 && uc > thresh) ? 1.f : 0.f;
         const int t0 = seg * kSegment;
         const int64_t off = static_cast<int64_t>(t0) * N;
@@ -251,11 +251,11 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
     extern __shared__ __align__(16) unsigned char lds_raw[];
     float* boundary = reinterpret_cast<float*>(lds_raw);  // used by SEGMENTED only
     const bool small = N <= 0xffffffffll;
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     if (WAVE) {
         const int64_t G = (HW + 63) / 64;
         const int64_t lanes = (N / HW) * G * 64;  // padded lane space: planes * G wavefronts
-        for (int64_t pc = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; pc < lanes;
+        for (int64_t pc = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; pc < lanes;
              pc += stride) {
             const int64_t wave = pc >> 6;
             const int64_t plane = wave / G;
@@ -282,7 +282,7 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
             }
         }
     } else {
-        for (int64_t col = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; col < N;
+        for (int64_t col = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; col < N;
              col += stride) {
             const int c = channel_of(col, C, HW, small);
             const float m = mean[c], iv = ivar[c];
@@ -315,8 +315,8 @@ lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restric
     extern __shared__ __align__(16) unsigned char lds_raw[];
     float* boundary = reinterpret_cast<float*>(lds_raw);  // used by SEGMENTED only
     const bool small = N <= 0xffffffffll;
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
-    for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < N;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < N;
          v += stride) {
         const int64_t col = N - 1 - v;  // opposite direction to sweep 1: its tail is still cached
         const int c = channel_of(col, C, HW, small);

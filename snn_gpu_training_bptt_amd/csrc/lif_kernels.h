@@ -69,6 +69,10 @@
 #ifndef SNNLIF_BWD_BLOCK
 #define SNNLIF_BWD_BLOCK 256
 #endif
+// Largest tensor (bytes) for which the forward and the fused backward use their small workgroups.
+#ifndef SNNLIF_SMALL_TENSOR_BYTES
+#define SNNLIF_SMALL_TENSOR_BYTES (size_t(160) << 20)
+#endif
 // VGPR budget (in 32-bit words) the fused backward may spend on the recomputed membrane potential.
 #ifndef SNNLIF_FUSED_U_WORDS
 #define SNNLIF_FUSED_U_WORDS 128
@@ -113,6 +117,20 @@ constexpr int lane_vec(size_t elem_bytes) {
 }
 constexpr int kFwdBlock = SNNLIF_FWD_BLOCK;
 constexpr int kBwdBlock = SNNLIF_BWD_BLOCK;
+
+// Workgroup size of the forward and the fused backward by the size of one tensor.  Tensors that
+// the 256 MB memory-side cache can hold together with their outputs are served at fabric speed, and
+// there small workgroups win (more, shorter-lived groups whose wavefronts are out of step with each
+// other; measured +15-20 % forward, +5-10 % backward between 16 and 128 MiB); tensors streamed from
+// HBM prefer the large workgroup, whose wavefronts walk neighbouring DRAM pages together (small
+// groups lose 5-10 % from 512 MiB on).  Between the two (192-256 MiB) it makes no difference.
+constexpr size_t kSmallTensorBytes = SNNLIF_SMALL_TENSOR_BYTES;
+inline int forward_block(size_t tensor_bytes) {
+    return (tensor_bytes <= kSmallTensorBytes && kFwdBlock > 128) ? 128 : kFwdBlock;
+}
+inline int backward_block(size_t tensor_bytes, int small = 64) {
+    return (tensor_bytes <= kSmallTensorBytes && kBwdBlock > small) ? small : kBwdBlock;
+}
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -233,8 +251,8 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
                    int64_t N, int64_t nvec, typename Arith<S>::type alpha,
                    typename Arith<S>::type thresh) {
     using C = typename Arith<S>::type;
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kFwdBlock;
-    for (int64_t v = static_cast<int64_t>(blockIdx.x) * kFwdBlock + threadIdx.x; v < nvec;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < nvec;
          v += stride) {
         const int64_t col = v * V;
         C u[V], s[V];
@@ -399,8 +417,8 @@ lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* _
                           typename Arith<S>::type thresh, typename Arith<S>::type beta,
                           typename Arith<S>::type interval) {
     using C = typename Arith<S>::type;
-    const int64_t stride = static_cast<int64_t>(gridDim.x) * kBwdBlock;
-    for (int64_t v = static_cast<int64_t>(blockIdx.x) * kBwdBlock + threadIdx.x; v < nvec;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < nvec;
          v += stride) {
         const int64_t col = backward_column(v, nvec, V);
         C uc[V], sc[V], gu[V];
@@ -638,7 +656,8 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
                       hipStream_t stream) {
     using C = typename Arith<S>::type;
     const int64_t nvec = N / V;
-    const dim3 grid(grid_for(nvec, kFwdBlock)), block(kFwdBlock);
+    const int threads = forward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S));
+    const dim3 grid(grid_for(nvec, threads)), block(threads);
     const int Ti = static_cast<int>(T);
     constexpr int TC = SNNLIF_FWD_ROWS;
     if (T <= 4 && TC > 4) {
@@ -714,7 +733,9 @@ int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, f
     return with_vec<maxv>(v, [&](auto vc) {
         constexpr int V = decltype(vc)::value;
         const int64_t nvec = N / V;
-        const dim3 grid(grid_for(nvec, kBwdBlock)), block(kBwdBlock);
+        const int threads =
+            backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S));
+        const dim3 grid(grid_for(nvec, threads)), block(threads);
         const int Ti = static_cast<int>(T);
         if (exact) {
             launch_kernel(lif_backward_fused_kernel<S, V, TW, true>, grid, block, 0, stream,
