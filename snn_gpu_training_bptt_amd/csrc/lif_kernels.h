@@ -69,9 +69,12 @@
 #ifndef SNNLIF_BWD_BLOCK
 #define SNNLIF_BWD_BLOCK 256
 #endif
-// Largest tensor (bytes) for which the forward and the fused backward use their small workgroups.
+// Largest tensor (bytes) for which the fused backward / the forward use their small workgroups.
 #ifndef SNNLIF_SMALL_TENSOR_BYTES
 #define SNNLIF_SMALL_TENSOR_BYTES (size_t(160) << 20)
+#endif
+#ifndef SNNLIF_SMALL_TENSOR_BYTES_FWD
+#define SNNLIF_SMALL_TENSOR_BYTES_FWD (size_t(256) << 20)
 #endif
 // VGPR budget (in 32-bit words) the fused backward may spend on the recomputed membrane potential.
 #ifndef SNNLIF_FUSED_U_WORDS
@@ -123,10 +126,13 @@ constexpr int kBwdBlock = SNNLIF_BWD_BLOCK;
 // there small workgroups win (more, shorter-lived groups whose wavefronts are out of step with each
 // other; measured +15-20 % forward, +5-10 % backward between 16 and 128 MiB); tensors streamed from
 // HBM prefer the large workgroup, whose wavefronts walk neighbouring DRAM pages together (small
-// groups lose 5-10 % from 512 MiB on).  Between the two (192-256 MiB) it makes no difference.
+// groups lose 5-10 % from 512 MiB on).  Between the two (192-256 MiB) it makes no difference to
+// the backward and to short forward windows, while forward windows of 24-32 steps still gain 5-10 %,
+// so the forward switches later than the backward.
 constexpr size_t kSmallTensorBytes = SNNLIF_SMALL_TENSOR_BYTES;
+constexpr size_t kSmallTensorBytesFwd = SNNLIF_SMALL_TENSOR_BYTES_FWD;
 inline int forward_block(size_t tensor_bytes) {
-    return (tensor_bytes <= kSmallTensorBytes && kFwdBlock > 128) ? 128 : kFwdBlock;
+    return (tensor_bytes <= kSmallTensorBytesFwd && kFwdBlock > 128) ? 128 : kFwdBlock;
 }
 inline int backward_block(size_t tensor_bytes, int small = 64) {
     return (tensor_bytes <= kSmallTensorBytes && kBwdBlock > small) ? small : kBwdBlock;
