@@ -76,6 +76,11 @@
 #ifndef SNNLIF_SMALL_TENSOR_BYTES_FWD
 #define SNNLIF_SMALL_TENSOR_BYTES_FWD (size_t(256) << 20)
 #endif
+// Windows of at most this many steps give a lane too few rows to keep enough bytes in flight with
+// one dword per access; they use 16-byte lanes instead (4 fp32 / 2 fp64 / 8 bf16 neurons per lane).
+#ifndef SNNLIF_WIDE_LANE_MAX_T
+#define SNNLIF_WIDE_LANE_MAX_T 2
+#endif
 // VGPR budget (in 32-bit words) the fused backward may spend on the recomputed membrane potential.
 #ifndef SNNLIF_FUSED_U_WORDS
 #define SNNLIF_FUSED_U_WORDS 128
@@ -679,6 +684,20 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
     return launch_status();
 }
 
+// Windows of at most SNNLIF_WIDE_LANE_MAX_T (<= 4) steps: only the 4-row instantiation is needed.
+template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S>
+int launch_forward_short(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha,
+                         float thresh, hipStream_t stream) {
+    using C = typename Arith<S>::type;
+    static_assert(SNNLIF_WIDE_LANE_MAX_T <= 4, "the short-window forward holds 4 rows");
+    const int64_t nvec = N / V;
+    const int threads = forward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S));
+    launch_kernel(lif_forward_kernel<S, M, V, 4, false, WRITE_U, WRITE_S>,
+                  dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
+                  static_cast<int>(T), N, nvec, C(alpha), C(thresh));
+    return launch_status();
+}
+
 template <typename S, typename M, bool WRITE_U, bool WRITE_S>
 int launch_forward(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
                    hipStream_t stream) {
@@ -693,6 +712,15 @@ int launch_forward(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alp
     const size_t elem[3] = {sizeof(S), sizeof(M), sizeof(S)};
     for (int i = 0; i < 3; ++i)
         if (!aligned_to(ptrs[i], elem[i])) return SNNLIF_ERR_ALIGN;
+    if (T <= SNNLIF_WIDE_LANE_MAX_T) {
+        constexpr int widev = static_cast<int>(16 / widest);
+        const int wv = pick_vec(widev, N, ptrs, elem, 3);
+        return with_vec<widev>(wv, [&](auto vc) {
+            constexpr int V = decltype(vc)::value;
+            return launch_forward_short<S, M, V, WRITE_U, WRITE_S>(x, mem, spike, T, N, alpha, thresh,
+                                                                   stream);
+        });
+    }
     const int v = pick_vec(maxv, N, ptrs, elem, 3);
     return with_vec<maxv>(v, [&](auto vc) {
         constexpr int V = decltype(vc)::value;
@@ -720,7 +748,8 @@ constexpr int fused_max_vec() {
     using C = typename Arith<S>::type;
     constexpr int words = static_cast<int>(sizeof(C) / 4);
     constexpr int cap = SNNLIF_FUSED_U_WORDS / (TW * words);
-    constexpr int hw = Arith<S>::kMaxVec;
+    constexpr int hw = TW <= SNNLIF_WIDE_LANE_MAX_T ? static_cast<int>(16 / sizeof(S))
+                                                    : Arith<S>::kMaxVec;
     return cap < 1 ? 1 : (cap < hw ? cap : hw);
 }
 

@@ -114,6 +114,16 @@ def test_windows_between_32_and_64(cabi, oracle, T, dtype):
         assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
 
 
+@pytest.mark.parametrize("T", [1, 2])
+@pytest.mark.parametrize("n_inner", [4096, 4098, 4097, 8])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_very_short_windows_use_wide_lanes(cabi, oracle, T, n_inner, dtype):
+    """One- and two-step windows move 16 bytes per lane when N and the bases allow it (N a multiple
+    of 4 for fp32), 8 or one element otherwise; every width must give the oracle's bits."""
+    x, g = make_inputs((T, 3, n_inner), 0.4, 0.9, seed=3000 + T + n_inner, dtype=dtype)
+    assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
+
+
 @pytest.mark.parametrize("alpha,thresh,beta,interval", [
     (0.3, 0.5, 1.0, 0.5),      # decay that is not a power of two: exposes any FMA contraction
     (0.25, 0.25, 1.0, 0.5),    # the reference's default threshold (snnlib_func.py:14)
