@@ -22,7 +22,9 @@
 //     beats 16-byte lanes by 5-15 %: the narrow kernels need ~25 VGPRs, so every SIMD holds its full
 //     8 waves, and the many small in-flight requests of one wave stay within a few DRAM pages per
 //     row instead of spreading over sixteen.  It also removes every alignment constraint for fp32
-//     and fp64 (element alignment is all a dword lane needs).
+//     and fp64 (element alignment is all a dword lane needs).  Windows of one or two steps are the
+//     exception: too few rows per lane to fill the memory pipeline, so they take 16-byte lanes
+//     when N and the base addresses allow it.
 //   * The backward recomputes u[0..T-1] from x into registers (T <= 32) instead of writing a
 //     membrane tensor to HBM and reading it back: 12 bytes per neuron-step instead of 20.
 //     Gradient rows are streamed in reverse time order through a double-buffered register window.
