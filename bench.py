@@ -60,7 +60,8 @@ WORKLOADS = {
 # this file (each counter scaled by its reading for a plain device copy of the same tensor:
 # --copy-calibration); the summary with the commands is profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt.
 # Counters cannot be read from inside this process, so workloads without a profiled figure report null.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 805276475}
+# bn_fire: the three backward kernels together, profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt.
+MEASURED_TRAFFIC_BYTES = {"cfg2": 805276475, "bn_fire": 1346500000}
 METRIC = "LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T=8,B=64,C=128,32x32"
 
 
@@ -276,7 +277,8 @@ def run_bn_fire(args):
         "roofline": {"kernel": "lif_bn_backward_partial_kernel + bn_channel_reduce/finalize + lif_bn_backward_input_kernel",
                      "bound": "hbm", "algorithmic_bytes_per_launch": 20 * ns, "avg_launch_ms": bwd_ms,
                      "achieved": 20 * ns / (bwd_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": 20 * ns / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS, "traffic": None,
+                     "frac": 20 * ns / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get("bn_fire"),
                      "fwd": {"algorithmic_bytes_per_launch": 8 * ns, "avg_launch_ms": fwd_ms,
                              "achieved": 8 * ns / (fwd_ms * 1e-3) / 1e9,
                              "frac": 8 * ns / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
