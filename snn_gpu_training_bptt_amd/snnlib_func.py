@@ -34,6 +34,16 @@ _DIM_CONV = (0, 1, 3, 4)    # axes a convolution bias gradient / conv-shaped bat
 _DILATION, _GROUPS = (1, 1), 1
 
 
+def _dynamics():
+    """Hyper-parameters of the forward recurrence, read from the module globals at call time."""
+    return alpha, thresh
+
+
+def _surrogate():
+    """Those plus the surrogate-gradient parameters the backward ops take."""
+    return alpha, thresh, beta, interval
+
+
 def _pad(grads, n):
     """Gradients for the first inputs, ``None`` for the remaining non-tensor ones."""
     return tuple(grads) + (None,) * (n - len(grads))
@@ -45,14 +55,14 @@ class FireFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, spatial):
         ctx.save_for_backward(spatial)
-        return snnlib.fire_s_fp(spatial, alpha, thresh)
+        return snnlib.fire_s_fp(spatial, *_dynamics())
 
     @staticmethod
     def backward(ctx, grad_spike):
         (spatial,) = ctx.saved_tensors
         # the native op makes both operands dense itself (the upstream gradient is often a
         # stride-0 expansion, e.g. after a mean over time)
-        return snnlib.fire_bp(spatial, grad_spike, alpha, thresh, beta, interval)
+        return snnlib.fire_bp(spatial, grad_spike, *_surrogate())
 
 
 class BnFunc(torch.autograd.Function):
@@ -76,7 +86,7 @@ class BnFireFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, spatial, weight_bn, bias_bn, var, mean, dim_bn, eps_bn):
-        ivar, spike = snnlib.bn_fire_s_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn, alpha, thresh)
+        ivar, spike = snnlib.bn_fire_s_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn, *_dynamics())
         ctx.save_for_backward(spatial, weight_bn, bias_bn, ivar, mean)
         ctx.dim_bn = dim_bn
         return spike
@@ -84,8 +94,7 @@ class BnFireFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_spike):
         # saved: spatial, weight_bn, bias_bn, ivar, mean
-        return _pad(snnlib.bn_fire_bp(*ctx.saved_tensors, ctx.dim_bn, grad_spike,
-                                      alpha, thresh, beta, interval), 7)
+        return _pad(snnlib.bn_fire_bp(*ctx.saved_tensors, ctx.dim_bn, grad_spike, *_surrogate()), 7)
 
 
 class BnFireFcFunc(torch.autograd.Function):
@@ -94,7 +103,7 @@ class BnFireFcFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, spatial, weight_bn, bias_bn, var, mean, dim_bn, eps_bn, weight_fc, bias_fc):
         ivar, fc = snnlib.bn_fire_fc_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn,
-                                        weight_fc, bias_fc, alpha, thresh)
+                                        weight_fc, bias_fc, *_dynamics())
         ctx.save_for_backward(spatial, weight_bn, bias_bn, ivar, mean, weight_fc, bias_fc)
         ctx.dim_bn = dim_bn
         return fc
@@ -103,7 +112,7 @@ class BnFireFcFunc(torch.autograd.Function):
     def backward(ctx, grad_fc):
         *bn_saved, weight_fc, bias_fc = ctx.saved_tensors
         grads = snnlib.bn_fire_fc_bp(*bn_saved, ctx.dim_bn, grad_fc, weight_fc, bias_fc, _DIM_FC,
-                                     alpha, thresh, beta, interval)
+                                     *_surrogate())
         # spatial and the two batch-norm parameters, then var / mean / dim_bn / eps_bn, then the fc pair
         return (*grads[:3], None, None, None, None, *grads[3:])
 
@@ -114,13 +123,12 @@ class FireFcFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, spatial, weight_fc, bias_fc):
         ctx.save_for_backward(spatial, weight_fc, bias_fc)
-        return snnlib.fire_fc_fp(spatial, weight_fc, bias_fc, alpha, thresh)
+        return snnlib.fire_fc_fp(spatial, weight_fc, bias_fc, *_dynamics())
 
     @staticmethod
     def backward(ctx, grad_fc):
         spatial, *fc_params = ctx.saved_tensors
-        return tuple(snnlib.fire_fc_bp(spatial, grad_fc, *fc_params, _DIM_FC,
-                                       alpha, thresh, beta, interval))
+        return tuple(snnlib.fire_fc_bp(spatial, grad_fc, *fc_params, _DIM_FC, *_surrogate()))
 
 
 class FcFunc(torch.autograd.Function):
@@ -151,7 +159,7 @@ class BnFireConvFunc(torch.autograd.Function):
                 weight_conv, bias_conv, stride, padding, if_bias_conv):
         ivar, conv = snnlib.bn_fire_conv_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn,
                                             weight_conv, bias_conv, stride, padding, _DILATION, _GROUPS,
-                                            conv_benchmark, False, alpha, thresh)
+                                            conv_benchmark, False, *_dynamics())
         ctx.save_for_backward(spatial, weight_bn, bias_bn, ivar, mean, weight_conv, bias_conv)
         ctx.stride, ctx.padding, ctx.if_bias_conv = stride, padding, if_bias_conv
         return conv
@@ -161,7 +169,7 @@ class BnFireConvFunc(torch.autograd.Function):
         *bn_saved, weight_conv, _ = ctx.saved_tensors
         g_spatial, g_weight_bn, g_bias_bn, g_weight_conv, g_bias_conv = snnlib.bn_fire_conv_bp(
             *bn_saved, _DIM_CONV, grad_conv, weight_conv, ctx.stride, ctx.padding, _DILATION, _GROUPS,
-            conv_benchmark, False, True, _DIM_CONV, alpha, thresh, beta, interval)
+            conv_benchmark, False, True, _DIM_CONV, *_surrogate())
         return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv,
                            leading=(g_spatial, g_weight_bn, g_bias_bn, None, None, None))
 
@@ -174,14 +182,14 @@ class FireConvFunc(torch.autograd.Function):
         ctx.save_for_backward(spatial, weight_conv, bias_conv)
         ctx.stride, ctx.padding, ctx.if_bias_conv = stride, padding, if_bias_conv
         return snnlib.fire_conv_fp(spatial, weight_conv, bias_conv, stride, padding, _DILATION, _GROUPS,
-                                   conv_benchmark, False, alpha, thresh)
+                                   conv_benchmark, False, *_dynamics())
 
     @staticmethod
     def backward(ctx, grad_conv):
         spatial, weight_conv, bias_conv = ctx.saved_tensors
         g_spatial, g_weight_conv, g_bias_conv = snnlib.fire_conv_bp(
             spatial, grad_conv, weight_conv, ctx.stride, ctx.padding, _DILATION, _GROUPS,
-            conv_benchmark, False, True, _DIM_CONV, alpha, thresh, beta, interval)
+            conv_benchmark, False, True, _DIM_CONV, *_surrogate())
         return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv, leading=(g_spatial,))
 
 
@@ -235,7 +243,7 @@ class BnDistFunc(BnFunc):
 def _sharded_bn_fire_input_grad(ctx, bn_saved, g_spike, local_xhat, local_xhatx):
     """Second half of a sharded bn + fire backward: average the means, then the input gradient."""
     g_xhat, g_xhatx = _mean_over_ranks(local_xhat, local_xhatx, ctx.reduce_op)
-    return snnlib.bn_fire_bp_dist2(*bn_saved, g_spike, g_xhat, g_xhatx, alpha, thresh, beta, interval)
+    return snnlib.bn_fire_bp_dist2(*bn_saved, g_spike, g_xhat, g_xhatx, *_surrogate())
 
 
 class BnFireFcDistFunc(BnFireFcFunc):
@@ -250,7 +258,7 @@ class BnFireFcDistFunc(BnFireFcFunc):
     def backward(ctx, grad_fc):
         *bn_saved, weight_fc, bias_fc = ctx.saved_tensors
         g_spike, local_xhat, local_xhatx, *param_grads = snnlib.bn_fire_fc_bp_dist1(
-            *bn_saved, ctx.dim_bn, grad_fc, weight_fc, bias_fc, _DIM_FC, alpha, thresh, beta, interval)
+            *bn_saved, ctx.dim_bn, grad_fc, weight_fc, bias_fc, _DIM_FC, *_surrogate())
         g_weight_bn, g_bias_bn, g_weight_fc, g_bias_fc = param_grads
         g_spatial = _sharded_bn_fire_input_grad(ctx, bn_saved, g_spike, local_xhat, local_xhatx)
         return (g_spatial, g_weight_bn, g_bias_bn, None, None, None, None, g_weight_fc, g_bias_fc,
@@ -270,7 +278,7 @@ class BnFireConvDistFunc(BnFireConvFunc):
         *bn_saved, weight_conv, _ = ctx.saved_tensors
         g_spike, local_xhat, local_xhatx, *param_grads = snnlib.bn_fire_conv_bp_dist1(
             *bn_saved, _DIM_CONV, grad_conv, weight_conv, ctx.stride, ctx.padding, _DILATION, _GROUPS,
-            conv_benchmark, False, True, _DIM_CONV, alpha, thresh, beta, interval)
+            conv_benchmark, False, True, _DIM_CONV, *_surrogate())
         g_weight_bn, g_bias_bn, g_weight_conv, g_bias_conv = param_grads
         g_spatial = _sharded_bn_fire_input_grad(ctx, bn_saved, g_spike, local_xhat, local_xhatx)
         return _conv_grads(ctx, g_spatial, g_weight_conv, g_bias_conv,
