@@ -215,3 +215,51 @@ def test_layers_captured_with_torch_cuda_graph():
                 assert torch.equal(a, e), f"replay with seed {seed}: {name}"
     finally:
         sf.alpha, sf.thresh, sf.beta, sf.interval = saved
+
+
+def test_host_threads_launching_concurrently(cabi):
+    """Four host threads, each with its own stream and tensors, calling the C ABI at the same time
+    (ctypes drops the GIL for the duration of a call): the library keeps no shared state, and the
+    timing hook of one thread must not leak into another's launches."""
+    import threading
+    from oracle import c_oracle
+    shape = (6, 4, 32, 16, 16)
+    results, errors = {}, []
+    start = threading.Barrier(4)
+
+    def worker(idx):
+        try:
+            gen = torch.Generator().manual_seed(90 + idx)
+            x_cpu = 0.5 + torch.randn(shape, generator=gen)
+            g_cpu = torch.randn(shape, generator=gen)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                x, g = x_cpu.cuda(), g_cpu.cuda()
+                spike, gx = torch.empty_like(x), torch.empty_like(x)
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                e1.record()
+                start.wait()
+                for it in range(20):
+                    if idx == 0 and it == 10:        # only this thread arms the hook
+                        cabi.time_next_kernel(e0, e1)
+                    cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+                    cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+                stream.synchronize()
+            results[idx] = (x_cpu, g_cpu, spike.cpu(), gx.cpu(), e0.elapsed_time(e1) if idx == 0 else None)
+        except Exception as exc:  # surfaced in the main thread below
+            errors.append((idx, repr(exc)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=120)
+    assert not errors, errors
+    assert sorted(results) == [0, 1, 2, 3]
+    for idx, (x_cpu, g_cpu, spike, gx, ms) in results.items():
+        _, spike_o = c_oracle.fire_forward(x_cpu.numpy(), ALPHA, THRESH)
+        gx_o = c_oracle.fire_backward(x_cpu.numpy(), g_cpu.numpy(), ALPHA, THRESH, BETA, INTERVAL)
+        assert np.array_equal(spike.numpy(), spike_o), f"thread {idx}: spikes"
+        assert np.array_equal(gx.numpy(), gx_o), f"thread {idx}: gradients"
+    assert results[0][4] > 0.0
