@@ -221,3 +221,64 @@ def test_cifar_style_stack_trains(mods):
         opt.step()
         losses.append(loss.item())
     assert losses[-1] < losses[0], losses
+
+
+def test_cifar_model_at_full_width(mods):
+    """The reference's CIFAR model at its real layer widths (snnlib/example/models.py:8-61: 128-128-128 /
+    256-256-256 / 512-512-512 convolutions, 8192-1024-512 fully connected, T = 6), assembled from this
+    build's layers: two SGD steps on a small batch, then inference with the running statistics."""
+    _, sop, _ = mods
+    import numpy as np
+    torch.manual_seed(61)
+    T, B = 6, 8
+
+    class Cifar(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            s1, s2, p = (1, 1), (2, 2), (1, 1)
+            self.conv1_1 = sop.Conv(3, 128, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv1_2 = sop.BnFireConv(128, 128, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv1_3 = sop.BnFireConv(128, 128, kernel_size=(3, 3), stride=s2, padding=p)
+            self.conv2_1 = sop.BnFireConv(128, 256, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv2_2 = sop.BnFireConv(256, 256, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv2_3 = sop.BnFireConv(256, 256, kernel_size=(3, 3), stride=s2, padding=p)
+            self.conv3_1 = sop.BnFireConv(256, 512, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv3_2 = sop.BnFireConv(512, 512, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv3_3 = sop.BnFireConv(512, 512, kernel_size=(3, 3), stride=s2, padding=p)
+            self.fc1 = sop.BnFireFc(4 * 4 * 512, 1024, dim_bn=(0, 1, 3, 4), cin_bn=512)
+            self.fc2 = sop.BnFireFc(1024, 512, dim_bn=(0, 1))
+            self.bn = sop.BnFire(512, dim_bn=(0, 1))
+            self.fc3 = torch.nn.Linear(512, 10)
+
+        def forward(self, images):
+            x = torch.stack([images for _ in range(T)], dim=0)
+            for name in ("conv1_1", "conv1_2", "conv1_3", "conv2_1", "conv2_2", "conv2_3",
+                         "conv3_1", "conv3_2", "conv3_3", "fc1", "fc2", "bn"):
+                x = getattr(self, name)(x)
+            return self.fc3(x.mean(dim=0))
+
+    net = Cifar().cuda()
+    images = torch.rand(B, 3, 32, 32).cuda()
+    labels = torch.randint(0, 10, (B,)).cuda()
+    trainable = [p for n, p in net.named_parameters() if "running" not in n]
+    opt = torch.optim.SGD(trainable, lr=0.02)
+    crit = torch.nn.CrossEntropyLoss()
+    losses = []
+    for _ in range(2):
+        opt.zero_grad(set_to_none=True)
+        loss = crit(net(images), labels)
+        loss.backward()
+        for n, p in net.named_parameters():
+            if "running" not in n:
+                assert p.grad is not None and bool(torch.isfinite(p.grad).all()), n
+        opt.step()
+        losses.append(float(loss.detach()))
+    assert all(np.isfinite(losses)), losses
+    spikes_seen = net.bn(torch.randn(T, B, 512, device="cuda"))
+    assert bool(((spikes_seen == 0) | (spikes_seen == 1)).all())
+    for m in net.modules():
+        if hasattr(m, "train_bn"):
+            m.train_bn = False
+    with torch.no_grad():
+        out = net(images)
+    assert out.shape == (B, 10) and bool(torch.isfinite(out).all())
