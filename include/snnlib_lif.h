@@ -128,7 +128,10 @@ int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spati
                    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
- * Batch-norm + fire forward (fp32 only: dtype must be SNNLIF_DTYPE_F32, else SNNLIF_ERR_UNSUPPORTED).
+ * Batch-norm + fire forward (dtype SNNLIF_DTYPE_F32 or SNNLIF_DTYPE_F64, which also is the type of the
+ * per-channel vectors; SNNLIF_DTYPE_BF16: SNNLIF_ERR_UNSUPPORTED).  In fp64 the per-channel statistics
+ * stay in double (the reference's double dispatch narrows them to float inside its kernels,
+ * snnlib/cuda/snn_kernel_fp.cu:184).
  * Tensors are [T, B, C, HW] (HW = 1 for [T, B, C]); weight, bias, var, mean, ivar are [C].
  *   scale[c] = weight[c] / sqrt(var[c] + eps);   ivar[c] = scale[c] / weight[c]
  *   u[t] = (alpha*u[t-1])*(1-s[t-1]) + (x[t] - mean[c])*scale[c] + bias[c];   s[t] = u[t] > thresh
@@ -142,7 +145,7 @@ int snnlif_bn_fire_s_fp(const void* spatial, const void* weight, const void* bia
 /*
  * Spikes of the batch-norm + fire layer recomputed from saved statistics, the way the backward of
  * the fused layers sees them: scale[c] = weight[c] * ivar[c] (not weight / sqrt(var + eps)), same
- * recurrence as snnlif_bn_fire_s_fp, fp32 only.  Replaces bn_fire_us_fp_kernel
+ * recurrence as snnlif_bn_fire_s_fp, fp32 or fp64.  Replaces bn_fire_us_fp_kernel
  * (snnlib/cuda/snn_kernel_bp.cu:481-530) as used by bn_fire_fc_bp_cuda (:890) and bn_fire_conv_bp_cuda
  * (:1215); the membrane potential it also writes there is not needed here because
  * snnlif_bn_fire_bp recomputes it in registers.
@@ -152,12 +155,12 @@ int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const vo
                                int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
                                void* stream);
 
-/* Bytes of device workspace snnlif_bn_fire_bp needs (two floats per neuron plus per-channel
- * staging).  0 for invalid arguments. */
+/* Bytes of device workspace snnlif_bn_fire_bp needs (two values of the storage type per neuron plus
+ * per-channel staging).  0 for invalid arguments. */
 size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);
 
 /*
- * Batch-norm + fire backward (fp32 only; T <= SNNLIF_BP_NO_WORKSPACE_MAX_T, else
+ * Batch-norm + fire backward (fp32 or fp64; T <= SNNLIF_BP_NO_WORKSPACE_MAX_T, else
  * SNNLIF_ERR_UNSUPPORTED; windows longer than SNNLIF_BP_FUSED_MAX_T read x twice per sweep).
  * With u recomputed from scale[c] = weight[c]*ivar[c], gy the fire reverse chain (see
  * snnlif_fire_bp), xhat = (x - mean[c])*ivar[c] and M = T*B*HW:
@@ -177,7 +180,7 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
 
 /*
  * The same backward in the two halves that a batch sharded over several GPUs runs on either side of
- * an all-reduce (fp32 only, T <= SNNLIF_BP_NO_WORKSPACE_MAX_T, shapes and workspace as snnlif_bn_fire_bp;
+ * an all-reduce (fp32 or fp64, T <= SNNLIF_BP_NO_WORKSPACE_MAX_T, shapes and workspace as snnlif_bn_fire_bp;
  * B is the local batch).
  *
  * snnlif_bn_fire_bp_dist1: the local parameter gradients and the local per-channel means

@@ -39,10 +39,10 @@ def _load():
         getattr(lib, f"lif_oracle_reverse_{sfx}").restype = None
         getattr(lib, f"lif_oracle_backward_{sfx}").argtypes = [ptr, ptr, ptr, ptr, i64, i64, i64, f32, f32, f32, f32]
         getattr(lib, f"lif_oracle_backward_{sfx}").restype = None
-    lib.lif_oracle_bn_forward_f32.argtypes = [ptr] * 8 + [i64] * 4 + [f32] * 3
-    lib.lif_oracle_bn_forward_f32.restype = None
-    lib.lif_oracle_bn_backward_f32.argtypes = [ptr] * 9 + [i64] * 4 + [f32] * 4
-    lib.lif_oracle_bn_backward_f32.restype = None
+        getattr(lib, f"lif_oracle_bn_forward_{sfx}").argtypes = [ptr] * 8 + [i64] * 4 + [f32] * 3
+        getattr(lib, f"lif_oracle_bn_forward_{sfx}").restype = None
+        getattr(lib, f"lif_oracle_bn_backward_{sfx}").argtypes = [ptr] * 9 + [i64] * 4 + [f32] * 4
+        getattr(lib, f"lif_oracle_bn_backward_{sfx}").restype = None
     _lib = lib
     return lib
 
@@ -101,28 +101,34 @@ def _bn_dims(a):
     return T, B, C, hw
 
 
-def _f32c(a):
-    return np.ascontiguousarray(a, dtype=np.float32)
+def _bn_real(x):
+    """dtype the batch-norm loops run in: float64 for float64 input, float32 otherwise."""
+    return np.float64 if np.asarray(x).dtype == np.float64 else np.float32
 
 
 def bn_fire_forward(x, weight, bias, var, mean, eps, alpha, thresh):
-    """Return ``(ivar, mem, spike)`` for fp32 ``x`` shaped ``[T, B, C, ...]`` and ``[C]`` parameters."""
-    x, weight, bias, var, mean = map(_f32c, (x, weight, bias, var, mean))
+    """Return ``(ivar, mem, spike)`` for fp32 or fp64 ``x`` shaped ``[T, B, C, ...]`` and ``[C]``
+    parameters (converted to the dtype of ``x``)."""
+    real = _bn_real(x)
+    x, weight, bias, var, mean = (np.ascontiguousarray(a, dtype=real) for a in (x, weight, bias, var, mean))
     T, B, C, hw = _bn_dims(x)
-    ivar = np.empty(C, dtype=np.float32)
+    ivar = np.empty(C, dtype=real)
     mem, spike = np.empty_like(x), np.empty_like(x)
-    _load().lif_oracle_bn_forward_f32(_p(x), _p(weight), _p(bias), _p(var), _p(mean), _p(ivar),
-                                      _p(mem), _p(spike), T, B, C, hw, eps, alpha, thresh)
+    fn = getattr(_load(), "lif_oracle_bn_forward_" + _suffix(x))
+    fn(_p(x), _p(weight), _p(bias), _p(var), _p(mean), _p(ivar), _p(mem), _p(spike), T, B, C, hw,
+       eps, alpha, thresh)
     return ivar, mem, spike
 
 
 def bn_fire_backward(x, weight, bias, ivar, mean, grad_spike, alpha, thresh, beta, interval):
     """Return ``(grad_x, grad_weight, grad_bias)``."""
-    x, weight, bias, ivar, mean, g = map(_f32c, (x, weight, bias, ivar, mean, grad_spike))
+    real = _bn_real(x)
+    x, weight, bias, ivar, mean, g = (np.ascontiguousarray(a, dtype=real)
+                                      for a in (x, weight, bias, ivar, mean, grad_spike))
     T, B, C, hw = _bn_dims(x)
     gx = np.empty_like(x)
-    gw, gb = np.empty(C, dtype=np.float32), np.empty(C, dtype=np.float32)
-    _load().lif_oracle_bn_backward_f32(_p(x), _p(weight), _p(bias), _p(ivar), _p(mean), _p(g),
-                                       _p(gx), _p(gw), _p(gb), T, B, C, hw, alpha, thresh, beta,
-                                       interval)
+    gw, gb = np.empty(C, dtype=real), np.empty(C, dtype=real)
+    fn = getattr(_load(), "lif_oracle_bn_backward_" + _suffix(x))
+    fn(_p(x), _p(weight), _p(bias), _p(ivar), _p(mean), _p(g), _p(gx), _p(gw), _p(gb), T, B, C, hw,
+       alpha, thresh, beta, interval)
     return gx, gw, gb

@@ -79,7 +79,7 @@ LIF_ORACLE_DEFINE(f32, float)
 LIF_ORACLE_DEFINE(f64, double)
 
 /*
- * Batch-norm + fire (fp32), following the reference's kernels:
+ * Batch-norm + fire (fp32 and fp64), following the reference's kernels:
  *   forward  : snnlib/cuda/snn_kernel_fp.cu:179-209 (bn_fire_s_fp_kernel; scale = weight / sqrt(var + eps),
  *              ivar = scale / weight)
  *   backward : snnlib/cuda/snn_kernel_bp.cu:448-478 (bn_fire_u_fp_kernel; scale = weight * ivar),
@@ -97,115 +97,122 @@ LIF_ORACLE_DEFINE(f64, double)
 #include <math.h>
 #include <stdlib.h>
 
-void lif_oracle_bn_forward_f32(const float* spatial, const float* weight, const float* bias,
-                               const float* var, const float* mean, float* ivar, float* mem,
-                               float* spike, int64_t T, int64_t B, int64_t C, int64_t HW,
-                               float eps_bn, float alpha, float thresh) {
-    const int64_t CHW = C * HW, step_stride = B * CHW;
-    for (int64_t i = 0; i < CHW; i++) {
-        const int64_t c = i / HW;
-        const float m = mean[c];
-        const float scale = weight[c] / sqrtf(var[c] + eps_bn);
-        const float shift = bias[c];
-        ivar[c] = scale / weight[c];
-        for (int64_t b = 0; b < B; b++) {
-            float potential = 0;
-            int fired = 0;
-            for (int64_t t = 0; t < T; t++) {
-                const int64_t at = t * step_stride + b * CHW + i;
-                potential = alpha * potential * (1 - fired) + (spatial[at] - m) * scale + shift;
-                fired = potential > thresh;
-                if (mem) mem[at] = potential;
-                if (spike) spike[at] = (float)fired;
-            }
-        }
-    }
-}
+#define LIF_ORACLE_BN_DEFINE(SUFFIX, REAL, WIDE, SQRT) \
+void lif_oracle_bn_forward_##SUFFIX(const REAL* spatial, const REAL* weight, const REAL* bias,                        \
+                               const REAL* var, const REAL* mean, REAL* ivar, REAL* mem,                              \
+                               REAL* spike, int64_t T, int64_t B, int64_t C, int64_t HW,                              \
+                               float eps_bn, float alpha, float thresh) {                                             \
+    const int64_t CHW = C * HW, step_stride = B * CHW;                                                                \
+    for (int64_t i = 0; i < CHW; i++) {                                                                               \
+        const int64_t c = i / HW;                                                                                     \
+        const REAL m = mean[c];                                                                                       \
+        const REAL scale = weight[c] / SQRT(var[c] + eps_bn);                                                         \
+        const REAL shift = bias[c];                                                                                   \
+        ivar[c] = scale / weight[c];                                                                                  \
+        for (int64_t b = 0; b < B; b++) {                                                                             \
+            REAL potential = 0;                                                                                       \
+            int fired = 0;                                                                                            \
+            for (int64_t t = 0; t < T; t++) {                                                                         \
+                const int64_t at = t * step_stride + b * CHW + i;                                                     \
+                potential = alpha * potential * (1 - fired) + (spatial[at] - m) * scale + shift;                      \
+                fired = potential > thresh;                                                                           \
+                if (mem) mem[at] = potential;                                                                         \
+                if (spike) spike[at] = (REAL)fired;                                                                   \
+            }                                                                                                         \
+        }                                                                                                             \
+    }                                                                                                                 \
+}                                                                                                                     \
+                                                                                                                      \
+void lif_oracle_bn_backward_##SUFFIX(const REAL* spatial, const REAL* weight, const REAL* bias,                       \
+                                const REAL* ivar, const REAL* mean, const REAL* grad_spike,                           \
+                                REAL* grad_spatial, REAL* grad_weight, REAL* grad_bias,                               \
+                                int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,                             \
+                                float thresh, float beta, float interval) {                                           \
+    const int64_t CHW = C * HW, step_stride = B * CHW;                                                                \
+    REAL* mem = (REAL*)malloc(sizeof(REAL) * (size_t)(T * step_stride));                                              \
+    REAL* p_xhat = (REAL*)malloc(sizeof(REAL) * (size_t)CHW);                                                         \
+    REAL* p_xhatx = (REAL*)malloc(sizeof(REAL) * (size_t)CHW);                                                        \
+    REAL* p_w = (REAL*)malloc(sizeof(REAL) * (size_t)CHW);                                                            \
+    REAL* p_b = (REAL*)malloc(sizeof(REAL) * (size_t)CHW);                                                            \
+                                                                                                                      \
+    /* recompute the membrane potential with scale = weight * ivar */                                                 \
+    for (int64_t i = 0; i < CHW; i++) {                                                                               \
+        const int64_t c = i / HW;                                                                                     \
+        const REAL m = mean[c], scale = weight[c] * ivar[c], shift = bias[c];                                         \
+        for (int64_t b = 0; b < B; b++) {                                                                             \
+            REAL potential = 0;                                                                                       \
+            int fired = 0;                                                                                            \
+            for (int64_t t = 0; t < T; t++) {                                                                         \
+                const int64_t at = t * step_stride + b * CHW + i;                                                     \
+                potential = alpha * potential * (1 - fired) + (spatial[at] - m) * scale + shift;                      \
+                fired = potential > thresh;                                                                           \
+                mem[at] = potential;                                                                                  \
+            }                                                                                                         \
+        }                                                                                                             \
+    }                                                                                                                 \
+    /* partial sums per (c, h, w) */                                                                                  \
+    for (int64_t i = 0; i < CHW; i++) {                                                                               \
+        const int64_t c = i / HW;                                                                                     \
+        const REAL m = mean[c], w = weight[c], iv = ivar[c];                                                          \
+        REAL sum_b = 0, sum_w = 0, sum_xhat = 0, sum_xhatx = 0;                                                       \
+        for (int64_t b = 0; b < B; b++) {                                                                             \
+            REAL carried = 0;                                                                                         \
+            for (int64_t t = T - 1; t >= 0; t--) {                                                                    \
+                const int64_t at = t * step_stride + b * CHW + i;                                                     \
+                const REAL u = mem[at];                                                                               \
+                REAL through_spike = 0;                                                                               \
+                if ((u - thresh) < interval && (thresh - u) < interval) {                                             \
+                    through_spike = grad_spike[at] - carried * alpha * u;                                             \
+                }                                                                                                     \
+                carried = through_spike * beta + carried * alpha * (u <= thresh);                                     \
+                const REAL x_bn = (spatial[at] - m) * iv;                                                             \
+                sum_b += carried;                                                                                     \
+                sum_w += carried * x_bn;                                                                              \
+                sum_xhat += carried * w;                                                                              \
+                sum_xhatx += carried * w * x_bn;                                                                      \
+            }                                                                                                         \
+        }                                                                                                             \
+        p_b[i] = sum_b;                                                                                               \
+        p_w[i] = sum_w;                                                                                               \
+        p_xhat[i] = sum_xhat / (T * B);                                                                               \
+        p_xhatx[i] = sum_xhatx / (T * B);                                                                             \
+    }                                                                                                                 \
+    /* reduce over the spatial positions of each channel; then the input gradient */                                  \
+    for (int64_t c = 0; c < C; c++) {                                                                                 \
+        WIDE acc_b = 0, acc_w = 0, acc_xhat = 0, acc_xhatx = 0;                                                       \
+        for (int64_t k = 0; k < HW; k++) {                                                                            \
+            acc_b += p_b[c * HW + k];                                                                                 \
+            acc_w += p_w[c * HW + k];                                                                                 \
+            acc_xhat += p_xhat[c * HW + k];                                                                           \
+            acc_xhatx += p_xhatx[c * HW + k];                                                                         \
+        }                                                                                                             \
+        grad_bias[c] = (REAL)acc_b;                                                                                   \
+        grad_weight[c] = (REAL)acc_w;                                                                                 \
+        const REAL g_xhat = (REAL)(acc_xhat / (WIDE)HW);                                                              \
+        const REAL g_xhatx = (REAL)(acc_xhatx / (WIDE)HW);                                                            \
+        const REAL m = mean[c], w = weight[c], iv = ivar[c];                                                          \
+        for (int64_t k = 0; k < HW; k++) {                                                                            \
+            const int64_t i = c * HW + k;                                                                             \
+            for (int64_t b = 0; b < B; b++) {                                                                         \
+                REAL carried = 0;                                                                                     \
+                for (int64_t t = T - 1; t >= 0; t--) {                                                                \
+                    const int64_t at = t * step_stride + b * CHW + i;                                                 \
+                    const REAL u = mem[at];                                                                           \
+                    REAL through_spike = 0;                                                                           \
+                    if ((u - thresh) < interval && (thresh - u) < interval) {                                         \
+                        through_spike = grad_spike[at] - carried * alpha * u;                                         \
+                    }                                                                                                 \
+                    carried = through_spike * beta + carried * alpha * (u <= thresh);                                 \
+                    grad_spatial[at] = carried * w * iv - iv * ((spatial[at] - m) * iv * g_xhatx + g_xhat);           \
+                }                                                                                                     \
+            }                                                                                                         \
+        }                                                                                                             \
+    }                                                                                                                 \
+    free(mem); free(p_xhat); free(p_xhatx); free(p_w); free(p_b);                                                     \
+}                                                                                                                     
 
-void lif_oracle_bn_backward_f32(const float* spatial, const float* weight, const float* bias,
-                                const float* ivar, const float* mean, const float* grad_spike,
-                                float* grad_spatial, float* grad_weight, float* grad_bias,
-                                int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
-                                float thresh, float beta, float interval) {
-    const int64_t CHW = C * HW, step_stride = B * CHW;
-    float* mem = (float*)malloc(sizeof(float) * (size_t)(T * step_stride));
-    float* p_xhat = (float*)malloc(sizeof(float) * (size_t)CHW);
-    float* p_xhatx = (float*)malloc(sizeof(float) * (size_t)CHW);
-    float* p_w = (float*)malloc(sizeof(float) * (size_t)CHW);
-    float* p_b = (float*)malloc(sizeof(float) * (size_t)CHW);
-
-    /* recompute the membrane potential with scale = weight * ivar */
-    for (int64_t i = 0; i < CHW; i++) {
-        const int64_t c = i / HW;
-        const float m = mean[c], scale = weight[c] * ivar[c], shift = bias[c];
-        for (int64_t b = 0; b < B; b++) {
-            float potential = 0;
-            int fired = 0;
-            for (int64_t t = 0; t < T; t++) {
-                const int64_t at = t * step_stride + b * CHW + i;
-                potential = alpha * potential * (1 - fired) + (spatial[at] - m) * scale + shift;
-                fired = potential > thresh;
-                mem[at] = potential;
-            }
-        }
-    }
-    /* partial sums per (c, h, w) */
-    for (int64_t i = 0; i < CHW; i++) {
-        const int64_t c = i / HW;
-        const float m = mean[c], w = weight[c], iv = ivar[c];
-        float sum_b = 0, sum_w = 0, sum_xhat = 0, sum_xhatx = 0;
-        for (int64_t b = 0; b < B; b++) {
-            float carried = 0;
-            for (int64_t t = T - 1; t >= 0; t--) {
-                const int64_t at = t * step_stride + b * CHW + i;
-                const float u = mem[at];
-                float through_spike = 0;
-                if ((u - thresh) < interval && (thresh - u) < interval) {
-                    through_spike = grad_spike[at] - carried * alpha * u;
-                }
-                carried = through_spike * beta + carried * alpha * (u <= thresh);
-                const float x_bn = (spatial[at] - m) * iv;
-                sum_b += carried;
-                sum_w += carried * x_bn;
-                sum_xhat += carried * w;
-                sum_xhatx += carried * w * x_bn;
-            }
-        }
-        p_b[i] = sum_b;
-        p_w[i] = sum_w;
-        p_xhat[i] = sum_xhat / (T * B);
-        p_xhatx[i] = sum_xhatx / (T * B);
-    }
-    /* reduce over the spatial positions of each channel; then the input gradient */
-    for (int64_t c = 0; c < C; c++) {
-        double acc_b = 0, acc_w = 0, acc_xhat = 0, acc_xhatx = 0;
-        for (int64_t k = 0; k < HW; k++) {
-            acc_b += p_b[c * HW + k];
-            acc_w += p_w[c * HW + k];
-            acc_xhat += p_xhat[c * HW + k];
-            acc_xhatx += p_xhatx[c * HW + k];
-        }
-        grad_bias[c] = (float)acc_b;
-        grad_weight[c] = (float)acc_w;
-        const float g_xhat = (float)(acc_xhat / (double)HW);
-        const float g_xhatx = (float)(acc_xhatx / (double)HW);
-        const float m = mean[c], w = weight[c], iv = ivar[c];
-        for (int64_t k = 0; k < HW; k++) {
-            const int64_t i = c * HW + k;
-            for (int64_t b = 0; b < B; b++) {
-                float carried = 0;
-                for (int64_t t = T - 1; t >= 0; t--) {
-                    const int64_t at = t * step_stride + b * CHW + i;
-                    const float u = mem[at];
-                    float through_spike = 0;
-                    if ((u - thresh) < interval && (thresh - u) < interval) {
-                        through_spike = grad_spike[at] - carried * alpha * u;
-                    }
-                    carried = through_spike * beta + carried * alpha * (u <= thresh);
-                    grad_spatial[at] = carried * w * iv - iv * ((spatial[at] - m) * iv * g_xhatx + g_xhat);
-                }
-            }
-        }
-    }
-    free(mem); free(p_xhat); free(p_xhatx); free(p_w); free(p_b);
-}
+/* fp32 as the reference trains; fp64 with the same loops in double (the reference's double dispatch keeps
+ * the per-channel statistics in float temporaries, snnlib/cuda/snn_kernel_bp.cu:563; this restatement and
+ * the device code do not narrow them).  Sums across positions: one precision up, rounded once. */
+LIF_ORACLE_BN_DEFINE(f32, float, double, sqrtf)
+LIF_ORACLE_BN_DEFINE(f64, double, long double, sqrt)

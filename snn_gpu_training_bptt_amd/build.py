@@ -5,7 +5,7 @@ be put on ``sys.path`` to make ``import snnlib`` work for reference-style code):
 
 * ``libsnnlif_gfx950.so`` -- HIP kernels + C ABI (``csrc/lif_kernels.h`` instantiated by
   ``csrc/lif_f32.hip``, ``lif_f64.hip``, ``lif_bf16.hip``, and ``csrc/lif_bn_kernels.h`` by
-  ``lif_bn_f32.hip``; entry points in ``csrc/lif_abi.hip``,
+  ``lif_bn_f32.hip``, ``lif_bn_f64.hip``; entry points in ``csrc/lif_abi.hip``,
   declared in ``include/snnlib_lif.h``), compiled by hipcc for gfx950 only;
 * ``snnlib.so``           -- the Python extension module ``snnlib`` (``csrc/snnlib_ext.cpp``), host
   C++ against PyTorch-ROCm's headers, linked to the library above through ``$ORIGIN``.
@@ -36,7 +36,8 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
-KERNEL_SOURCES = ["lif_abi.hip", "lif_f32.hip", "lif_f64.hip", "lif_bf16.hip", "lif_bn_f32.hip"]
+KERNEL_SOURCES = ["lif_abi.hip", "lif_f32.hip", "lif_f64.hip", "lif_bf16.hip", "lif_bn_f32.hip",
+                  "lif_bn_f64.hip"]
 
 
 def _run(cmd, verbose):

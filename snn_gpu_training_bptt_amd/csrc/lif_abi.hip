@@ -46,7 +46,7 @@ const char* snnlif_strerror(int code) {
         case SNNLIF_ERR_DTYPE: return "snnlif: unsupported dtype (expected SNNLIF_DTYPE_F32, _F64 or _BF16)";
         case SNNLIF_ERR_WORKSPACE: return "snnlif: workspace missing or smaller than snnlif_fire_bp_workspace_bytes()";
         case SNNLIF_ERR_ALIGN: return "snnlif: pointer not aligned to its element size (workspace: 16 bytes)";
-        case SNNLIF_ERR_UNSUPPORTED: return "snnlif: not implemented for these arguments (batch-norm fire: fp32 only, backward T <= 1024)";
+        case SNNLIF_ERR_UNSUPPORTED: return "snnlif: not implemented for these arguments (batch-norm fire: fp32 / fp64 only, backward T <= 1024)";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -117,49 +117,106 @@ inline int bn_shape_error(int64_t T, int64_t B, int64_t C, int64_t HW) {
 
 }  // namespace
 
+// The batch-norm entry points take float or double storage (bf16: SNNLIF_ERR_UNSUPPORTED).
+// Returns the element size, or 0 with *rc set to the error.
+static size_t bn_element_size(int dtype, int* rc) {
+    if (arith_size(dtype) == 0) {
+        *rc = SNNLIF_ERR_DTYPE;
+        return 0;
+    }
+    if (dtype == SNNLIF_DTYPE_F32) return sizeof(float);
+    if (dtype == SNNLIF_DTYPE_F64) return sizeof(double);
+    *rc = SNNLIF_ERR_UNSUPPORTED;
+    return 0;
+}
+
+static bool all_aligned(const void* const* ptrs, int n, size_t bytes) {
+    for (int i = 0; i < n; ++i)
+        if (!snnlif::aligned_to(ptrs[i], bytes)) return false;
+    return true;
+}
+
+// Calls the f32 or the f64 instantiation of a launcher with typed pointers.
+#define SNNLIF_BN_DISPATCH(es, CALL_F32, CALL_F64) ((es) == sizeof(float) ? (CALL_F32) : (CALL_F64))
+#define CF(p) static_cast<const float*>(p)
+#define MF(p) static_cast<float*>(p)
+#define CD(p) static_cast<const double*>(p)
+#define MD(p) static_cast<double*>(p)
+
 int snnlif_bn_fire_s_fp(const void* spatial, const void* weight, const void* bias, const void* var,
                         const void* mean, void* ivar, void* spike, int dtype, int64_t T, int64_t B,
                         int64_t C, int64_t HW, float eps, float alpha, float thresh, void* stream) {
-    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
-    if (dtype != SNNLIF_DTYPE_F32) return SNNLIF_ERR_UNSUPPORTED;
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
     const int se = bn_shape_error(T, B, C, HW);
     if (se != SNNLIF_OK) return se;
     if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
     if (!spatial || !weight || !bias || !var || !mean || !ivar || !spike) return SNNLIF_ERR_ARG;
     const void* ptrs[7] = {spatial, weight, bias, var, mean, ivar, spike};
-    for (const void* p : ptrs)
-        if (!snnlif::aligned_to(p, sizeof(float))) return SNNLIF_ERR_ALIGN;
-    return snnlif::bn_forward_f32(
-        static_cast<const float*>(spatial), static_cast<const float*>(weight),
-        static_cast<const float*>(bias), static_cast<const float*>(var),
-        static_cast<const float*>(mean), static_cast<float*>(ivar), static_cast<float*>(spike),
-        /*from_ivar=*/false, T, B, C, HW, eps, alpha, thresh, static_cast<hipStream_t>(stream));
+    if (!all_aligned(ptrs, 7, es)) return SNNLIF_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_forward_f32(CF(spatial), CF(weight), CF(bias), CF(var), CF(mean), MF(ivar),
+                               MF(spike), /*from_ivar=*/false, T, B, C, HW, eps, alpha, thresh, st),
+        snnlif::bn_forward_f64(CD(spatial), CD(weight), CD(bias), CD(var), CD(mean), MD(ivar),
+                               MD(spike), /*from_ivar=*/false, T, B, C, HW, eps, alpha, thresh, st));
 }
 
 int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const void* bias,
                                const void* ivar, const void* mean, void* spike, int dtype, int64_t T,
                                int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
                                void* stream) {
-    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
-    if (dtype != SNNLIF_DTYPE_F32) return SNNLIF_ERR_UNSUPPORTED;
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
     const int se = bn_shape_error(T, B, C, HW);
     if (se != SNNLIF_OK) return se;
     if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
     if (!spatial || !weight || !bias || !ivar || !mean || !spike) return SNNLIF_ERR_ARG;
     const void* ptrs[6] = {spatial, weight, bias, ivar, mean, spike};
-    for (const void* p : ptrs)
-        if (!snnlif::aligned_to(p, sizeof(float))) return SNNLIF_ERR_ALIGN;
-    return snnlif::bn_forward_f32(
-        static_cast<const float*>(spatial), static_cast<const float*>(weight),
-        static_cast<const float*>(bias), static_cast<const float*>(ivar),
-        static_cast<const float*>(mean), nullptr, static_cast<float*>(spike), /*from_ivar=*/true, T,
-        B, C, HW, 0.f, alpha, thresh, static_cast<hipStream_t>(stream));
+    if (!all_aligned(ptrs, 6, es)) return SNNLIF_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_forward_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean), nullptr,
+                               MF(spike), /*from_ivar=*/true, T, B, C, HW, 0.f, alpha, thresh, st),
+        snnlif::bn_forward_f64(CD(spatial), CD(weight), CD(bias), CD(ivar), CD(mean), nullptr,
+                               MD(spike), /*from_ivar=*/true, T, B, C, HW, 0.f, alpha, thresh, st));
 }
 
 size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW) {
-    if (dtype != SNNLIF_DTYPE_F32 || bn_shape_error(T, B, C, HW) != SNNLIF_OK) return 0;
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0 || bn_shape_error(T, B, C, HW) != SNNLIF_OK) return 0;
     if (T == 0 || B * C * HW == 0) return 0;
-    return snnlif::bn_backward_workspace_floats(B, C, HW) * sizeof(float);
+    return snnlif::bn_backward_workspace_elems(B, C, HW) * es;
+}
+
+// Shared argument checks of the three backward entry points; `needs_workspace` = sweep 1 runs.
+static int bn_backward_checks(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW,
+                              const void* const* ptrs, int n, bool needs_workspace,
+                              const void* workspace, size_t workspace_bytes, size_t* es_out,
+                              bool* empty) {
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    *es_out = es;
+    *empty = (T == 0 || B * C * HW == 0);
+    if (*empty) return SNNLIF_OK;
+    if (T > SNNLIF_BP_NO_WORKSPACE_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
+    for (int i = 0; i < n; ++i)
+        if (ptrs[i] == nullptr) return SNNLIF_ERR_ARG;
+    if (!all_aligned(ptrs, n, es)) return SNNLIF_ERR_ALIGN;
+    if (needs_workspace) {
+        const size_t need = snnlif::bn_backward_workspace_elems(B, C, HW) * es;
+        if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
+        if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
+    }
+    return SNNLIF_OK;
 }
 
 int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias, const void* ivar,
@@ -167,28 +224,22 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
                       void* grad_weight, void* grad_bias, int dtype, int64_t T, int64_t B, int64_t C,
                       int64_t HW, float alpha, float thresh, float beta, float interval,
                       void* workspace, size_t workspace_bytes, void* stream) {
-    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
-    if (dtype != SNNLIF_DTYPE_F32) return SNNLIF_ERR_UNSUPPORTED;
-    const int se = bn_shape_error(T, B, C, HW);
-    if (se != SNNLIF_OK) return se;
-    if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
-    if (T > SNNLIF_BP_NO_WORKSPACE_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
-    if (!spatial || !weight || !bias || !ivar || !mean || !grad_spike || !grad_spatial ||
-        !grad_weight || !grad_bias)
-        return SNNLIF_ERR_ARG;
-    const void* ptrs[9] = {spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight, grad_bias};
-    for (const void* p : ptrs)
-        if (!snnlif::aligned_to(p, sizeof(float))) return SNNLIF_ERR_ALIGN;
-    const size_t need = snnlif::bn_backward_workspace_floats(B, C, HW) * sizeof(float);
-    if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
-    if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
-    return snnlif::bn_backward_f32(
-        static_cast<const float*>(spatial), static_cast<const float*>(weight),
-        static_cast<const float*>(bias), static_cast<const float*>(ivar),
-        static_cast<const float*>(mean), static_cast<const float*>(grad_spike),
-        static_cast<float*>(grad_spatial), static_cast<float*>(grad_weight),
-        static_cast<float*>(grad_bias), T, B, C, HW, alpha, thresh, beta, interval,
-        static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
+    const void* ptrs[9] = {spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
+                           grad_bias};
+    size_t es = 0;
+    bool empty = false;
+    const int rc = bn_backward_checks(dtype, T, B, C, HW, ptrs, 9, true, workspace, workspace_bytes,
+                                      &es, &empty);
+    if (rc != SNNLIF_OK || empty) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_backward_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean), CF(grad_spike),
+                                MF(grad_spatial), MF(grad_weight), MF(grad_bias), T, B, C, HW, alpha,
+                                thresh, beta, interval, MF(workspace), st),
+        snnlif::bn_backward_f64(CD(spatial), CD(weight), CD(bias), CD(ivar), CD(mean), CD(grad_spike),
+                                MD(grad_spatial), MD(grad_weight), MD(grad_bias), T, B, C, HW, alpha,
+                                thresh, beta, interval, MD(workspace), st));
 }
 
 int snnlif_bn_fire_bp_dist1(const void* spatial, const void* weight, const void* bias,
@@ -197,30 +248,25 @@ int snnlif_bn_fire_bp_dist1(const void* spatial, const void* weight, const void*
                             int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
                             float thresh, float beta, float interval, void* workspace,
                             size_t workspace_bytes, void* stream) {
-    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
-    if (dtype != SNNLIF_DTYPE_F32) return SNNLIF_ERR_UNSUPPORTED;
-    const int se = bn_shape_error(T, B, C, HW);
-    if (se != SNNLIF_OK) return se;
-    // an empty batch has no statistics to report: the channel arrays are left untouched
-    if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
-    if (T > SNNLIF_BP_NO_WORKSPACE_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
-    if (!spatial || !weight || !bias || !ivar || !mean || !grad_spike || !mean_gxhat ||
-        !mean_gxhatx || !grad_weight || !grad_bias)
-        return SNNLIF_ERR_ARG;
     const void* ptrs[10] = {spatial, weight, bias, ivar, mean, grad_spike, mean_gxhat, mean_gxhatx,
                             grad_weight, grad_bias};
-    for (const void* p : ptrs)
-        if (!snnlif::aligned_to(p, sizeof(float))) return SNNLIF_ERR_ALIGN;
-    const size_t need = snnlif::bn_backward_workspace_floats(B, C, HW) * sizeof(float);
-    if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
-    if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
-    return snnlif::bn_backward_stats_f32(
-        static_cast<const float*>(spatial), static_cast<const float*>(weight),
-        static_cast<const float*>(bias), static_cast<const float*>(ivar),
-        static_cast<const float*>(mean), static_cast<const float*>(grad_spike),
-        static_cast<float*>(grad_weight), static_cast<float*>(grad_bias),
-        static_cast<float*>(mean_gxhat), static_cast<float*>(mean_gxhatx), T, B, C, HW, alpha,
-        thresh, beta, interval, static_cast<float*>(workspace), static_cast<hipStream_t>(stream));
+    size_t es = 0;
+    bool empty = false;
+    // an empty batch has no statistics to report: the channel arrays are left untouched
+    const int rc = bn_backward_checks(dtype, T, B, C, HW, ptrs, 10, true, workspace,
+                                      workspace_bytes, &es, &empty);
+    if (rc != SNNLIF_OK || empty) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_backward_stats_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean),
+                                      CF(grad_spike), MF(grad_weight), MF(grad_bias), MF(mean_gxhat),
+                                      MF(mean_gxhatx), T, B, C, HW, alpha, thresh, beta, interval,
+                                      MF(workspace), st),
+        snnlif::bn_backward_stats_f64(CD(spatial), CD(weight), CD(bias), CD(ivar), CD(mean),
+                                      CD(grad_spike), MD(grad_weight), MD(grad_bias), MD(mean_gxhat),
+                                      MD(mean_gxhatx), T, B, C, HW, alpha, thresh, beta, interval,
+                                      MD(workspace), st));
 }
 
 int snnlif_bn_fire_bp_dist2(const void* spatial, const void* weight, const void* bias,
@@ -228,26 +274,27 @@ int snnlif_bn_fire_bp_dist2(const void* spatial, const void* weight, const void*
                             const void* grad_xhat, const void* grad_xhatx, void* grad_spatial,
                             int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
                             float thresh, float beta, float interval, void* stream) {
-    if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
-    if (dtype != SNNLIF_DTYPE_F32) return SNNLIF_ERR_UNSUPPORTED;
-    const int se = bn_shape_error(T, B, C, HW);
-    if (se != SNNLIF_OK) return se;
-    if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
-    if (T > SNNLIF_BP_NO_WORKSPACE_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
-    if (!spatial || !weight || !bias || !ivar || !mean || !grad_spike || !grad_xhat || !grad_xhatx ||
-        !grad_spatial)
-        return SNNLIF_ERR_ARG;
     const void* ptrs[9] = {spatial, weight, bias, ivar, mean, grad_spike, grad_xhat, grad_xhatx,
                            grad_spatial};
-    for (const void* p : ptrs)
-        if (!snnlif::aligned_to(p, sizeof(float))) return SNNLIF_ERR_ALIGN;
-    return snnlif::bn_backward_input_f32(
-        static_cast<const float*>(spatial), static_cast<const float*>(weight),
-        static_cast<const float*>(bias), static_cast<const float*>(ivar),
-        static_cast<const float*>(mean), static_cast<const float*>(grad_spike),
-        static_cast<const float*>(grad_xhat), static_cast<const float*>(grad_xhatx),
-        static_cast<float*>(grad_spatial), T, B, C, HW, alpha, thresh, beta, interval,
-        static_cast<hipStream_t>(stream));
+    size_t es = 0;
+    bool empty = false;
+    const int rc = bn_backward_checks(dtype, T, B, C, HW, ptrs, 9, false, nullptr, 0, &es, &empty);
+    if (rc != SNNLIF_OK || empty) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_backward_input_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean),
+                                      CF(grad_spike), CF(grad_xhat), CF(grad_xhatx), MF(grad_spatial),
+                                      T, B, C, HW, alpha, thresh, beta, interval, st),
+        snnlif::bn_backward_input_f64(CD(spatial), CD(weight), CD(bias), CD(ivar), CD(mean),
+                                      CD(grad_spike), CD(grad_xhat), CD(grad_xhatx), MD(grad_spatial),
+                                      T, B, C, HW, alpha, thresh, beta, interval, st));
 }
+
+#undef SNNLIF_BN_DISPATCH
+#undef CF
+#undef MF
+#undef CD
+#undef MD
 
 }  // extern "C"

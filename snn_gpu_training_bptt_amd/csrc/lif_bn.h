@@ -1,5 +1,5 @@
-// Host-side interface of the batch-norm + fire kernels (lif_bn_kernels.h, lif_bn_f32.hip), shared
-// with the C ABI in lif_abi.hip.
+// Host-side interface of the batch-norm + fire kernels (lif_bn_kernels.h, lif_bn_launch.h, instantiated
+// for float in lif_bn_f32.hip and for double in lif_bn_f64.hip), shared with the C ABI in lif_abi.hip.
 #ifndef SNNLIF_LIF_BN_H
 #define SNNLIF_LIF_BN_H
 
@@ -20,40 +20,45 @@ inline int bn_reduce_splits(int64_t B, int64_t C) {
     return static_cast<int>(s);
 }
 
-// floats: part_gy[N], part_gyx[N], split[2*S*C], coef[2*C]
-inline size_t bn_backward_workspace_floats(int64_t B, int64_t C, int64_t HW) {
+// Workspace of the backward in elements of the scalar type:
+// part_gy[N], part_gyx[N], split[2*S*C], coef[2*C].
+inline size_t bn_backward_workspace_elems(int64_t B, int64_t C, int64_t HW) {
     const int S = bn_reduce_splits(B, C);
     return static_cast<size_t>(2 * B * C * HW) + static_cast<size_t>(2) * S * C +
            static_cast<size_t>(2 * C);
 }
 
-// from_ivar = false: stat is the variance and ivar is written; true: stat is the inverse standard
-// deviation and ivar is not touched.
-int bn_forward_f32(const float* x, const float* weight, const float* bias, const float* stat,
-                   const float* mean, float* ivar, float* spike, bool from_ivar, int64_t T,
-                   int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,
-                   hipStream_t stream);
+// Per scalar type F (suffix f32 = float, f64 = double):
+//   bn_forward_*         from_ivar = false: stat is the variance and ivar is written; true: stat is
+//                        the inverse standard deviation and ivar is not touched.
+//   bn_backward_stats_*  sweep 1 + channel reduction: parameter gradients and the two per-channel
+//                        means (what a batch sharded over several GPUs runs before its all-reduce);
+//   bn_backward_input_*  sweep 2: the input gradient from those means (after the all-reduce);
+//   bn_backward_*        the two back to back, the means staged at the end of the workspace.
+#define SNNLIF_DECLARE_BN_DTYPE(SUFFIX, F)                                                         \
+    int bn_forward_##SUFFIX(const F* x, const F* weight, const F* bias, const F* stat,             \
+                            const F* mean, F* ivar, F* spike, bool from_ivar, int64_t T,           \
+                            int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,\
+                            hipStream_t stream);                                                   \
+    int bn_backward_stats_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,      \
+                                   const F* mean, const F* g, F* grad_weight, F* grad_bias,        \
+                                   F* mean_gxhat, F* mean_gxhatx, int64_t T, int64_t B, int64_t C, \
+                                   int64_t HW, float alpha, float thresh, float beta,              \
+                                   float interval, F* workspace, hipStream_t stream);              \
+    int bn_backward_input_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,      \
+                                   const F* mean, const F* g, const F* mean_gxhat,                 \
+                                   const F* mean_gxhatx, F* gx, int64_t T, int64_t B, int64_t C,   \
+                                   int64_t HW, float alpha, float thresh, float beta,              \
+                                   float interval, hipStream_t stream);                            \
+    int bn_backward_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,            \
+                             const F* mean, const F* g, F* gx, F* grad_weight, F* grad_bias,       \
+                             int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,             \
+                             float thresh, float beta, float interval, F* workspace,               \
+                             hipStream_t stream);
 
-// The backward in its two halves (what a batch sharded over several GPUs runs on either side of the
-// all-reduce of the two per-channel means): sweep 1 + channel reduction, then sweep 2.
-// bn_backward_f32 is the two back to back.
-int bn_backward_stats_f32(const float* x, const float* weight, const float* bias, const float* ivar,
-                          const float* mean, const float* g, float* grad_weight, float* grad_bias,
-                          float* mean_gxhat, float* mean_gxhatx, int64_t T, int64_t B, int64_t C,
-                          int64_t HW, float alpha, float thresh, float beta, float interval,
-                          float* workspace, hipStream_t stream);
-
-int bn_backward_input_f32(const float* x, const float* weight, const float* bias, const float* ivar,
-                          const float* mean, const float* g, const float* mean_gxhat,
-                          const float* mean_gxhatx, float* gx, int64_t T, int64_t B, int64_t C,
-                          int64_t HW, float alpha, float thresh, float beta, float interval,
-                          hipStream_t stream);
-
-int bn_backward_f32(const float* x, const float* weight, const float* bias, const float* ivar,
-                    const float* mean, const float* g, float* gx, float* grad_weight,
-                    float* grad_bias, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
-                    float thresh, float beta, float interval, float* workspace,
-                    hipStream_t stream);
+SNNLIF_DECLARE_BN_DTYPE(f32, float)
+SNNLIF_DECLARE_BN_DTYPE(f64, double)
+#undef SNNLIF_DECLARE_BN_DTYPE
 
 }  // namespace snnlif
 

@@ -1,4 +1,4 @@
-// Batch-norm + LIF fire kernels (fp32) for MI355X: the per-channel affine of a batch norm is
+// Batch-norm + LIF fire kernels (F = float or double; one neuron per lane) for MI355X: the per-channel affine of a batch norm is
 // applied to the input current inside the fire recurrence, forward and backward.
 //
 // Reference: snnlib/cuda/snn_kernel_fp.cu:157-240 (bn_fire_s_fp_kernel + launcher) and
@@ -41,6 +41,10 @@ namespace snnlif {
 
 constexpr int kReduceBlock = 256;
 
+__device__ __forceinline__ float real_sqrt(float v) { return sqrtf(v); }
+__device__ __forceinline__ double real_sqrt(double v) { return sqrt(v); }
+
+
 // Channel of a neuron column in a [B, C, HW] neuron axis.
 __device__ __forceinline__ int channel_of(int64_t col, int64_t C, int64_t HW, bool small) {
     if (small) {  // everything fits 32 bits: cheap unsigned division
@@ -57,31 +61,31 @@ __device__ __forceinline__ int channel_of(int64_t col, int64_t C, int64_t HW, bo
 // published (how the backward of the fused layers recomputes the spikes, as the reference's
 // bn_fire_us_fp_kernel does, snnlib/cuda/snn_kernel_bp.cu:481-530).
 // ---------------------------------------------------------------------------------------------
-template <int TC, bool MULTI, bool FROM_IVAR>
+template <typename F, int TC, bool MULTI, bool FROM_IVAR>
 __global__ void __launch_bounds__(kFwdBlock)
-lif_bn_forward_kernel(const float* __restrict__ x, const float* __restrict__ weight,
-                      const float* __restrict__ bias, const float* __restrict__ stat,
-                      const float* __restrict__ mean, float* __restrict__ ivar,
-                      float* __restrict__ spike, int T, int64_t N, int64_t C, int64_t HW, float eps,
-                      float alpha, float thresh) {
+lif_bn_forward_kernel(const F* __restrict__ x, const F* __restrict__ weight,
+                      const F* __restrict__ bias, const F* __restrict__ stat,
+                      const F* __restrict__ mean, F* __restrict__ ivar,
+                      F* __restrict__ spike, int T, int64_t N, int64_t C, int64_t HW, F eps,
+                      F alpha, F thresh) {
     const bool small = N <= 0xffffffffll;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t col = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; col < N;
          col += stride) {
         const int c = channel_of(col, C, HW, small);
-        const float m = mean[c];
-        const float wgt = weight[c];
-        const float scale = FROM_IVAR ? wgt * stat[c] : wgt / sqrtf(stat[c] + eps);
-        const float b = bias[c];
+        const F m = mean[c];
+        const F wgt = weight[c];
+        const F scale = FROM_IVAR ? wgt * stat[c] : wgt / real_sqrt(stat[c] + eps);
+        const F b = bias[c];
         // first neuron of the channel in batch entry 0 publishes the channel's ivar
         if (!FROM_IVAR && col == static_cast<int64_t>(c) * HW) ivar[c] = scale / wgt;
 
-        float u = 0.f, s = 0.f;
-        Pack<float, 1> cur[TC];
-        Pack<float, 1> nxt[MULTI ? TC : 1];
+        F u = F(0), s = F(0);
+        Pack<F, 1> cur[TC];
+        Pack<F, 1> nxt[MULTI ? TC : 1];
 #pragma unroll
         for (int k = 0; k < TC; ++k) {
-            if (k < T) cur[k] = load_pack<float, 1, false>(x + static_cast<int64_t>(k) * N + col);
+            if (k < T) cur[k] = load_pack<F, 1, false>(x + static_cast<int64_t>(k) * N + col);
         }
         for (int t0 = 0; t0 < T; t0 += TC) {
             if (MULTI && t0 + TC < T) {
@@ -90,18 +94,18 @@ lif_bn_forward_kernel(const float* __restrict__ x, const float* __restrict__ wei
                     const int t = t0 + TC + k;
                     if (t < T)
                         nxt[MULTI ? k : 0] =
-                            load_pack<float, 1, false>(x + static_cast<int64_t>(t) * N + col);
+                            load_pack<F, 1, false>(x + static_cast<int64_t>(t) * N + col);
                 }
             }
 #pragma unroll
             for (int k = 0; k < TC; ++k) {
                 const int t = t0 + k;
                 if (t < T) {
-                    u = (alpha * u) * (1.f - s) + (cur[k].e[0] - m) * scale + b;
-                    s = (u > thresh) ? 1.f : 0.f;
-                    Pack<float, 1> so;
+                    u = (alpha * u) * (F(1) - s) + (cur[k].e[0] - m) * scale + b;
+                    s = (u > thresh) ? F(1) : F(0);
+                    Pack<F, 1> so;
                     so.e[0] = s;
-                    store_pack<float, 1>(spike + static_cast<int64_t>(t) * N + col, so);
+                    store_pack<F, 1>(spike + static_cast<int64_t>(t) * N + col, so);
                 }
             }
             if (!MULTI) break;
@@ -120,50 +124,50 @@ lif_bn_forward_kernel(const float* __restrict__ x, const float* __restrict__ wei
 // after it.  Calls emit(t, gy, x_t) for t = rows-1 .. 0 (t counts from the window's first row).  On
 // exit uc / sc are the state after the window and gu the gradient at its first step.
 // ---------------------------------------------------------------------------------------------
-template <int TW, bool EXACT, typename Emit>
-__device__ __forceinline__ void bn_reverse_window(const float* __restrict__ x,
-                                                  const float* __restrict__ g, int rows, int64_t N,
-                                                  int64_t col, float m, float scale, float b,
-                                                  float& uc, float& sc, float& gu, float alpha,
-                                                  float thresh, float beta, float interval,
+template <typename F, int TW, bool EXACT, typename Emit>
+__device__ __forceinline__ void bn_reverse_window(const F* __restrict__ x,
+                                                  const F* __restrict__ g, int rows, int64_t N,
+                                                  int64_t col, F m, F scale, F b,
+                                                  F& uc, F& sc, F& gu, F alpha,
+                                                  F thresh, F beta, F interval,
                                                   Emit&& emit) {
-    float xin[TW], gin[TW], u[TW];
+    F xin[TW], gin[TW], u[TW];
 #pragma unroll
     for (int t = 0; t < TW; ++t) {
-        xin[t] = 0.f;
+        xin[t] = F(0);
         if (EXACT || t < rows)
-            xin[t] = load_pack<float, 1, false>(x + static_cast<int64_t>(t) * N + col).e[0];
+            xin[t] = load_pack<F, 1, false>(x + static_cast<int64_t>(t) * N + col).e[0];
     }
 #pragma unroll
     for (int t = TW - 1; t >= 0; --t) {
-        gin[t] = 0.f;
+        gin[t] = F(0);
         if (EXACT || t < rows)
-            gin[t] = load_pack<float, 1, true>(g + static_cast<int64_t>(t) * N + col).e[0];
+            gin[t] = load_pack<F, 1, true>(g + static_cast<int64_t>(t) * N + col).e[0];
     }
 #pragma unroll
     for (int t = 0; t < TW; ++t) {
-        uc = (alpha * uc) * (1.f - sc) + (xin[t] - m) * scale + b;
-        sc = (uc > thresh) ? 1.f : 0.f;
+        uc = (alpha * uc) * (F(1) - sc) + (xin[t] - m) * scale + b;
+        sc = (uc > thresh) ? F(1) : F(0);
         u[t] = uc;
     }
 #pragma unroll
     for (int t = TW - 1; t >= 0; --t) {
         if (EXACT || t < rows) {
-            lif_reverse_step<float>(gu, u[t], gin[t], alpha, thresh, beta, interval);
+            lif_reverse_step<F>(gu, u[t], gin[t], alpha, thresh, beta, interval);
             emit(t, gu, xin[t]);
         }
     }
 }
 
 // The whole time axis as one window (T <= TW).
-template <int TW, bool EXACT, typename Emit>
-__device__ __forceinline__ void bn_reverse_chain(const float* __restrict__ x,
-                                                 const float* __restrict__ g, int T, int64_t N,
-                                                 int64_t col, float m, float scale, float b,
-                                                 float alpha, float thresh, float beta,
-                                                 float interval, Emit&& emit) {
-    float uc = 0.f, sc = 0.f, gu = 0.f;
-    bn_reverse_window<TW, EXACT>(x, g, T, N, col, m, scale, b, uc, sc, gu, alpha, thresh, beta,
+template <typename F, int TW, bool EXACT, typename Emit>
+__device__ __forceinline__ void bn_reverse_chain(const F* __restrict__ x,
+                                                 const F* __restrict__ g, int T, int64_t N,
+                                                 int64_t col, F m, F scale, F b,
+                                                 F alpha, F thresh, F beta,
+                                                 F interval, Emit&& emit) {
+    F uc = F(0), sc = F(0), gu = F(0);
+    bn_reverse_window<F, TW, EXACT>(x, g, T, N, col, m, scale, b, uc, sc, gu, alpha, thresh, beta,
                                  interval, emit);
 }
 
@@ -171,26 +175,26 @@ __device__ __forceinline__ void bn_reverse_chain(const float* __restrict__ x,
 // lif_backward_segmented_kernel does it: forward over all but the last segment keeping the membrane
 // potential at each boundary in this lane's own LDS slots (`boundary`: [segment][blockDim.x] floats
 // of dynamic LDS), then the segments last to first.  emit gets the absolute time step.
-template <typename Emit>
-__device__ __forceinline__ void bn_reverse_segmented(const float* __restrict__ x,
-                                                     const float* __restrict__ g, int T, int64_t N,
-                                                     int64_t col, float m, float scale, float b,
-                                                     float alpha, float thresh, float beta,
-                                                     float interval, float* boundary, Emit&& emit) {
+template <typename F, typename Emit>
+__device__ __forceinline__ void bn_reverse_segmented(const F* __restrict__ x,
+                                                     const F* __restrict__ g, int T, int64_t N,
+                                                     int64_t col, F m, F scale, F b,
+                                                     F alpha, F thresh, F beta,
+                                                     F interval, F* boundary, Emit&& emit) {
     const int nseg = (T + kSegment - 1) / kSegment;
     constexpr int ROWS = 8;
     static_assert(kSegment % ROWS == 0, "a segment is a whole number of forward groups");
-    float uc = 0.f, sc = 0.f, gu = 0.f;
+    F uc = F(0), sc = F(0), gu = F(0);
     for (int seg = 0; seg + 1 < nseg; ++seg) {
         for (int t0 = seg * kSegment; t0 < (seg + 1) * kSegment; t0 += ROWS) {
-            float rows[ROWS];
+            F rows[ROWS];
 #pragma unroll
             for (int k = 0; k < ROWS; ++k)
-                rows[k] = load_pack<float, 1, false>(x + static_cast<int64_t>(t0 + k) * N + col).e[0];
+                rows[k] = load_pack<F, 1, false>(x + static_cast<int64_t>(t0 + k) * N + col).e[0];
 #pragma unroll
             for (int k = 0; k < ROWS; ++k) {
-                uc = (alpha * uc) * (1.f - sc) + (rows[k] - m) * scale + b;
-                sc = (uc > thresh) ? 1.f : 0.f;
+                uc = (alpha * uc) * (F(1) - sc) + (rows[k] - m) * scale + b;
+                sc = (uc > thresh) ? F(1) : F(0);
             }
         }
         boundary[(seg + 1) * blockDim.x + threadIdx.x] = uc;
@@ -198,37 +202,38 @@ __device__ __forceinline__ void bn_reverse_segmented(const float* __restrict__ x
     {
         const int t0 = (nseg - 1) * kSegment;
         const int64_t off = static_cast<int64_t>(t0) * N;
-        bn_reverse_window<kSegment, false>(x + off, g + off, T - t0, N, col, m, scale, b, uc, sc, gu,
+        bn_reverse_window<F, kSegment, false>(x + off, g + off, T - t0, N, col, m, scale, b, uc, sc, gu,
                                            alpha, thresh, beta, interval,
-                                           [&](int t, float gy, float xt) { emit(t0 + t, gy, xt); });
+                                           [&](int t, F gy, F xt) { emit(t0 + t, gy, xt); });
     }
     for (int seg = nseg - 2; seg >= 0; --seg) {
-        uc = seg == 0 ? 0.f : boundary[seg * blockDim.x + threadIdx.x];
-        sc = (seg != 0 && uc > thresh) ? 1.f : 0.f;
+        uc = seg == 0 ? F(0) : boundary[seg * blockDim.x + threadIdx.x];
+        sc = (seg != 0 && uc > thresh) ? F(1) : F(0);
         const int t0 = seg * kSegment;
         const int64_t off = static_cast<int64_t>(t0) * N;
-        bn_reverse_window<kSegment, true>(x + off, g + off, kSegment, N, col, m, scale, b, uc, sc, gu,
+        bn_reverse_window<F, kSegment, true>(x + off, g + off, kSegment, N, col, m, scale, b, uc, sc, gu,
                                           alpha, thresh, beta, interval,
-                                          [&](int t, float gy, float xt) { emit(t0 + t, gy, xt); });
+                                          [&](int t, F gy, F xt) { emit(t0 + t, gy, xt); });
     }
 }
 
 // Dispatch between the two: SEGMENTED kernels are instantiated with TW = kSegment.
-template <int TW, bool EXACT, bool SEGMENTED, typename Emit>
-__device__ __forceinline__ void bn_reverse(const float* __restrict__ x, const float* __restrict__ g,
-                                           int T, int64_t N, int64_t col, float m, float scale,
-                                           float b, float alpha, float thresh, float beta,
-                                           float interval, float* boundary, Emit&& emit) {
+template <typename F, int TW, bool EXACT, bool SEGMENTED, typename Emit>
+__device__ __forceinline__ void bn_reverse(const F* __restrict__ x, const F* __restrict__ g,
+                                           int T, int64_t N, int64_t col, F m, F scale,
+                                           F b, F alpha, F thresh, F beta,
+                                           F interval, F* boundary, Emit&& emit) {
     if constexpr (SEGMENTED) {
-        bn_reverse_segmented(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, boundary,
+        bn_reverse_segmented<F>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, boundary,
                              emit);
     } else {
-        bn_reverse_chain<TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, emit);
+        bn_reverse_chain<F, TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, emit);
     }
 }
 
 // Sum over the 64 lanes of a wavefront; lane 0 holds the result.
-__device__ __forceinline__ float wave_sum(float v) {
+template <typename F>
+__device__ __forceinline__ F wave_sum(F v) {
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v += __shfl_down(v, off, 64);
     return v;
@@ -240,16 +245,16 @@ __device__ __forceinline__ float wave_sum(float v) {
 // wavefronts per plane, the last one partly idle when HW is not a multiple of 64 -- so all lanes of
 // a wavefront share a channel and their sums are folded by shuffles: one pair of floats per
 // wavefront, part_* indexed [plane][chunk] (B*C*G entries).
-template <int TW, bool EXACT, bool WAVE, bool SEGMENTED = false>
+template <typename F, int TW, bool EXACT, bool WAVE, bool SEGMENTED = false>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
-lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restrict__ g,
-                               const float* __restrict__ weight, const float* __restrict__ bias,
-                               const float* __restrict__ ivar, const float* __restrict__ mean,
-                               float* __restrict__ part_gy, float* __restrict__ part_gyx, int T,
-                               int64_t N, int64_t C, int64_t HW, float alpha, float thresh,
-                               float beta, float interval) {
+lif_bn_backward_partial_kernel(const F* __restrict__ x, const F* __restrict__ g,
+                               const F* __restrict__ weight, const F* __restrict__ bias,
+                               const F* __restrict__ ivar, const F* __restrict__ mean,
+                               F* __restrict__ part_gy, F* __restrict__ part_gyx, int T,
+                               int64_t N, int64_t C, int64_t HW, F alpha, F thresh,
+                               F beta, F interval) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    float* boundary = reinterpret_cast<float*>(lds_raw);  // used by SEGMENTED only
+    F* boundary = reinterpret_cast<F*>(lds_raw);  // used by SEGMENTED only
     const bool small = N <= 0xffffffffll;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     if (WAVE) {
@@ -261,15 +266,15 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
             const int64_t plane = wave / G;
             const int64_t k = (wave - plane * G) * 64 + (pc & 63);  // position inside the plane
             const int c = static_cast<int>(plane % C);
-            float acc_gy = 0.f, acc_gyx = 0.f;
+            F acc_gy = F(0), acc_gyx = F(0);
             if (k < HW) {
                 const int64_t col = plane * HW + k;
-                const float m = mean[c], iv = ivar[c];
-                const float scale = weight[c] * iv;
-                const float b = bias[c];
-                bn_reverse<TW, EXACT, SEGMENTED>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
-                                                 interval, boundary, [&](int, float gy, float xt) {
-                                                     const float xhat = (xt - m) * iv;
+                const F m = mean[c], iv = ivar[c];
+                const F scale = weight[c] * iv;
+                const F b = bias[c];
+                bn_reverse<F, TW, EXACT, SEGMENTED>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
+                                                 interval, boundary, [&](int, F gy, F xt) {
+                                                     const F xhat = (xt - m) * iv;
                                                      acc_gy += gy;
                                                      acc_gyx += gy * xhat;
                                                  });
@@ -285,13 +290,13 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
         for (int64_t col = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; col < N;
              col += stride) {
             const int c = channel_of(col, C, HW, small);
-            const float m = mean[c], iv = ivar[c];
-            const float scale = weight[c] * iv;
-            const float b = bias[c];
-            float acc_gy = 0.f, acc_gyx = 0.f;
-            bn_reverse<TW, EXACT, SEGMENTED>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
-                                             interval, boundary, [&](int, float gy, float xt) {
-                                                 const float xhat = (xt - m) * iv;
+            const F m = mean[c], iv = ivar[c];
+            const F scale = weight[c] * iv;
+            const F b = bias[c];
+            F acc_gy = F(0), acc_gyx = F(0);
+            bn_reverse<F, TW, EXACT, SEGMENTED>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
+                                             interval, boundary, [&](int, F gy, F xt) {
+                                                 const F xhat = (xt - m) * iv;
                                                  acc_gy += gy;
                                                  acc_gyx += gy * xhat;
                                              });
@@ -303,33 +308,33 @@ lif_bn_backward_partial_kernel(const float* __restrict__ x, const float* __restr
 
 // Sweep 2: input gradient.  mean_gxhat[C], mean_gxhatx[C]: the per-channel means that sweep 1 and
 // the channel reduction produced (averaged over the ranks first when the batch is sharded).
-template <int TW, bool EXACT, bool SEGMENTED = false>
+template <typename F, int TW, bool EXACT, bool SEGMENTED = false>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
-lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restrict__ g,
-                             const float* __restrict__ weight, const float* __restrict__ bias,
-                             const float* __restrict__ ivar, const float* __restrict__ mean,
-                             const float* __restrict__ mean_gxhat,
-                             const float* __restrict__ mean_gxhatx, float* __restrict__ gx, int T,
-                             int64_t N, int64_t C, int64_t HW, float alpha, float thresh, float beta,
-                             float interval) {
+lif_bn_backward_input_kernel(const F* __restrict__ x, const F* __restrict__ g,
+                             const F* __restrict__ weight, const F* __restrict__ bias,
+                             const F* __restrict__ ivar, const F* __restrict__ mean,
+                             const F* __restrict__ mean_gxhat,
+                             const F* __restrict__ mean_gxhatx, F* __restrict__ gx, int T,
+                             int64_t N, int64_t C, int64_t HW, F alpha, F thresh, F beta,
+                             F interval) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    float* boundary = reinterpret_cast<float*>(lds_raw);  // used by SEGMENTED only
+    F* boundary = reinterpret_cast<F*>(lds_raw);  // used by SEGMENTED only
     const bool small = N <= 0xffffffffll;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < N;
          v += stride) {
         const int64_t col = N - 1 - v;  // opposite direction to sweep 1: its tail is still cached
         const int c = channel_of(col, C, HW, small);
-        const float m = mean[c], iv = ivar[c], wgt = weight[c];
-        const float scale = wgt * iv;
-        const float b = bias[c];
-        const float gxhat = mean_gxhat[c], gxhatx = mean_gxhatx[c];
-        bn_reverse<TW, EXACT, SEGMENTED>(
+        const F m = mean[c], iv = ivar[c], wgt = weight[c];
+        const F scale = wgt * iv;
+        const F b = bias[c];
+        const F gxhat = mean_gxhat[c], gxhatx = mean_gxhatx[c];
+        bn_reverse<F, TW, EXACT, SEGMENTED>(
             x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, boundary,
-            [&](int t, float gy, float xt) {
-                Pack<float, 1> out;
+            [&](int t, F gy, F xt) {
+                Pack<F, 1> out;
                 out.e[0] = gy * wgt * iv - iv * ((xt - m) * iv * gxhatx + gxhat);
-                store_pack<float, 1>(gx + static_cast<int64_t>(t) * N + col, out);
+                store_pack<F, 1>(gx + static_cast<int64_t>(t) * N + col, out);
             });
     }
 }
@@ -340,16 +345,17 @@ lif_bn_backward_input_kernel(const float* __restrict__ x, const float* __restric
 // (consecutive addresses), so the sum order is fixed by the geometry alone.
 // split = {gy[S][C], gyx[S][C]}.
 // ---------------------------------------------------------------------------------------------
+template <typename F>
 __global__ void __launch_bounds__(kReduceBlock)
-bn_channel_reduce_kernel(const float* __restrict__ part_gy, const float* __restrict__ part_gyx,
-                         float* __restrict__ split, int64_t B, int64_t C, int64_t HW, int64_t bs,
+bn_channel_reduce_kernel(const F* __restrict__ part_gy, const F* __restrict__ part_gyx,
+                         F* __restrict__ split, int64_t B, int64_t C, int64_t HW, int64_t bs,
                          int S) {
     const int c = blockIdx.x;
     const int s = blockIdx.y;
     const int64_t b0 = static_cast<int64_t>(s) * bs;
     const int64_t b1 = (b0 + bs < B) ? (b0 + bs) : B;
     const int64_t CHW = C * HW;
-    float a = 0.f, ax = 0.f;
+    F a = F(0), ax = F(0);
     if (HW >= kReduceBlock / 4) {
         for (int64_t b = b0; b < b1; ++b) {
             const int64_t base = b * CHW + static_cast<int64_t>(c) * HW;
@@ -367,7 +373,7 @@ bn_channel_reduce_kernel(const float* __restrict__ part_gy, const float* __restr
             ax += part_gyx[at];
         }
     }
-    __shared__ float lds[2][kReduceBlock / 64];
+    __shared__ F lds[2][kReduceBlock / 64];
     a = wave_sum(a);
     ax = wave_sum(ax);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -377,7 +383,7 @@ bn_channel_reduce_kernel(const float* __restrict__ part_gy, const float* __restr
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        float ta = 0.f, tax = 0.f;
+        F ta = F(0), tax = F(0);
 #pragma unroll
         for (int w = 0; w < kReduceBlock / 64; ++w) {
             ta += lds[0][w];
@@ -391,23 +397,24 @@ bn_channel_reduce_kernel(const float* __restrict__ part_gy, const float* __restr
 // Whole reduction of one channel in one workgroup, for partials that are few (the wave-summed
 // form): sums the B*G entries of channel c (G entries per batch entry), then writes the parameter
 // gradients and the two coefficients of the input-gradient sweep.
+template <typename F>
 __global__ void __launch_bounds__(kReduceBlock)
-bn_channel_reduce_finalize_kernel(const float* __restrict__ part_gy,
-                                  const float* __restrict__ part_gyx,
-                                  const float* __restrict__ weight, float* __restrict__ grad_weight,
-                                  float* __restrict__ grad_bias, float* __restrict__ mean_gxhat,
-                                  float* __restrict__ mean_gxhatx, int64_t B, int64_t C, int64_t G,
-                                  float count) {
+bn_channel_reduce_finalize_kernel(const F* __restrict__ part_gy,
+                                  const F* __restrict__ part_gyx,
+                                  const F* __restrict__ weight, F* __restrict__ grad_weight,
+                                  F* __restrict__ grad_bias, F* __restrict__ mean_gxhat,
+                                  F* __restrict__ mean_gxhatx, int64_t B, int64_t C, int64_t G,
+                                  F count) {
     const int c = blockIdx.x;
     const int64_t n = B * G;
-    float a = 0.f, ax = 0.f;
+    F a = F(0), ax = F(0);
     for (int64_t e = threadIdx.x; e < n; e += kReduceBlock) {
         const int64_t b = e / G, i = e % G;
         const int64_t at = (b * C + c) * G + i;
         a += part_gy[at];
         ax += part_gyx[at];
     }
-    __shared__ float lds[2][kReduceBlock / 64];
+    __shared__ F lds[2][kReduceBlock / 64];
     a = wave_sum(a);
     ax = wave_sum(ax);
     const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
@@ -417,7 +424,7 @@ bn_channel_reduce_finalize_kernel(const float* __restrict__ part_gy,
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        float ta = 0.f, tax = 0.f;
+        F ta = F(0), tax = F(0);
 #pragma unroll
         for (int w = 0; w < kReduceBlock / 64; ++w) {
             ta += lds[0][w];
@@ -425,7 +432,7 @@ bn_channel_reduce_finalize_kernel(const float* __restrict__ part_gy,
         }
         grad_bias[c] = ta;
         grad_weight[c] = tax;
-        const float wgt = weight[c];
+        const F wgt = weight[c];
         mean_gxhat[c] = (ta * wgt) / count;
         mean_gxhatx[c] = (tax * wgt) / count;
     }
@@ -433,21 +440,22 @@ bn_channel_reduce_finalize_kernel(const float* __restrict__ part_gy,
 
 // One lane per channel: fold the S splits in order, emit the parameter gradients and the two
 // coefficients the input-gradient sweep needs.
+template <typename F>
 __global__ void __launch_bounds__(kReduceBlock)
-bn_channel_finalize_kernel(const float* __restrict__ split, const float* __restrict__ weight,
-                           float* __restrict__ grad_weight, float* __restrict__ grad_bias,
-                           float* __restrict__ mean_gxhat, float* __restrict__ mean_gxhatx,
-                           int64_t C, int S, float count) {
+bn_channel_finalize_kernel(const F* __restrict__ split, const F* __restrict__ weight,
+                           F* __restrict__ grad_weight, F* __restrict__ grad_bias,
+                           F* __restrict__ mean_gxhat, F* __restrict__ mean_gxhatx,
+                           int64_t C, int S, F count) {
     const int64_t c = static_cast<int64_t>(blockIdx.x) * kReduceBlock + threadIdx.x;
     if (c >= C) return;
-    float a = 0.f, ax = 0.f;
+    F a = F(0), ax = F(0);
     for (int s = 0; s < S; ++s) {
         a += split[static_cast<int64_t>(s) * C + c];
         ax += split[static_cast<int64_t>(S) * C + static_cast<int64_t>(s) * C + c];
     }
     grad_bias[c] = a;
     grad_weight[c] = ax;
-    const float wgt = weight[c];
+    const F wgt = weight[c];
     mean_gxhat[c] = (a * wgt) / count;
     mean_gxhatx[c] = (ax * wgt) / count;
 }

@@ -273,6 +273,7 @@ Tensor fire_bp(Tensor spatial, Tensor grad_spike, float alpha, float thresh, flo
 
 struct BnOperands {
     BnDims d;
+    int dtype;  // SNNLIF_DTYPE_F32 or SNNLIF_DTYPE_F64; the per-channel tensors share it
     Tensor x, weight, bias, stat, mean;
 };
 
@@ -281,9 +282,11 @@ BnOperands bn_operands(const Tensor& spatial, const Tensor& weight_bn, const Ten
                        const Tensor& stat, const Tensor& mean, const char* op,
                        const char* stat_name) {
     check_input(spatial, op, "spatial");
-    TORCH_CHECK(spatial.scalar_type() == at::kFloat, "snnlib.", op,
-                ": only float32 is supported, got ", spatial.scalar_type());
+    TORCH_CHECK(spatial.scalar_type() == at::kFloat || spatial.scalar_type() == at::kDouble,
+                "snnlib.", op, ": only float32 and float64 are supported, got ",
+                spatial.scalar_type());
     BnOperands o;
+    o.dtype = spatial.scalar_type() == at::kFloat ? SNNLIF_DTYPE_F32 : SNNLIF_DTYPE_F64;
     o.d = bn_dims_of(spatial, op);
     o.x = spatial.contiguous();
     o.weight = channel_param(weight_bn, o.x, o.d.C, op, "weight_bn");
@@ -301,7 +304,7 @@ std::vector<Tensor> bn_fire_s_fp(Tensor spatial, Tensor weight_bn, Tensor bias_b
     Tensor spike = torch::empty_like(o.x, at::MemoryFormat::Contiguous);
     check_rc(snnlif_bn_fire_s_fp(o.x.data_ptr(), o.weight.data_ptr(), o.bias.data_ptr(),
                                  o.stat.data_ptr(), o.mean.data_ptr(), ivar.data_ptr(),
-                                 spike.data_ptr(), SNNLIF_DTYPE_F32, o.d.T, o.d.B, o.d.C, o.d.HW,
+                                 spike.data_ptr(), o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW,
                                  eps_bn, alpha, thresh, current_stream()),
              "bn_fire_s_fp");
     return {ivar, spike};
@@ -317,7 +320,7 @@ Tensor bn_fire_spikes_from_ivar(const Tensor& spatial, const Tensor& weight_bn,
     Tensor spike = torch::empty_like(o.x, at::MemoryFormat::Contiguous);
     check_rc(snnlif_bn_fire_s_recompute(o.x.data_ptr(), o.weight.data_ptr(), o.bias.data_ptr(),
                                         o.stat.data_ptr(), o.mean.data_ptr(), spike.data_ptr(),
-                                        SNNLIF_DTYPE_F32, o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh,
+                                        o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh,
                                         current_stream()),
              op);
     return spike;
@@ -337,13 +340,13 @@ std::vector<Tensor> bn_fire_bp(Tensor spatial, Tensor weight_bn, Tensor bias_bn,
     Tensor grad_weight = torch::empty_like(o.weight, at::MemoryFormat::Contiguous);
     Tensor grad_bias = torch::empty_like(o.weight, at::MemoryFormat::Contiguous);
     const size_t ws_bytes =
-        snnlif_bn_fire_bp_workspace_bytes(SNNLIF_DTYPE_F32, o.d.T, o.d.B, o.d.C, o.d.HW);
+        snnlif_bn_fire_bp_workspace_bytes(o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW);
     Tensor workspace =
         torch::empty({static_cast<int64_t>(ws_bytes)}, o.x.options().dtype(at::kByte));
     check_rc(snnlif_bn_fire_bp(o.x.data_ptr(), o.weight.data_ptr(), o.bias.data_ptr(),
                                o.stat.data_ptr(), o.mean.data_ptr(), g.data_ptr(),
                                grad_spatial.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(),
-                               SNNLIF_DTYPE_F32, o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh, beta,
+                               o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh, beta,
                                interval, ws_bytes ? workspace.data_ptr() : nullptr, ws_bytes,
                                current_stream()),
              "bn_fire_bp");
@@ -370,13 +373,13 @@ std::vector<Tensor> bn_fire_bp_dist1(Tensor spatial, Tensor weight_bn, Tensor bi
     Tensor grad_weight = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
     Tensor grad_bias = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
     const size_t ws_bytes =
-        snnlif_bn_fire_bp_workspace_bytes(SNNLIF_DTYPE_F32, o.d.T, o.d.B, o.d.C, o.d.HW);
+        snnlif_bn_fire_bp_workspace_bytes(o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW);
     Tensor workspace =
         torch::empty({static_cast<int64_t>(ws_bytes)}, o.x.options().dtype(at::kByte));
     check_rc(snnlif_bn_fire_bp_dist1(o.x.data_ptr(), o.weight.data_ptr(), o.bias.data_ptr(),
                                      o.stat.data_ptr(), o.mean.data_ptr(), g.data_ptr(),
                                      mean_gxhat.data_ptr(), mean_gxhatx.data_ptr(),
-                                     grad_weight.data_ptr(), grad_bias.data_ptr(), SNNLIF_DTYPE_F32,
+                                     grad_weight.data_ptr(), grad_bias.data_ptr(), o.dtype,
                                      o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh, beta, interval,
                                      ws_bytes ? workspace.data_ptr() : nullptr, ws_bytes,
                                      current_stream()),
@@ -401,7 +404,7 @@ Tensor bn_fire_bp_dist2(Tensor spatial, Tensor weight_bn, Tensor bias_bn, Tensor
     check_rc(snnlif_bn_fire_bp_dist2(o.x.data_ptr(), o.weight.data_ptr(), o.bias.data_ptr(),
                                      o.stat.data_ptr(), o.mean.data_ptr(), g.data_ptr(),
                                      gxhat.data_ptr(), gxhatx.data_ptr(), grad_spatial.data_ptr(),
-                                     SNNLIF_DTYPE_F32, o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh,
+                                     o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW, alpha, thresh,
                                      beta, interval, current_stream()),
              op);
     return grad_spatial;

@@ -364,3 +364,47 @@ def test_bn_fire_loops_match_autograd_through_batch_norm(shape):
     assert np.abs(gx - xr.grad.numpy()).max() <= 1e-5 * scale(gx)
     assert np.abs(gw - wr.grad.numpy()).max() <= 1e-5 * scale(gw)
     assert np.abs(gb - br.grad.numpy()).max() <= 1e-5 * scale(gb)
+
+
+@pytest.mark.parametrize("shape", [(6, 4, 8, 8, 8), (6, 16, 8), (3, 2, 5, 7), (1, 6, 3, 5)])
+def test_bn_fire_double_precision_loops(shape):
+    """The fp64 instantiation of the same loops: against autograd in double through batch_norm + the
+    gold fire loop (errors at double rounding level), against the textbook closed form when T = 1, and
+    against the fp32 loops on the same inputs."""
+    eps = 1e-5
+    x, g, w, b, var, mean = (t.double() for t in _bn_case(shape, 43))
+    dims = (0, 1) + tuple(range(3, len(shape)))
+    var, mean = torch.var_mean(x, dim=dims, unbiased=False)
+    n = lambda t: t.numpy()
+    ivar, mem, spike = c_oracle.bn_fire_forward(n(x), n(w), n(b), n(var), n(mean), eps, 0.25, 0.5)
+    gx, gw, gb = c_oracle.bn_fire_backward(n(x), n(w), n(b), ivar, n(mean), n(g), 0.25, 0.5, 0.8, 0.6)
+    assert ivar.dtype == mem.dtype == gx.dtype == gw.dtype == np.float64
+
+    xr, wr, br = x.clone().requires_grad_(True), w.clone().requires_grad_(True), b.clone().requires_grad_(True)
+    # hyper-parameters reach the loops as C floats (as in the reference's kernels): give the double
+    # graph the same values
+    f = lambda v: float(np.float32(v))
+    u, s = gold_fire.gold_bn_fire(xr, wr, br, None, None, True, f(eps), 0.25, 0.5, f(0.8), f(0.6))
+    s.backward(g)
+    assert np.array_equal(spike, n(s.detach()))
+    np.testing.assert_allclose(mem, n(u.detach()), rtol=1e-12, atol=1e-13)
+    for got, want in ((gx, xr.grad), (gw, wr.grad), (gb, br.grad)):
+        assert np.abs(got - n(want)).max() <= 1e-11 * (np.abs(got).max() + 1e-300)
+
+    if shape[0] == 1:
+        sh = (1, 1, shape[2]) + (1,) * (len(shape) - 3)
+        iv = 1.0 / np.sqrt(n(var).reshape(sh) + np.float64(np.float32(eps)))
+        xhat = (n(x) - n(mean).reshape(sh)) * iv
+        y = xhat * n(w).reshape(sh) + n(b).reshape(sh)
+        gy = n(g) * (np.abs(y - 0.5) < np.float64(np.float32(0.6))) * np.float64(np.float32(0.8))
+        gxhat = gy * n(w).reshape(sh)
+        expect = iv * (gxhat - gxhat.mean(axis=dims, keepdims=True) - xhat * (gxhat * xhat).mean(axis=dims, keepdims=True))
+        np.testing.assert_allclose(gx, expect, rtol=1e-9, atol=1e-12)
+
+    # the fp32 loops on the same (fp32-representable) inputs
+    x32 = x.float()
+    var32, mean32 = torch.var_mean(x32, dim=dims, unbiased=False)
+    iv32, mem32, spike32 = c_oracle.bn_fire_forward(n(x32), n(w.float()), n(b.float()), n(var32), n(mean32), eps, 0.25, 0.5)
+    assert iv32.dtype == np.float32
+    np.testing.assert_allclose(iv32, c_oracle.bn_fire_forward(n(x32.double()), n(w.float().double()), n(b.float().double()),
+                                                               n(var32.double()), n(mean32.double()), eps, 0.25, 0.5)[0], rtol=1e-6)

@@ -3,7 +3,8 @@ offsets through the C ABI against the CPU oracle: the cases nobody thought of li
 
 fp32 / fp64: spikes, membrane potentials and gradients bit-identical.  bf16 storage: spikes exact,
 potentials and gradients equal to the fp32 oracle on the bf16-rounded inputs rounded once to bf16.
-Batch-norm + fire: spikes and inverse standard deviation bit-identical, gradients to 1e-5 of scale.
+Batch-norm + fire (fp32 and fp64): spikes and inverse standard deviation bit-identical, gradients to
+1e-5 (fp32) / 1e-11 (fp64) of scale.
 """
 import numpy as np
 import pytest
@@ -94,23 +95,26 @@ def test_random_bn_fire_case(cabi, oracle, seed):
     beta = float(rng.choice([0.7, 1.0]))
     interval = float(rng.choice([0.5, 1.5]))
     eps = 1e-5
+    dtype = torch.float64 if rng.integers(0, 3) == 0 else torch.float32
     shape = (T, B, C, HW)
     gen = torch.Generator().manual_seed(seed)
-    x = 0.5 + torch.randn(shape, generator=gen) * (0.5 + torch.rand((C, 1), generator=gen))
-    g = torch.randn(shape, generator=gen)
-    w = 0.5 + torch.rand(C, generator=gen)
-    b = 0.2 * torch.randn(C, generator=gen)
+    x = (0.5 + torch.randn(shape, generator=gen) * (0.5 + torch.rand((C, 1), generator=gen))).to(dtype)
+    g = torch.randn(shape, generator=gen).to(dtype)
+    w = (0.5 + torch.rand(C, generator=gen)).to(dtype)
+    b = (0.2 * torch.randn(C, generator=gen)).to(dtype)
     var, mean = torch.var_mean(x, dim=(0, 1, 3), unbiased=False)
     var = var + 0.05          # also meaningful when T*B*HW == 1
     xd, gd, wd, bd, vd, md = (t.cuda() for t in (x, g, w, b, var, mean))
     ivar, spike = torch.empty_like(vd), torch.empty_like(xd)
     cabi.bn_fire_s_fp_into(xd, wd, bd, vd, md, ivar, spike, eps, alpha, thresh)
     gx, gw, gb = torch.empty_like(xd), torch.empty_like(wd), torch.empty_like(wd)
-    ws = torch.empty(cabi.bn_fire_bp_workspace_bytes(cabi.DTYPE_F32, T, B, C, HW), dtype=torch.uint8, device="cuda")
+    code = cabi.DTYPE_F64 if dtype == torch.float64 else cabi.DTYPE_F32
+    ws = torch.empty(cabi.bn_fire_bp_workspace_bytes(code, T, B, C, HW), dtype=torch.uint8, device="cuda")
     cabi.bn_fire_bp_into(xd, wd, bd, ivar, md, gd, gx, gw, gb, alpha, thresh, beta, interval, ws)
     torch.cuda.synchronize()
 
-    what = f"T={T} B={B} C={C} HW={HW} a={alpha} th={thresh} b={beta} iv={interval}"
+    what = f"T={T} B={B} C={C} HW={HW} {dtype} a={alpha} th={thresh} b={beta} iv={interval}"
+    tol, floor = (1e-11, 1e-14) if dtype == torch.float64 else (1e-5, 1e-7)
     ivar_o, _, spike_o = oracle.bn_fire_forward(x.numpy(), w.numpy(), b.numpy(), var.numpy(), mean.numpy(), eps, alpha, thresh)
     gx_o, gw_o, gb_o = oracle.bn_fire_backward(x.numpy(), w.numpy(), b.numpy(), ivar_o, mean.numpy(), g.numpy(),
                                                alpha, thresh, beta, interval)
@@ -119,4 +123,4 @@ def test_random_bn_fire_case(cabi, oracle, seed):
     for got, want, name in ((gb, gb_o, "bias"), (gw, gw_o, "weight"), (gx, gx_o, "input")):
         scale = np.abs(want).max() + 1e-12
         err = np.abs(got.cpu().numpy() - want).max()
-        assert err <= 1e-5 * scale + 1e-7, f"{what}: {name} gradient err {err:.3e} vs scale {scale:.3e}"
+        assert err <= tol * scale + floor, f"{what}: {name} gradient err {err:.3e} vs scale {scale:.3e}"
