@@ -261,12 +261,6 @@ def run_bn_fire(args):
     fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
     bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
 
-    # parity on a sample of channels (channels are independent given their statistics)
-    from oracle import c_oracle
-    pick = [0, 1, C // 2, C - 1]
-    take = lambda t: t[:, :8, pick].contiguous().cpu().numpy()
-    p = lambda t: t[pick].cpu().numpy()
-    ivar_o, _, spike_o = c_oracle.bn_fire_forward(take(x), p(weight), p(bias), p(var), p(mean), eps, ALPHA, THRESH)
     result = {
         "metric": "BnFire fwd+bwd neuron-steps/s (next-row op, not the headline metric)",
         "value": ns * args.steps / wall, "unit": "neuron-steps/s", "n_gpus": 1, "steps": args.steps,
@@ -282,9 +276,28 @@ def run_bn_fire(args):
                      "fwd": {"algorithmic_bytes_per_launch": 8 * ns, "avg_launch_ms": fwd_ms,
                              "achieved": 8 * ns / (fwd_ms * 1e-3) / 1e9,
                              "frac": 8 * ns / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
-        "parity": {"sampled_spikes_bit_exact": bool(np.array_equal(take(spike), spike_o)),
-                   "sampled_ivar_bit_exact": bool(np.array_equal(p(ivar), ivar_o))},
     }
+    if not args.no_cpu_baseline:
+        # CPU leg: the scalar C loops of the oracle on a bounded sample (channels are independent given
+        # their statistics; the backward's means are those of the sample), one host thread.  Its
+        # forward outputs double as the parity check of this run.
+        from oracle import c_oracle
+        pick = [0, 1, C // 2, C - 1]
+        take = lambda t: t[:, :8, pick].contiguous().cpu().numpy()
+        p = lambda t: t[pick].cpu().numpy()
+        xs, gs = take(x), take(g)
+        t0 = time.perf_counter()
+        ivar_o, _, spike_o = c_oracle.bn_fire_forward(xs, p(weight), p(bias), p(var), p(mean), eps, ALPHA, THRESH)
+        t1 = time.perf_counter()
+        c_oracle.bn_fire_backward(xs, p(weight), p(bias), ivar_o, p(mean), gs, ALPHA, THRESH, BETA, INTERVAL)
+        t2 = time.perf_counter()
+        result["cpu_baseline"] = {
+            "value": xs.size / (t2 - t0), "unit": "neuron-steps/s", "cores": 1, "kind": "port",
+            "sample": f"channels {pick} of batch entries [0, 8) ({xs.size} neuron-steps), forward + backward of "
+                      "oracle/lif_oracle.c (scalar C loops), single run",
+            "fwd_s": t1 - t0, "bwd_s": t2 - t1}
+        result["parity"] = {"sampled_spikes_bit_exact": bool(np.array_equal(take(spike), spike_o)),
+                            "sampled_ivar_bit_exact": bool(np.array_equal(p(ivar), ivar_o))}
     print(json.dumps(result), flush=True)
 
 
