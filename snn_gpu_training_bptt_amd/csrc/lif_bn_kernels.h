@@ -1,5 +1,6 @@
-// Batch-norm + LIF fire kernels (F = float or double; one neuron per lane) for MI355X: the per-channel affine of a batch norm is
-// applied to the input current inside the fire recurrence, forward and backward.
+// Batch-norm + LIF fire kernels (F = float or double; one neuron per lane) for MI355X: the
+// per-channel affine of a batch norm is applied to the input current inside the fire recurrence,
+// forward and backward.
 //
 // Reference: snnlib/cuda/snn_kernel_fp.cu:157-240 (bn_fire_s_fp_kernel + launcher) and
 // snnlib/cuda/snn_kernel_bp.cu:432-479 (bn_fire_u_fp_kernel), :533-610 (bn_fire_bp_wb_kernel),
