@@ -155,8 +155,9 @@ int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const vo
                                int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
                                void* stream);
 
-/* Bytes of device workspace snnlif_bn_fire_bp needs (two values of the storage type per neuron plus
- * per-channel staging).  0 for invalid arguments. */
+/* Bytes of device workspace snnlif_bn_fire_bp needs: two partial sums of the storage type per
+ * wavefront of sweep 1 (ceil(HW/64) wavefronts per (batch entry, channel) plane) when HW >= 32, two
+ * per neuron otherwise, plus per-channel staging.  0 for invalid arguments. */
 size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);
 
 /*

@@ -20,12 +20,24 @@ inline int bn_reduce_splits(int64_t B, int64_t C) {
     return static_cast<int>(s);
 }
 
+// Sweep 1 of the backward lays wavefronts over the (batch entry, channel) planes when a plane has at
+// least this many positions (all lanes of a wavefront then share a channel and fold their sums by
+// shuffles); smaller planes keep one lane per neuron in storage order.
+constexpr int64_t kBnWavePlaneMin = 32;
+inline bool bn_wave_partials(int64_t HW) { return HW >= kBnWavePlaneMin; }
+
+// Partial sums sweep 1 leaves per quantity: one per wavefront (ceil(HW/64) per plane) or one per neuron.
+inline size_t bn_partial_count(int64_t B, int64_t C, int64_t HW) {
+    if (bn_wave_partials(HW)) return static_cast<size_t>(B * C) * static_cast<size_t>((HW + 63) / 64);
+    return static_cast<size_t>(B * C * HW);
+}
+
 // Workspace of the backward in elements of the scalar type:
-// part_gy[N], part_gyx[N], split[2*S*C], coef[2*C].
+// part_gy[P], part_gyx[P], split[2*S*C] (per-neuron partials only), coef[2*C], P = bn_partial_count.
 inline size_t bn_backward_workspace_elems(int64_t B, int64_t C, int64_t HW) {
-    const int S = bn_reduce_splits(B, C);
-    return static_cast<size_t>(2 * B * C * HW) + static_cast<size_t>(2) * S * C +
-           static_cast<size_t>(2 * C);
+    const size_t split =
+        bn_wave_partials(HW) ? 0 : static_cast<size_t>(2) * bn_reduce_splits(B, C) * static_cast<size_t>(C);
+    return 2 * bn_partial_count(B, C, HW) + split + static_cast<size_t>(2 * C);
 }
 
 // Per scalar type F (suffix f32 = float, f64 = double):

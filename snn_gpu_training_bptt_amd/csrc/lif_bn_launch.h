@@ -66,9 +66,10 @@ int bn_backward_stats_window(const F* x, const F* weight, const F* bias, const F
                              hipStream_t stream) {
     const int64_t N = B * C * HW;
     const int S = bn_reduce_splits(B, C);
+    const size_t P = bn_partial_count(B, C, HW);
     F* part_gy = workspace;
-    F* part_gyx = part_gy + N;
-    F* split = part_gyx + N;
+    F* part_gyx = part_gy + P;
+    F* split = part_gyx + P;
     const int threads =
         backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(F), kBnSmallBlock);
     const dim3 block(threads);
@@ -79,7 +80,7 @@ int bn_backward_stats_window(const F* x, const F* weight, const F* bias, const F
 
     // Planes with few positions (fully connected shapes) would leave most lanes of a plane-aligned
     // wavefront idle; they keep one lane per neuron and per-neuron partials.
-    const bool wave = HW >= 32;
+    const bool wave = bn_wave_partials(HW);
     const int64_t G = (HW + 63) / 64;
     const dim3 grid_partial(wave ? grid_for(B * C * G * 64, threads) : grid_for(N, threads));
     int rc;

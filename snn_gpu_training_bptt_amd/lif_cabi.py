@@ -101,6 +101,47 @@ def _require_dense_gpu(*tensors):
             raise ValueError("dense (contiguous) tensor required")
 
 
+def _require_like(spatial, **tensors):
+    """Every named tensor must have ``spatial``'s shape, dtype and device: the C ABI sees only
+    pointers and derives all sizes from ``spatial``, so a smaller or differently typed buffer would
+    become an out-of-bounds device access."""
+    for name, t in tensors.items():
+        if t is None:
+            continue
+        if t.shape != spatial.shape:
+            raise ValueError(f"{name} has shape {tuple(t.shape)}, spatial has {tuple(spatial.shape)}")
+        if t.dtype != spatial.dtype:
+            raise ValueError(f"{name} has dtype {t.dtype}, spatial has {spatial.dtype}")
+        if t.device != spatial.device:
+            raise ValueError(f"{name} is on {t.device}, spatial is on {spatial.device}")
+
+
+def _require_per_channel(spatial, channels, **tensors):
+    """Per-channel vectors: ``channels`` values of ``spatial``'s dtype on its device."""
+    for name, t in tensors.items():
+        if t.numel() != channels:
+            raise ValueError(f"{name} has {t.numel()} values, spatial has {channels} channels")
+        if t.dtype != spatial.dtype:
+            raise ValueError(f"{name} has dtype {t.dtype}, spatial has {spatial.dtype}")
+        if t.device != spatial.device:
+            raise ValueError(f"{name} is on {t.device}, spatial is on {spatial.device}")
+
+
+def _require_workspace(spatial, workspace, need, what):
+    """A uint8 device buffer of at least ``need`` bytes (``None`` allowed when nothing is needed)."""
+    import torch
+    if workspace is None:
+        if need:
+            raise ValueError(f"{what} needs a workspace of {need} bytes")
+        return
+    if workspace.dtype != torch.uint8:
+        raise ValueError(f"workspace must be a uint8 tensor, got {workspace.dtype}")
+    if workspace.device != spatial.device:
+        raise ValueError(f"workspace is on {workspace.device}, spatial is on {spatial.device}")
+    if workspace.numel() < need:
+        raise ValueError(f"workspace holds {workspace.numel()} bytes, {what} needs {need}")
+
+
 def time_next_kernel(start_event, stop_event):
     """Attach two ``torch.cuda.Event(enable_timing=True)`` objects to the next kernel this thread
     launches through the library (see ``snnlif_time_next_kernel``).  The events must already exist
@@ -112,8 +153,9 @@ def time_next_kernel(start_event, stop_event):
 
 def fire_s_fp_into(spatial, spike, alpha, thresh):
     """``snnlif_fire_s_fp`` on torch tensors already resident on the GPU; writes ``spike``."""
-    _require_dense_gpu(spatial, spike)
+    _require_like(spatial, spike=spike)
     T, N = _dims(spatial)
+    _require_dense_gpu(spatial, spike)
     rc = load().snnlif_fire_s_fp(spatial.data_ptr(), spike.data_ptr(), _torch_dtype_code(spatial),
                                  T, N, alpha, thresh, _stream_handle(spatial))
     _check(rc, "snnlif_fire_s_fp")
@@ -122,8 +164,9 @@ def fire_s_fp_into(spatial, spike, alpha, thresh):
 
 def fire_us_fp_into(spatial, mem, spike, alpha, thresh):
     """``snnlif_fire_us_fp``; ``mem`` or ``spike`` may be None to skip that output."""
-    _require_dense_gpu(spatial, mem, spike)
+    _require_like(spatial, mem=mem, spike=spike)
     T, N = _dims(spatial)
+    _require_dense_gpu(spatial, mem, spike)
     rc = load().snnlif_fire_us_fp(spatial.data_ptr(),
                                   mem.data_ptr() if mem is not None else None,
                                   spike.data_ptr() if spike is not None else None,
@@ -139,10 +182,13 @@ def fire_bp_workspace_bytes(dtype_code, T, N):
 
 def fire_bp_into(spatial, grad_spike, grad_spatial, alpha, thresh, beta, interval, workspace=None):
     """``snnlif_fire_bp``; ``workspace`` is a uint8 device tensor when the shape needs one."""
-    _require_dense_gpu(spatial, grad_spike, grad_spatial, workspace)
+    _require_like(spatial, grad_spike=grad_spike, grad_spatial=grad_spatial)
     T, N = _dims(spatial)
+    _require_workspace(spatial, workspace, fire_bp_workspace_bytes(_torch_dtype_code(spatial), T, N),
+                       "snnlif_fire_bp")
     ws_ptr = workspace.data_ptr() if workspace is not None else None
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
+    _require_dense_gpu(spatial, grad_spike, grad_spatial, workspace)
     rc = load().snnlif_fire_bp(spatial.data_ptr(), grad_spike.data_ptr(), grad_spatial.data_ptr(),
                                _torch_dtype_code(spatial), T, N, alpha, thresh, beta, interval,
                                ws_ptr, ws_bytes, _stream_handle(spatial))
@@ -158,8 +204,10 @@ def _bn_dims(t):
 
 def bn_fire_s_fp_into(spatial, weight, bias, var, mean, ivar, spike, eps, alpha, thresh):
     """``snnlif_bn_fire_s_fp`` on fp32 device tensors; writes ``ivar`` ([C]) and ``spike``."""
-    _require_dense_gpu(spatial, weight, bias, var, mean, ivar, spike)
     T, B, C, HW = _bn_dims(spatial)
+    _require_like(spatial, spike=spike)
+    _require_per_channel(spatial, C, weight=weight, bias=bias, var=var, mean=mean, ivar=ivar)
+    _require_dense_gpu(spatial, weight, bias, var, mean, ivar, spike)
     rc = load().snnlif_bn_fire_s_fp(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                     var.data_ptr(), mean.data_ptr(), ivar.data_ptr(),
                                     spike.data_ptr(), _torch_dtype_code(spatial), T, B, C, HW, eps,
@@ -170,8 +218,10 @@ def bn_fire_s_fp_into(spatial, weight, bias, var, mean, ivar, spike, eps, alpha,
 
 def bn_fire_s_recompute_into(spatial, weight, bias, ivar, mean, spike, alpha, thresh):
     """``snnlif_bn_fire_s_recompute``: spikes from saved ``ivar`` / ``mean`` (backward-side scale)."""
-    _require_dense_gpu(spatial, weight, bias, ivar, mean, spike)
     T, B, C, HW = _bn_dims(spatial)
+    _require_like(spatial, spike=spike)
+    _require_per_channel(spatial, C, weight=weight, bias=bias, ivar=ivar, mean=mean)
+    _require_dense_gpu(spatial, weight, bias, ivar, mean, spike)
     rc = load().snnlif_bn_fire_s_recompute(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                            ivar.data_ptr(), mean.data_ptr(), spike.data_ptr(),
                                            _torch_dtype_code(spatial), T, B, C, HW, alpha, thresh,
@@ -187,9 +237,15 @@ def bn_fire_bp_workspace_bytes(dtype_code, T, B, C, HW):
 def bn_fire_bp_into(spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
                     grad_bias, alpha, thresh, beta, interval, workspace):
     """``snnlif_bn_fire_bp`` on fp32 device tensors; ``workspace`` is a uint8 device tensor."""
+    T, B, C, HW = _bn_dims(spatial)
+    _require_like(spatial, grad_spike=grad_spike, grad_spatial=grad_spatial)
+    _require_per_channel(spatial, C, weight=weight, bias=bias, ivar=ivar, mean=mean,
+                         grad_weight=grad_weight, grad_bias=grad_bias)
+    _require_workspace(spatial, workspace,
+                       bn_fire_bp_workspace_bytes(_torch_dtype_code(spatial), T, B, C, HW),
+                       "snnlif_bn_fire_bp")
     _require_dense_gpu(spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
                        grad_bias, workspace)
-    T, B, C, HW = _bn_dims(spatial)
     rc = load().snnlif_bn_fire_bp(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                   ivar.data_ptr(), mean.data_ptr(), grad_spike.data_ptr(),
                                   grad_spatial.data_ptr(), grad_weight.data_ptr(),
@@ -223,9 +279,12 @@ def bn_fire_bp_dist1_into(spatial, weight, bias, ivar, mean, grad_spike, mean_gx
 def bn_fire_bp_dist2_into(spatial, weight, bias, ivar, mean, grad_spike, grad_xhat, grad_xhatx,
                           grad_spatial, alpha, thresh, beta, interval):
     """``snnlif_bn_fire_bp_dist2`` on fp32 device tensors: the half after the all-reduce."""
+    T, B, C, HW = _bn_dims(spatial)
+    _require_like(spatial, grad_spike=grad_spike, grad_spatial=grad_spatial)
+    _require_per_channel(spatial, C, weight=weight, bias=bias, ivar=ivar, mean=mean,
+                         grad_xhat=grad_xhat, grad_xhatx=grad_xhatx)
     _require_dense_gpu(spatial, weight, bias, ivar, mean, grad_spike, grad_xhat, grad_xhatx,
                        grad_spatial)
-    T, B, C, HW = _bn_dims(spatial)
     rc = load().snnlif_bn_fire_bp_dist2(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                         ivar.data_ptr(), mean.data_ptr(), grad_spike.data_ptr(),
                                         grad_xhat.data_ptr(), grad_xhatx.data_ptr(),

@@ -233,3 +233,62 @@ def test_layer_parameters_carry_the_reference_names_and_order():
         if "weight_bn" in names:
             assert layer.train_bn is True and layer.factor is None, what
             assert bool((layer.weight_bn == 1).all()) and bool((layer.running_mean == 0).all()), what
+
+
+def test_ctypes_helpers_reject_mismatched_buffers_before_any_launch():
+    """The C ABI sees pointers only and sizes everything from ``spatial``; the ctypes helpers are the
+    one place that can catch a buffer that is too small or of another type.  Host tensors suffice to
+    show that the size checks come first (a consistent set of host tensors is then refused for
+    living on the host)."""
+    from snn_gpu_training_bptt_amd import lif_cabi
+    x = torch.zeros(4, 2, 8, 3, 3)
+    per_channel = torch.ones(8)
+    with pytest.raises(ValueError, match="spike has shape"):
+        lif_cabi.fire_s_fp_into(x, torch.zeros(4, 2, 8, 3, 2), 0.25, 0.5)
+    with pytest.raises(ValueError, match="grad_spatial has dtype"):
+        lif_cabi.fire_bp_into(x, x.clone(), x.double(), 0.25, 0.5, 1.0, 0.5)
+    with pytest.raises(ValueError, match="mem has shape"):
+        lif_cabi.fire_us_fp_into(x, x[:3].clone(), None, 0.25, 0.5)
+    long_window = torch.zeros(1030, 1, 4)
+    with pytest.raises(ValueError, match="needs a workspace"):
+        lif_cabi.fire_bp_into(long_window, long_window.clone(), long_window.clone(), 0.25, 0.5, 1.0, 0.5)
+    with pytest.raises(ValueError, match="workspace holds 16 bytes"):
+        lif_cabi.fire_bp_into(long_window, long_window.clone(), long_window.clone(), 0.25, 0.5, 1.0, 0.5,
+                              workspace=torch.zeros(16, dtype=torch.uint8))
+    with pytest.raises(ValueError, match="ivar has 4 values"):
+        lif_cabi.bn_fire_s_fp_into(x, per_channel, per_channel, per_channel, per_channel, torch.ones(4),
+                                   x.clone(), 1e-5, 0.25, 0.5)
+    with pytest.raises(ValueError, match="grad_weight has dtype"):
+        lif_cabi.bn_fire_bp_into(x, per_channel, per_channel, per_channel, per_channel, x.clone(), x.clone(),
+                                 per_channel.double(), per_channel, 0.25, 0.5, 1.0, 0.5,
+                                 torch.zeros(1 << 16, dtype=torch.uint8))
+    with pytest.raises(ValueError, match="workspace must be a uint8 tensor"):
+        lif_cabi.bn_fire_bp_into(x, per_channel, per_channel, per_channel, per_channel, x.clone(), x.clone(),
+                                 per_channel.clone(), per_channel.clone(), 0.25, 0.5, 1.0, 0.5,
+                                 torch.zeros(1 << 16))
+    with pytest.raises(ValueError, match="snnlif_bn_fire_bp needs"):
+        lif_cabi.bn_fire_bp_into(x, per_channel, per_channel, per_channel, per_channel, x.clone(), x.clone(),
+                                 per_channel.clone(), per_channel.clone(), 0.25, 0.5, 1.0, 0.5,
+                                 torch.zeros(8, dtype=torch.uint8))
+    with pytest.raises(ValueError, match="grad_xhatx has 3 values"):
+        lif_cabi.bn_fire_bp_dist2_into(x, per_channel, per_channel, per_channel, per_channel, x.clone(),
+                                       per_channel, torch.ones(3), x.clone(), 0.25, 0.5, 1.0, 0.5)
+    # sizes and types all consistent: only now is the device looked at
+    with pytest.raises(ValueError, match="device tensor required"):
+        lif_cabi.fire_s_fp_into(x, x.clone(), 0.25, 0.5)
+
+
+def test_batch_norm_workspace_follows_the_partial_sum_layout():
+    """Two partial sums per wavefront of sweep 1 (ceil(HW/64) per plane) for planes of at least 32
+    positions, two per neuron plus the split staging otherwise, plus two values per channel."""
+    from snn_gpu_training_bptt_amd import lif_cabi
+    f32, f64 = lif_cabi.DTYPE_F32, lif_cabi.DTYPE_F64
+    need = lif_cabi.bn_fire_bp_workspace_bytes
+    assert need(f32, 8, 64, 128, 1024) == 4 * (2 * 64 * 128 * 16 + 2 * 128)
+    assert need(f32, 8, 4, 6, 49) == 4 * (2 * 4 * 6 * 1 + 2 * 6)
+    assert need(f32, 8, 4, 6, 65) == 4 * (2 * 4 * 6 * 2 + 2 * 6)
+    assert need(f64, 8, 4, 6, 65) == 2 * need(f32, 8, 4, 6, 65)
+    # 31 positions: one lane per neuron; S = min(B, 2048 / C) splits of the batch axis
+    assert need(f32, 8, 4, 6, 31) == 4 * (2 * 4 * 6 * 31 + 2 * 4 * 6 + 2 * 6)
+    assert need(f32, 8, 64, 1024, 1) == 4 * (2 * 64 * 1024 + 2 * 2 * 1024 + 2 * 1024)
+    assert need(f32, 0, 4, 6, 31) == 0 and need(lif_cabi.DTYPE_BF16, 8, 4, 6, 31) == 0

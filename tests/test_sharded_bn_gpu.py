@@ -138,8 +138,12 @@ def test_argument_checks_of_the_halves(cabi):
     x, g, w, b, var, mean = make((4, 2, 3, 2, 2), seed=44)
     out = [torch.empty_like(w) for _ in range(4)]
     small = torch.empty(8, dtype=torch.uint8, device="cuda")
-    with pytest.raises(cabi.SnnlifError, match="workspace"):
+    with pytest.raises(ValueError, match="workspace"):     # the ctypes helper checks sizes first
         cabi.bn_fire_bp_dist1_into(x, w, b, var, mean, g, *out, ALPHA, THRESH, BETA, INTERVAL, small)
+    rc = lib.snnlif_bn_fire_bp_dist1(x.data_ptr(), w.data_ptr(), b.data_ptr(), var.data_ptr(), mean.data_ptr(),
+                                     g.data_ptr(), *(t.data_ptr() for t in out), f32, 4, 2, 3, 4, ALPHA, THRESH,
+                                     BETA, INTERVAL, small.data_ptr(), small.numel(), None)
+    assert rc == cabi.ERR_WORKSPACE
 
 
 @pytest.mark.parametrize("shape,dim_bn", [((6, 4, 8), (0, 1)), ((6, 4, 8, 8, 8), (0, 1, 3, 4))])
