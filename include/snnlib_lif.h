@@ -50,6 +50,7 @@ extern "C" {
 #define SNNLIF_ERR_DTYPE      -2 /* dtype is not one of SNNLIF_DTYPE_* */
 #define SNNLIF_ERR_WORKSPACE  -3 /* workspace missing or smaller than snnlif_fire_bp_workspace_bytes() */
 #define SNNLIF_ERR_ALIGN      -4 /* a pointer is not aligned to its element size */
+#define SNNLIF_ERR_SCRATCH    -6 /* shape needs more than SNNLIF_STATIC_SCRATCH_BYTES (snnlif_bn_fire_bp_static) */
 #define SNNLIF_ERR_UNSUPPORTED -5 /* valid arguments this entry point does not implement (see its comment) */
 
 /* Every T up to this keeps the whole recomputed membrane potential in registers in the backward
@@ -58,6 +59,10 @@ extern "C" {
 /* Largest T for which snnlif_fire_bp needs no workspace: up to here longer windows are processed
  * in register-sized segments whose boundary potentials live in LDS (16 bytes per neuron-step). */
 #define SNNLIF_BP_NO_WORKSPACE_MAX_T 1024
+
+/* Size of the fixed device array snnlif_bn_fire_bp_static works in (held once per GPU the library
+ * runs on, for the life of the process). */
+#define SNNLIF_STATIC_SCRATCH_BYTES (16u << 20)
 
 /* ABI version of the loaded library (== SNNLIF_ABI_VERSION it was built with). */
 int snnlif_abi_version(void);
@@ -178,6 +183,27 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
                       void* grad_weight, void* grad_bias, int dtype, int64_t T, int64_t B, int64_t C,
                       int64_t HW, float alpha, float thresh, float beta, float interval,
                       void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * snnlif_bn_fire_bp for callers that can neither allocate device memory nor hand in a workspace: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference (whose bn_fire_bp_cuda allocates five temporaries per call,
+ * snnlib/cuda/snn_kernel_bp.cu:700, 711-714).  Same arguments, checks, kernels and results (bit for bit)
+ * as snnlif_bn_fire_bp, minus the workspace: the partial sums live in a fixed device array of
+ * SNNLIF_STATIC_SCRATCH_BYTES that the library holds once per GPU.  Shapes for which
+ * snnlif_bn_fire_bp_workspace_bytes() exceeds that size return SNNLIF_ERR_SCRATCH and launch nothing
+ * (at fp32: more than about 2 million wavefront partials B*C*ceil(HW/64) when HW >= 32, or about
+ * 2 million neurons B*C*HW when HW < 32).  The call allocates and frees nothing.  The first call made
+ * with a given device current resolves that device's copy of the array (make it outside graph
+ * capture); all calls on one GPU share the array, so two calls whose kernels may overlap on that GPU
+ * (different streams without an ordering between them) race -- order them.  Nothing needs to be
+ * cleared between calls: every value read from the array is written earlier in the same call.
+ */
+int snnlif_bn_fire_bp_static(const void* spatial, const void* weight, const void* bias,
+                             const void* ivar, const void* mean, const void* grad_spike,
+                             void* grad_spatial, void* grad_weight, void* grad_bias, int dtype,
+                             int64_t T, int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
+                             float beta, float interval, void* stream);
 
 /*
  * The same backward in the two halves that a batch sharded over several GPUs runs on either side of

@@ -1,7 +1,17 @@
 // C ABI of libsnnlif_gfx950.so (include/snnlib_lif.h): argument checks and dtype dispatch in front
-// of the per-dtype kernel launchers.  No device code lives in this file.
+// of the per-dtype kernel launchers.  No kernel lives in this file; the only device-side object is
+// the fixed scratch array behind snnlif_bn_fire_bp_static.
+#include <atomic>
+
 #include "lif_bn.h"
 #include "lif_kernels.h"
+
+// Device memory of the one entry point that may not take a workspace from its caller
+// (snnlif_bn_fire_bp_static).  Every GPU the library runs on holds its own copy of this array, at its
+// own address, until the process ends.  In host code the name below is only a handle for
+// hipGetSymbolAddress: it is never passed to a kernel or to a memory routine; static_scratch() hands
+// out the device address instead.
+static __device__ __align__(256) unsigned char scratch[SNNLIF_STATIC_SCRATCH_BYTES];
 
 namespace snnlif {
 thread_local KernelTimer tl_kernel_timer;
@@ -16,6 +26,29 @@ inline size_t arith_size(int dtype) {
         case SNNLIF_DTYPE_BF16: return sizeof(float);
         default: return 0;
     }
+}
+
+// Device address of `scratch` on the current device, resolved on the first call made with that
+// device current and kept per device.  Returns SNNLIF_OK, SNNLIF_ERR_ARG for a device ordinal beyond
+// the table, or the hipError_t of the failing runtime call.
+constexpr int kMaxDevices = 64;
+std::atomic<void*> g_scratch_address[kMaxDevices];
+
+int static_scratch(void** out) {
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return static_cast<int>(err);
+    if (device < 0 || device >= kMaxDevices) return SNNLIF_ERR_ARG;
+    void* address = g_scratch_address[device].load(std::memory_order_acquire);
+    if (address == nullptr) {
+        // two threads racing here resolve the same address; the second store is harmless
+        err = hipGetSymbolAddress(&address, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return static_cast<int>(err);
+        if (address == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+        g_scratch_address[device].store(address, std::memory_order_release);
+    }
+    *out = address;
+    return SNNLIF_OK;
 }
 
 inline int shape_error(int64_t T, int64_t N) {
@@ -46,6 +79,7 @@ const char* snnlif_strerror(int code) {
         case SNNLIF_ERR_DTYPE: return "snnlif: unsupported dtype (expected SNNLIF_DTYPE_F32, _F64 or _BF16)";
         case SNNLIF_ERR_WORKSPACE: return "snnlif: workspace missing or smaller than snnlif_fire_bp_workspace_bytes()";
         case SNNLIF_ERR_ALIGN: return "snnlif: pointer not aligned to its element size (workspace: 16 bytes)";
+        case SNNLIF_ERR_SCRATCH: return "snnlif: this shape needs more scratch memory than the library's fixed array holds (SNNLIF_STATIC_SCRATCH_BYTES); call snnlif_bn_fire_bp with a workspace instead";
         case SNNLIF_ERR_UNSUPPORTED: return "snnlif: not implemented for these arguments (batch-norm fire: fp32 / fp64 only, backward T <= 1024)";
         default: break;
     }
@@ -231,6 +265,35 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
     const int rc = bn_backward_checks(dtype, T, B, C, HW, ptrs, 9, true, workspace, workspace_bytes,
                                       &es, &empty);
     if (rc != SNNLIF_OK || empty) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_backward_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean), CF(grad_spike),
+                                MF(grad_spatial), MF(grad_weight), MF(grad_bias), T, B, C, HW, alpha,
+                                thresh, beta, interval, MF(workspace), st),
+        snnlif::bn_backward_f64(CD(spatial), CD(weight), CD(bias), CD(ivar), CD(mean), CD(grad_spike),
+                                MD(grad_spatial), MD(grad_weight), MD(grad_bias), T, B, C, HW, alpha,
+                                thresh, beta, interval, MD(workspace), st));
+}
+
+int snnlif_bn_fire_bp_static(const void* spatial, const void* weight, const void* bias,
+                             const void* ivar, const void* mean, const void* grad_spike,
+                             void* grad_spatial, void* grad_weight, void* grad_bias, int dtype,
+                             int64_t T, int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
+                             float beta, float interval, void* stream) {
+    const void* ptrs[9] = {spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
+                           grad_bias};
+    size_t es = 0;
+    bool empty = false;
+    int rc = bn_backward_checks(dtype, T, B, C, HW, ptrs, 9, false, nullptr, 0, &es, &empty);
+    if (rc != SNNLIF_OK || empty) return rc;
+    if (snnlif::bn_backward_workspace_elems(B, C, HW) * es > SNNLIF_STATIC_SCRATCH_BYTES)
+        return SNNLIF_ERR_SCRATCH;
+    void* workspace = nullptr;
+    rc = static_scratch(&workspace);
+    if (rc != SNNLIF_OK) return rc;
+    // Every value the reduction reads from the scratch array is written by sweep 1 of this same call,
+    // so nothing has to be cleared between calls.
     hipStream_t st = static_cast<hipStream_t>(stream);
     return SNNLIF_BN_DISPATCH(
         es,

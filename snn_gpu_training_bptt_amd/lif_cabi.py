@@ -12,7 +12,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "lib", "libsnnlif_gfx950.so")
 
 DTYPE_F32, DTYPE_F64, DTYPE_BF16 = 0, 1, 2
-OK, ERR_ARG, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_UNSUPPORTED = 0, -1, -2, -3, -4, -5
+OK, ERR_ARG, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_UNSUPPORTED, ERR_SCRATCH = 0, -1, -2, -3, -4, -5, -6
+STATIC_SCRATCH_BYTES = 16 << 20
 BP_FUSED_MAX_T = 32
 BP_NO_WORKSPACE_MAX_T = 1024
 
@@ -31,6 +32,7 @@ SYMBOLS = {
     "snnlif_bn_fire_s_recompute": (_int, [_vp] * 6 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_bn_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "snnlif_bn_fire_bp": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
+    "snnlif_bn_fire_bp_static": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp]),
     "snnlif_bn_fire_bp_dist1": (_int, [_vp] * 10 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
     "snnlif_bn_fire_bp_dist2": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp]),
 }
@@ -257,13 +259,40 @@ def bn_fire_bp_into(spatial, weight, bias, ivar, mean, grad_spike, grad_spatial,
     return grad_spatial, grad_weight, grad_bias
 
 
+def bn_fire_bp_static_into(spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
+                           grad_bias, alpha, thresh, beta, interval):
+    """``snnlif_bn_fire_bp_static``: the same backward with its partial sums in the library's fixed
+    device array instead of a caller workspace (shapes beyond it raise ``SnnlifError`` with code
+    ``ERR_SCRATCH``)."""
+    T, B, C, HW = _bn_dims(spatial)
+    _require_like(spatial, grad_spike=grad_spike, grad_spatial=grad_spatial)
+    _require_per_channel(spatial, C, weight=weight, bias=bias, ivar=ivar, mean=mean,
+                         grad_weight=grad_weight, grad_bias=grad_bias)
+    _require_dense_gpu(spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
+                       grad_bias)
+    rc = load().snnlif_bn_fire_bp_static(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
+                                         ivar.data_ptr(), mean.data_ptr(), grad_spike.data_ptr(),
+                                         grad_spatial.data_ptr(), grad_weight.data_ptr(),
+                                         grad_bias.data_ptr(), _torch_dtype_code(spatial), T, B, C,
+                                         HW, alpha, thresh, beta, interval, _stream_handle(spatial))
+    _check(rc, "snnlif_bn_fire_bp_static")
+    return grad_spatial, grad_weight, grad_bias
+
+
 def bn_fire_bp_dist1_into(spatial, weight, bias, ivar, mean, grad_spike, mean_gxhat, mean_gxhatx,
                           grad_weight, grad_bias, alpha, thresh, beta, interval, workspace):
     """``snnlif_bn_fire_bp_dist1`` on fp32 device tensors: the half of the backward before the
     all-reduce of a sharded batch."""
+    T, B, C, HW = _bn_dims(spatial)
+    _require_like(spatial, grad_spike=grad_spike)
+    _require_per_channel(spatial, C, weight=weight, bias=bias, ivar=ivar, mean=mean,
+                         mean_gxhat=mean_gxhat, mean_gxhatx=mean_gxhatx, grad_weight=grad_weight,
+                         grad_bias=grad_bias)
+    _require_workspace(spatial, workspace,
+                       bn_fire_bp_workspace_bytes(_torch_dtype_code(spatial), T, B, C, HW),
+                       "snnlif_bn_fire_bp_dist1")
     _require_dense_gpu(spatial, weight, bias, ivar, mean, grad_spike, mean_gxhat, mean_gxhatx,
                        grad_weight, grad_bias, workspace)
-    T, B, C, HW = _bn_dims(spatial)
     rc = load().snnlif_bn_fire_bp_dist1(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                         ivar.data_ptr(), mean.data_ptr(), grad_spike.data_ptr(),
                                         mean_gxhat.data_ptr(), mean_gxhatx.data_ptr(),

@@ -45,6 +45,10 @@ def test_constants_match_the_header():
     assert int(macros["SNNLIF_ERR_DTYPE"]) == lif_cabi.ERR_DTYPE
     assert int(macros["SNNLIF_ERR_WORKSPACE"]) == lif_cabi.ERR_WORKSPACE
     assert int(macros["SNNLIF_ERR_ALIGN"]) == lif_cabi.ERR_ALIGN
+    assert int(macros["SNNLIF_ERR_UNSUPPORTED"]) == lif_cabi.ERR_UNSUPPORTED
+    assert int(macros["SNNLIF_ERR_SCRATCH"]) == lif_cabi.ERR_SCRATCH
+    shift = re.search(r"#define\s+SNNLIF_STATIC_SCRATCH_BYTES\s+\((\d+)u\s*<<\s*(\d+)\)", text)
+    assert int(shift.group(1)) << int(shift.group(2)) == lif_cabi.STATIC_SCRATCH_BYTES
     assert int(macros["SNNLIF_BP_FUSED_MAX_T"]) == lif_cabi.BP_FUSED_MAX_T
     assert int(macros["SNNLIF_BP_NO_WORKSPACE_MAX_T"]) == lif_cabi.BP_NO_WORKSPACE_MAX_T
     lib = lif_cabi.load()
@@ -292,3 +296,20 @@ def test_batch_norm_workspace_follows_the_partial_sum_layout():
     assert need(f32, 8, 4, 6, 31) == 4 * (2 * 4 * 6 * 31 + 2 * 4 * 6 + 2 * 6)
     assert need(f32, 8, 64, 1024, 1) == 4 * (2 * 64 * 1024 + 2 * 2 * 1024 + 2 * 1024)
     assert need(f32, 0, 4, 6, 31) == 0 and need(lif_cabi.DTYPE_BF16, 8, 4, 6, 31) == 0
+
+
+def test_static_scratch_backward_refuses_oversized_shapes_without_a_gpu():
+    """The size check of the entry point that allocates nothing comes before any device call, so it
+    can be seen here with stand-in (aligned, never dereferenced) pointers."""
+    from snn_gpu_training_bptt_amd import lif_cabi
+    lib = lif_cabi.load()
+    fake = [ctypes.c_void_p(4096)] * 9
+    tail = (0.25, 0.5, 1.0, 0.5, None)
+    f32 = lif_cabi.DTYPE_F32
+    B, C, HW = 3 << 10, 1 << 10, 1       # 3 Mi neurons, one lane each: 24 MiB of partial sums
+    assert lif_cabi.bn_fire_bp_workspace_bytes(f32, 4, B, C, HW) > lif_cabi.STATIC_SCRATCH_BYTES
+    assert lib.snnlif_bn_fire_bp_static(*fake, f32, 4, B, C, HW, *tail) == lif_cabi.ERR_SCRATCH
+    assert lib.snnlif_bn_fire_bp_static(*fake, lif_cabi.DTYPE_BF16, 4, 2, 8, 1, *tail) == lif_cabi.ERR_UNSUPPORTED
+    assert lib.snnlif_bn_fire_bp_static(*[None] * 9, f32, 4, 2, 8, 1, *tail) == lif_cabi.ERR_ARG
+    assert lib.snnlif_bn_fire_bp_static(*[None] * 9, f32, 0, 2, 8, 1, *tail) == lif_cabi.OK
+    assert "SNNLIF_STATIC_SCRATCH_BYTES" in lif_cabi.strerror(lif_cabi.ERR_SCRATCH)
