@@ -19,6 +19,13 @@ pre-allocated outputs.  The default workload is the headline configuration
                  mean duration, measured inside the timed region with HIP events attached to the
                  dispatches (kernel begin / kernel end) of about 25 steps spread evenly over it,
                  against the 8 TB/s HBM peak.  ``fwd`` and ``fwd_bwd`` give the same figure for the forward kernel (8 B) and for the pair (20 B).
+* ``roofline.cold`` the same kernels with nothing of ``x`` left in the 256 MB memory-side cache when
+                 the backward starts: several independent (x, g, spike, grad_x) sets of the workload's
+                 shape, all forwards first, then all backwards, so that at least three other tensors'
+                 worth of traffic lies between a tensor's forward and its backward (a deep network
+                 puts whole layers there).  Kernel durations from the same attached events.  The
+                 figures outside ``cold`` come from the step loop on one set, where the backward runs
+                 right after the forward and finds part of ``x`` still cached.
 * ``cpu_baseline`` the pure-PyTorch restatement of the reference's gold path
                  (``oracle/gold_fire.py``) on the host cores, forward + autograd backward on the same
                  inputs, best of 3 after a warm-up; its outputs also serve as the parity check of
@@ -56,13 +63,27 @@ WORKLOADS = {
     "cfg5": ((16, 128, 512, 16, 16), 0.5, 1.0, "float32"),
     "cfg5_bf16": ((16, 128, 512, 16, 16), 0.5, 1.0, "bfloat16"),
 }
-# HBM bytes per launch of the backward kernel, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of
-# this file (each counter scaled by its reading for a plain device copy of the same tensor:
-# --copy-calibration); the summary with the commands is profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt.
-# Counters cannot be read from inside this process, so workloads without a profiled figure report null.
-# bn_fire: the three backward kernels together, profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt.
-MEASURED_TRAFFIC_BYTES = {"cfg2": 805276475, "bn_fire": 1346500000}
+# HBM bytes per launch of the backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
+# of this file (each counter scaled by its reading for a plain device copy of the same tensor:
+# --copy-calibration).  Counters cannot be read from inside this process, so the figures are kept here
+# with the profile summary they come from; a workload without a profiled figure reports null.
+# "hot": the kernel of the step loop (SNNLIF_KEEP_SPATIAL), "cold": the streamed kernel of the cold leg.
+# bn_fire: the three backward kernels together.
+MEASURED_TRAFFIC = {
+    "cfg2": {"hot": 805276475, "cold": None, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt"},
+    "bn_fire": {"hot": 1346500000, "cold": None, "source": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt"},
+}
+HEADLINE = "cfg2"
 METRIC = "LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T=8,B=64,C=128,32x32"
+
+
+def metric_name(workload, shape, dtype_name):
+    """The headline configuration carries the metric's published name; every other workload says
+    which shape it ran."""
+    if workload == HEADLINE:
+        return METRIC
+    T, B, C, H, W = shape
+    return f"LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T={T},B={B},C={C},{H}x{W} {dtype_name} ({workload})"
 
 
 def make_inputs(torch, shape, mean, std, dtype):
@@ -93,6 +114,67 @@ def cpu_baseline(torch, x, g, repeats=3):
         outs = (s.detach(), xr.grad.detach())
         del u, s, xr
     return best, threads, outs
+
+
+def cold_cache_leg(torch, lif_cabi, x, g, spike_expected, bytes_fwd, bytes_bwd, rounds=6):
+    """Forward and backward kernel durations when the backward cannot find ``x`` in the memory-side
+    cache: K independent tensor sets, all K forwards, then all K backwards, `rounds` times (after
+    one untimed round).  Between the forward and the backward of one set lie the other sets'
+    forwards and backwards, several times the cache's capacity.  Every dispatch carries its own
+    start/stop events; the wall clock over the timed rounds is reported too."""
+    tensor_bytes = x.numel() * x.element_size()
+    sets = 4 if tensor_bytes <= (512 << 20) else 2
+    while sets * 2 * tensor_bytes < (2 << 30):      # small tensors: enough sets to cycle 2 GiB
+        sets *= 2
+    sets = min(sets, 64)
+    xs = [x] + [x.clone() for _ in range(sets - 1)]
+    gs = [g] + [g.clone() for _ in range(sets - 1)]
+    spikes = [torch.empty_like(x) for _ in range(sets)]
+    gxs = [torch.empty_like(x) for _ in range(sets)]
+
+    def one_round(events):
+        for k in range(sets):
+            if events is not None:
+                lif_cabi.time_next_kernel(events[0][k][0], events[0][k][1])
+            lif_cabi.fire_s_fp_into(xs[k], spikes[k], ALPHA, THRESH, keep_spatial=False)
+        for k in range(sets):
+            if events is not None:
+                lif_cabi.time_next_kernel(events[1][k][0], events[1][k][1])
+            lif_cabi.fire_bp_into(xs[k], gs[k], gxs[k], ALPHA, THRESH, BETA, INTERVAL, keep_spatial=False)
+
+    ev = [[[[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(sets)]
+           for _ in range(2)] for _ in range(rounds)]
+    for per_round in ev:
+        for per_kind in per_round:
+            for pair in per_kind:
+                for e in pair:
+                    e.record()
+    one_round(None)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for r in range(rounds):
+        one_round(ev[r])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    fwd = [p[0].elapsed_time(p[1]) for per_round in ev for p in per_round[0]]
+    bwd = [p[0].elapsed_time(p[1]) for per_round in ev for p in per_round[1]]
+    fwd_ms, bwd_ms = sum(fwd) / len(fwd), sum(bwd) / len(bwd)
+    same = all(torch.equal(sp, spike_expected) for sp in spikes) and all(torch.equal(q, gxs[0]) for q in gxs[1:])
+    rate = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    return {
+        "what": f"{sets} independent tensor sets, all forwards then all backwards, {rounds} timed rounds after "
+                f"one untimed: {sets * 2 - 1} or more other tensors' traffic between a set's forward and its backward",
+        "sets": sets, "launches_timed": len(fwd),
+        "fwd": {"avg_launch_ms": fwd_ms, "achieved": rate(bytes_fwd, fwd_ms),
+                "frac": rate(bytes_fwd, fwd_ms) / HBM_PEAK_GBPS},
+        "bwd": {"avg_launch_ms": bwd_ms, "achieved": rate(bytes_bwd, bwd_ms),
+                "frac": rate(bytes_bwd, bwd_ms) / HBM_PEAK_GBPS},
+        "fwd_bwd": {"kernel_ms": fwd_ms + bwd_ms, "achieved": rate(bytes_fwd + bytes_bwd, fwd_ms + bwd_ms),
+                    "frac": rate(bytes_fwd + bytes_bwd, fwd_ms + bwd_ms) / HBM_PEAK_GBPS},
+        "wall_ms_per_pair": wall / (rounds * sets) * 1e3,
+        "neuron_steps_per_s": x.numel() * rounds * sets / wall,
+        "outputs_equal_across_sets": bool(same),
+    }
 
 
 def build_synthetic_snn(torch, fire_factory, seed=0):
@@ -272,7 +354,8 @@ def run_bn_fire(args):
                      "bound": "hbm", "algorithmic_bytes_per_launch": 20 * ns, "avg_launch_ms": bwd_ms,
                      "achieved": 20 * ns / (bwd_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": 20 * ns / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get("bn_fire"),
+                     "traffic": MEASURED_TRAFFIC["bn_fire"]["hot"],
+                     "traffic_source": MEASURED_TRAFFIC["bn_fire"]["source"],
                      "fwd": {"algorithmic_bytes_per_launch": 8 * ns, "avg_launch_ms": fwd_ms,
                              "achieved": 8 * ns / (fwd_ms * 1e-3) / 1e9,
                              "frac": 8 * ns / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
@@ -308,6 +391,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step", "bn_fire"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cold-leg", action="store_true",
+                    help="skip the cold-cache leg (roofline.cold)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain device copies of the input tensor (known size: one "
                          "read + one write of it) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
@@ -356,9 +441,11 @@ def main():
     ws_bytes = lif_cabi.fire_bp_workspace_bytes(code, T, n_steps_total // T)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
 
+    # The step loop runs the backward straight after the forward on the same input current, step after
+    # step, and says so (SNNLIF_KEEP_SPATIAL); the cold leg below makes no such promise.
     def step():
-        lif_cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
-        lif_cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws)
+        lif_cabi.fire_s_fp_into(x, spike, ALPHA, THRESH, keep_spatial=True)
+        lif_cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws, keep_spatial=True)
 
     for _ in range(args.warmup):
         step()
@@ -390,10 +477,10 @@ def main():
         ev = kev.get(k)
         if ev is not None:
             lif_cabi.time_next_kernel(ev[0], ev[1])
-        lif_cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+        lif_cabi.fire_s_fp_into(x, spike, ALPHA, THRESH, keep_spatial=True)
         if ev is not None:
             lif_cabi.time_next_kernel(ev[2], ev[3])
-        lif_cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws)
+        lif_cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws, keep_spatial=True)
     t_enqueued = time.perf_counter()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
@@ -413,7 +500,7 @@ def main():
     spike_rate = float(spike.float().mean().item())
 
     result = {
-        "metric": METRIC,
+        "metric": metric_name(args.workload, shape, dtype_name),
         "value": value,
         "unit": "neuron-steps/s",
         "n_gpus": 1,
@@ -440,7 +527,8 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": bwd_gbps / HBM_PEAK_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("hot"),
+            "traffic_source": MEASURED_TRAFFIC.get(args.workload, {}).get("source"),
             "algorithmic_bytes_per_launch": bytes_bwd,
             "avg_launch_ms": bwd_ms,
             "timing": f"HIP events attached to the dispatches (kernel begin / kernel end) of {len(kev)} of the "
@@ -452,6 +540,11 @@ def main():
                         "achieved": pair_gbps, "frac": pair_gbps / HBM_PEAK_GBPS},
         },
     }
+
+    if not args.no_cold_leg:
+        cold = cold_cache_leg(torch, lif_cabi, x, g, spike, bytes_fwd, bytes_bwd)
+        cold["bwd"]["traffic"] = MEASURED_TRAFFIC.get(args.workload, {}).get("cold")
+        result["roofline"]["cold"] = cold
 
     if not args.no_cpu_baseline:
         best, threads, (s_ref, gx_ref) = cpu_baseline(torch, x_cpu, g_cpu)

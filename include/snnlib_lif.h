@@ -21,7 +21,8 @@
  *     `workspace` argument.
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).  Calls only enqueue
  *     work; they never synchronise.
- *   - `dtype` selects the storage type of every tensor argument (see SNNLIF_DTYPE_*).  Arithmetic
+ *   - `dtype` selects the storage type of every tensor argument (see SNNLIF_DTYPE_*; the fire entry
+ *     points also take a cache hint, SNNLIF_KEEP_SPATIAL or SNNLIF_STREAM_SPATIAL, or-ed into it).  Arithmetic
  *     is IEEE fp32 for F32 and BF16 storage and fp64 for F64 storage, in the reference's operation
  *     order, without fused multiply-add contraction.
  *   - Return value: SNNLIF_OK (0), a negative SNNLIF_ERR_* argument error, or a positive
@@ -43,6 +44,23 @@ extern "C" {
 #define SNNLIF_DTYPE_F32  0 /* float storage, fp32 arithmetic (the reference's training dtype) */
 #define SNNLIF_DTYPE_F64  1 /* double storage, fp64 arithmetic */
 #define SNNLIF_DTYPE_BF16 2 /* bfloat16 storage, fp32 arithmetic, round-to-nearest-even stores */
+
+/*
+ * Cache hints, or-ed into the `dtype` argument of snnlif_fire_s_fp, snnlif_fire_us_fp and snnlif_fire_bp
+ * (accepted and without effect elsewhere; both at once: SNNLIF_ERR_DTYPE).  Results never depend on them.
+ * No counterpart in the reference.
+ *   SNNLIF_KEEP_SPATIAL    the caller will read `spatial` again soon -- the backward runs straight after
+ *       the forward, or the same input current is used step after step.  `spatial` is loaded with the
+ *       default cache policy, so that the 256 MB memory-side cache may keep it for its next reader,
+ *       and the launch shape is the one that serves cache hits best.
+ *   SNNLIF_STREAM_SPATIAL  it will not: `spatial` is streamed from HBM with the non-temporal hint like
+ *       every other tensor, and the launch shape is the one that streams best.  This is the case of a
+ *       network, where whole layers run between a layer's forward and its backward.
+ *   neither                tensors of more than 32 MiB are streamed, smaller ones kept (a tensor that
+ *       small is likely to be cache-resident whatever lies between its two readers).
+ */
+#define SNNLIF_KEEP_SPATIAL   0x100
+#define SNNLIF_STREAM_SPATIAL 0x200
 
 /* Return codes (hipError_t values are positive). */
 #define SNNLIF_OK              0

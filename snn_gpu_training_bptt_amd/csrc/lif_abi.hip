@@ -19,8 +19,19 @@ thread_local KernelTimer tl_kernel_timer;
 
 namespace {
 
+// `dtype` arguments carry the storage type in their low byte and the cache hints above it.
+constexpr int kHintBits = SNNLIF_KEEP_SPATIAL | SNNLIF_STREAM_SPATIAL;
+inline int storage_of(int dtype) { return dtype & 0xff; }
+inline snnlif::SpatialHint hint_of(int dtype) {
+    if (dtype & SNNLIF_KEEP_SPATIAL) return snnlif::SpatialHint::keep;
+    if (dtype & SNNLIF_STREAM_SPATIAL) return snnlif::SpatialHint::stream;
+    return snnlif::SpatialHint::none;
+}
+
+// Size of the arithmetic type; 0 for an unknown storage type, unknown flag bits or both hints at once.
 inline size_t arith_size(int dtype) {
-    switch (dtype) {
+    if (dtype < 0 || (dtype & ~(0xff | kHintBits)) != 0 || (dtype & kHintBits) == kHintBits) return 0;
+    switch (storage_of(dtype)) {
         case SNNLIF_DTYPE_F32: return sizeof(float);
         case SNNLIF_DTYPE_F64: return sizeof(double);
         case SNNLIF_DTYPE_BF16: return sizeof(float);
@@ -76,7 +87,7 @@ const char* snnlif_strerror(int code) {
     switch (code) {
         case SNNLIF_OK: return "success";
         case SNNLIF_ERR_ARG: return "snnlif: invalid argument (NULL tensor pointer, negative or overflowing T/N)";
-        case SNNLIF_ERR_DTYPE: return "snnlif: unsupported dtype (expected SNNLIF_DTYPE_F32, _F64 or _BF16)";
+        case SNNLIF_ERR_DTYPE: return "snnlif: unsupported dtype (expected SNNLIF_DTYPE_F32, _F64 or _BF16, optionally or-ed with SNNLIF_KEEP_SPATIAL or SNNLIF_STREAM_SPATIAL)";
         case SNNLIF_ERR_WORKSPACE: return "snnlif: workspace missing or smaller than snnlif_fire_bp_workspace_bytes()";
         case SNNLIF_ERR_ALIGN: return "snnlif: pointer not aligned to its element size (workspace: 16 bytes)";
         case SNNLIF_ERR_SCRATCH: return "snnlif: this shape needs more scratch memory than the library's fixed array holds (SNNLIF_STATIC_SCRATCH_BYTES); call snnlif_bn_fire_bp with a workspace instead";
@@ -95,10 +106,11 @@ int snnlif_fire_us_fp(const void* spatial, void* mem, void* spike, int dtype, in
     if (T == 0 || N == 0) return SNNLIF_OK;
     if (spatial == nullptr || (mem == nullptr && spike == nullptr)) return SNNLIF_ERR_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (dtype) {
-        case SNNLIF_DTYPE_F32: return snnlif::forward_f32(spatial, mem, spike, T, N, alpha, thresh, st);
-        case SNNLIF_DTYPE_F64: return snnlif::forward_f64(spatial, mem, spike, T, N, alpha, thresh, st);
-        default: return snnlif::forward_bf16(spatial, mem, spike, T, N, alpha, thresh, st);
+    const snnlif::SpatialHint keep = hint_of(dtype);
+    switch (storage_of(dtype)) {
+        case SNNLIF_DTYPE_F32: return snnlif::forward_f32(spatial, mem, spike, T, N, alpha, thresh, keep, st);
+        case SNNLIF_DTYPE_F64: return snnlif::forward_f64(spatial, mem, spike, T, N, alpha, thresh, keep, st);
+        default: return snnlif::forward_bf16(spatial, mem, spike, T, N, alpha, thresh, keep, st);
     }
 }
 
@@ -128,13 +140,14 @@ int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spati
     if (T == 0 || N == 0) return SNNLIF_OK;
     if (spatial == nullptr || grad_spike == nullptr || grad_spatial == nullptr) return SNNLIF_ERR_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    switch (dtype) {
+    const snnlif::SpatialHint keep = hint_of(dtype);
+    switch (storage_of(dtype)) {
         case SNNLIF_DTYPE_F32:
-            return snnlif::backward_f32(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, workspace, workspace_bytes, st);
+            return snnlif::backward_f32(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
         case SNNLIF_DTYPE_F64:
-            return snnlif::backward_f64(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, workspace, workspace_bytes, st);
+            return snnlif::backward_f64(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
         default:
-            return snnlif::backward_bf16(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, workspace, workspace_bytes, st);
+            return snnlif::backward_bf16(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
     }
 }
 
@@ -158,8 +171,9 @@ static size_t bn_element_size(int dtype, int* rc) {
         *rc = SNNLIF_ERR_DTYPE;
         return 0;
     }
-    if (dtype == SNNLIF_DTYPE_F32) return sizeof(float);
-    if (dtype == SNNLIF_DTYPE_F64) return sizeof(double);
+    // the cache hints are accepted and have no effect: both sweeps of the backward read x anyway
+    if (storage_of(dtype) == SNNLIF_DTYPE_F32) return sizeof(float);
+    if (storage_of(dtype) == SNNLIF_DTYPE_F64) return sizeof(double);
     *rc = SNNLIF_ERR_UNSUPPORTED;
     return 0;
 }

@@ -33,12 +33,22 @@
 //     with the missing rows replaced by zeros (no per-row control flow around live registers,
 //     which costs the compiler hundreds of VGPRs).
 //   * The op is element-wise and HBM-bound: no LDS, no cross-lane traffic, no MFMA.
-//   * Cache policy per stream: spikes and gradients are touched once and carry the non-temporal
-//     hint; the input current x is read by the forward and again by the backward, so it alone is
-//     loaded with the default policy and may stay in the 256 MB memory-side cache.  The forward
-//     walks the neuron axis upwards and the backward downwards, so whatever part of x is still
-//     cached when the backward starts (all of it up to 256 MiB, the most recently read part
-//     otherwise) is the part the backward asks for first.
+//   * Cache policy and launch shape follow what the caller says about the input current x
+//     (template parameter KEEP of the kernels, SNNLIF_KEEP_SPATIAL of the C ABI):
+//       - streamed (the default): x is read once per kernel from HBM, like every other tensor, with
+//         the non-temporal hint.  This is the case of a network, where whole layers run between a
+//         layer's forward and its backward.  Measured with nothing cached, the DRAM then prefers
+//         fewer and larger streams in flight: 256-thread workgroups throughout and the backward
+//         capped at 4-5 wavefronts per SIMD (+5-9 points of bandwidth over the shape below).
+//       - kept: the caller will read x again soon (the backward straight after the forward, the same
+//         x step after step).  x is then loaded with the default policy and may stay in the 256 MB
+//         memory-side cache, spikes and gradients keep the non-temporal hint so they do not displace
+//         it, the forward walks the neuron axis upwards and the backward downwards (whatever part of
+//         x is still cached when the backward starts is what it asks for first), and small
+//         workgroups with all 8 wavefronts per SIMD resident serve cache hits best.
+//     Without a word from the caller tensors of at most 32 MiB are treated as kept (at that size a
+//     launch is latency-bound and the tensor is likely to be cache-resident whatever lies between its
+//     two readers) and larger ones as streamed.
 //   * Built with -ffp-contract=off: each product and sum is rounded on its own, as PyTorch's
 //     element-wise CPU/GPU ops do, which makes spikes, potentials and gradients bit-identical to
 //     the per-op rounded reference arithmetic.
@@ -92,6 +102,24 @@
 #ifndef SNNLIF_BWD_DESCENDING
 #define SNNLIF_BWD_DESCENDING 1
 #endif
+// Tensors of at most this many bytes are handled as "kept" whatever the caller says (see above).
+#ifndef SNNLIF_RESIDENT_TENSOR_BYTES
+#define SNNLIF_RESIDENT_TENSOR_BYTES (size_t(32) << 20)
+#endif
+// Streamed policy: workgroup size of both kernels, wavefronts per SIMD of the backward for windows
+// of at most 8 rows / longer ones, of the forward for windows of more than 8 rows.
+#ifndef SNNLIF_STREAM_BLOCK
+#define SNNLIF_STREAM_BLOCK 256
+#endif
+#ifndef SNNLIF_STREAM_BWD_WAVES_SHORT
+#define SNNLIF_STREAM_BWD_WAVES_SHORT 5
+#endif
+#ifndef SNNLIF_STREAM_BWD_WAVES_LONG
+#define SNNLIF_STREAM_BWD_WAVES_LONG 4
+#endif
+#ifndef SNNLIF_STREAM_FWD_WAVES_LONG
+#define SNNLIF_STREAM_FWD_WAVES_LONG 4
+#endif
 // Rows of x the forward requests before consuming the first (windows longer than this are
 // streamed with the next group of rows in flight).
 #ifndef SNNLIF_FWD_ROWS
@@ -109,15 +137,28 @@
 namespace snnlif {
 
 // Wavefronts per SIMD the backward kernels allow themselves for a register window of `rows` time
-// steps.  A wavefront keeps 2*rows row requests in flight; past roughly 100 of them per SIMD the
-// streams of different wavefronts start to evict each other's DRAM pages, and measured bandwidth
-// drops (by 4 % at 16 rows and 9 % at 32 rows with all 8 wavefronts resident; windows of up to 8
-// rows are best left uncapped).  SNNLIF_BWD_MAX_WAVES overrides.
-constexpr int backward_waves(int rows) {
+// steps.  A wavefront keeps 2*rows row requests in flight.
+// Kept x (part of the traffic served by the memory-side cache): past roughly 100 requests per SIMD the
+// streams of different wavefronts start to evict each other's DRAM pages (-4 % at 16 rows and -9 % at
+// 32 rows with all 8 wavefronts resident; windows of up to 8 rows are best left uncapped).
+// Streamed x (everything from HBM): fewer wavefronts already pay for short windows (8 rows: 84 % of
+// peak at 5 wavefronts against 78 % at 8).  SNNLIF_BWD_MAX_WAVES overrides both.
+constexpr int backward_waves(int rows, bool keep = true) {
 #ifdef SNNLIF_BWD_MAX_WAVES
     return SNNLIF_BWD_MAX_WAVES;
 #else
+    if (!keep) return rows <= 8 ? SNNLIF_STREAM_BWD_WAVES_SHORT : SNNLIF_STREAM_BWD_WAVES_LONG;
     return rows <= 8 ? 8 : (rows <= 12 ? 5 : 4);
+#endif
+}
+
+// The forward keeps `rows` (twice that when the window is streamed in groups) requests per wavefront
+// in flight; only long streamed windows gain from a cap.
+constexpr int forward_waves(int rows, bool keep) {
+#ifdef SNNLIF_FWD_MAX_WAVES
+    return SNNLIF_FWD_MAX_WAVES;
+#else
+    return (!keep && rows > 8) ? SNNLIF_STREAM_FWD_WAVES_LONG : 8;
 #endif
 }
 
@@ -138,10 +179,24 @@ constexpr int kBwdBlock = SNNLIF_BWD_BLOCK;
 // so the forward switches later than the backward.
 constexpr size_t kSmallTensorBytes = SNNLIF_SMALL_TENSOR_BYTES;
 constexpr size_t kSmallTensorBytesFwd = SNNLIF_SMALL_TENSOR_BYTES_FWD;
-inline int forward_block(size_t tensor_bytes) {
+constexpr size_t kResidentTensorBytes = SNNLIF_RESIDENT_TENSOR_BYTES;
+// What the caller said about x: nothing, "will be read again soon" (SNNLIF_KEEP_SPATIAL) or "will not,
+// however small it is" (SNNLIF_STREAM_SPATIAL).
+enum class SpatialHint { none, keep, stream };
+
+// Whether a launch uses the "kept" form of a kernel: the caller's word, else by size (a tensor small
+// enough to be cache-resident anyway is kept).
+inline bool keep_policy(SpatialHint hint, size_t tensor_bytes) {
+    if (hint == SpatialHint::keep) return true;
+    if (hint == SpatialHint::stream) return false;
+    return tensor_bytes <= kResidentTensorBytes;
+}
+inline int forward_block(size_t tensor_bytes, bool keep = true) {
+    if (!keep) return SNNLIF_STREAM_BLOCK < kFwdBlock ? SNNLIF_STREAM_BLOCK : kFwdBlock;
     return (tensor_bytes <= kSmallTensorBytesFwd && kFwdBlock > 128) ? 128 : kFwdBlock;
 }
-inline int backward_block(size_t tensor_bytes, int small = 64) {
+inline int backward_block(size_t tensor_bytes, int small = 64, bool keep = true) {
+    if (!keep) return SNNLIF_STREAM_BLOCK < kBwdBlock ? SNNLIF_STREAM_BLOCK : kBwdBlock;
     return (tensor_bytes <= kSmallTensorBytes && kBwdBlock > small) ? small : kBwdBlock;
 }
 
@@ -256,10 +311,11 @@ __device__ __forceinline__ void lif_reverse_step(C& gu, C u, C g, C alpha, C thr
 // public op, the arithmetic type when it is the backward's workspace), V: neurons per lane,
 // TC: rows requested before the first is consumed.  MULTI = false: the whole window fits in TC
 // rows.  MULTI = true: the window is streamed TC rows at a time with the next TC rows already in
-// flight while the current ones are processed.
+// flight while the current ones are processed.  KEEP: x is loaded with the default cache policy
+// (see the file header); otherwise with the non-temporal hint.
 // ---------------------------------------------------------------------------------------------
-template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S>
-__global__ void __launch_bounds__(kFwdBlock)
+template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP>
+__global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(forward_waves(TC, KEEP))
 lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__ spike, int T,
                    int64_t N, int64_t nvec, typename Arith<S>::type alpha,
                    typename Arith<S>::type thresh) {
@@ -278,7 +334,8 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
         Pack<S, V> nxt[MULTI ? TC : 1];
 #pragma unroll
         for (int k = 0; k < TC; ++k) {
-            if (k < T) cur[k] = load_pack<S, V, false>(x + static_cast<int64_t>(k) * N + col);
+            if (k < T)
+                cur[k] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(k) * N + col);
         }
         for (int t0 = 0; t0 < T; t0 += TC) {
             if (MULTI && t0 + TC < T) {
@@ -286,8 +343,8 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
                 for (int k = 0; k < TC; ++k) {
                     const int t = t0 + TC + k;
                     if (t < T)
-                        nxt[MULTI ? k : 0] =
-                            load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
+                        nxt[MULTI ? k : 0] = load_pack<S, V, !KEEP>(
+                            x + static_cast<int64_t>(t) * N + col);
                 }
             }
 #pragma unroll
@@ -327,8 +384,9 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 // only produce values nobody reads) and the reverse sweep skips them.
 // Gradient rows are fetched in groups of at most GC, the newest time steps first; the fetch of the
 // next (earlier) group is issued before the current group is consumed.
+// KEEP: x is loaded with the default cache policy, otherwise with the non-temporal hint.
 // ---------------------------------------------------------------------------------------------
-template <typename S, int V, int TW, bool EXACT>
+template <typename S, int V, int TW, bool EXACT, bool KEEP = true>
 __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S* __restrict__ g,
                                                 S* __restrict__ gx, int rows, int64_t N,
                                                 int64_t col, typename Arith<S>::type (&uc)[V],
@@ -347,10 +405,11 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
 #pragma unroll
     for (int t = 0; t < TW; ++t) {
         if (EXACT) {
-            xin[t] = load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
+            xin[t] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(t) * N + col);
         } else {
             xin[t] = zero_pack<S, V>();
-            if (t < rows) xin[t] = load_pack<S, V, false>(x + static_cast<int64_t>(t) * N + col);
+            if (t < rows)
+                xin[t] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(t) * N + col);
         }
     }
     Pack<S, V> gbuf[2][GC];
@@ -423,8 +482,8 @@ __device__ __forceinline__ int64_t backward_column(int64_t v, int64_t nvec, int 
 // ---------------------------------------------------------------------------------------------
 // Fused backward for T <= TW: the whole time axis is one register window.
 // ---------------------------------------------------------------------------------------------
-template <typename S, int V, int TW, bool EXACT>
-__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
+template <typename S, int V, int TW, bool EXACT, bool KEEP>
+__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW, KEEP))
 lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
                           int T, int64_t N, int64_t nvec, typename Arith<S>::type alpha,
                           typename Arith<S>::type thresh, typename Arith<S>::type beta,
@@ -441,8 +500,8 @@ lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* _
             sc[j] = C(0);
             gu[j] = C(0);
         }
-        backward_window<S, V, TW, EXACT>(x, g, gx, T, N, col, uc, sc, gu, alpha, thresh, beta,
-                                         interval);
+        backward_window<S, V, TW, EXACT, KEEP>(x, g, gx, T, N, col, uc, sc, gu, alpha, thresh, beta,
+                                               interval);
     }
 }
 
@@ -664,45 +723,55 @@ inline int with_vec(int v, F&& f) {
     return f(std::integral_constant<int, 1>());
 }
 
-template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S>
-int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
-                      hipStream_t stream) {
+// One forward launch with TC rows per group.
+template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP>
+int launch_forward_rows(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
+                        int threads, hipStream_t stream) {
     using C = typename Arith<S>::type;
     const int64_t nvec = N / V;
-    const int threads = forward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S));
-    const dim3 grid(grid_for(nvec, threads)), block(threads);
-    const int Ti = static_cast<int>(T);
-    constexpr int TC = SNNLIF_FWD_ROWS;
-    if (T <= 4 && TC > 4) {
-        launch_kernel(lif_forward_kernel<S, M, V, 4, false, WRITE_U, WRITE_S>, grid,
-                           block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
-    } else if (T <= TC) {
-        launch_kernel(lif_forward_kernel<S, M, V, TC, false, WRITE_U, WRITE_S>, grid,
-                           block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
-    } else {
-        launch_kernel(lif_forward_kernel<S, M, V, TC, true, WRITE_U, WRITE_S>, grid,
-                           block, 0, stream, x, mem, spike, Ti, N, nvec, C(alpha), C(thresh));
-    }
-    return launch_status();
-}
-
-// Windows of at most SNNLIF_WIDE_LANE_MAX_T (<= 4) steps: only the 4-row instantiation is needed.
-template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S>
-int launch_forward_short(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha,
-                         float thresh, hipStream_t stream) {
-    using C = typename Arith<S>::type;
-    static_assert(SNNLIF_WIDE_LANE_MAX_T <= 4, "the short-window forward holds 4 rows");
-    const int64_t nvec = N / V;
-    const int threads = forward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S));
-    launch_kernel(lif_forward_kernel<S, M, V, 4, false, WRITE_U, WRITE_S>,
+    launch_kernel(lif_forward_kernel<S, M, V, TC, MULTI, WRITE_U, WRITE_S, KEEP>,
                   dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
                   static_cast<int>(T), N, nvec, C(alpha), C(thresh));
     return launch_status();
 }
 
-template <typename S, typename M, bool WRITE_U, bool WRITE_S>
-int launch_forward(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
-                   hipStream_t stream) {
+// Rows per group by window length.  Kept x: the whole window up to SNNLIF_FWD_ROWS rows, longer ones
+// streamed in groups of that many.  Streamed x: windows of up to 16 rows are requested whole (a
+// window of 9-16 rows as one group measures +5-8 points over two groups of 8), longer ones go in
+// groups of 16.
+template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S, bool KEEP>
+int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
+                     hipStream_t stream) {
+    const int threads =
+        forward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S), KEEP);
+    constexpr int TC = SNNLIF_FWD_ROWS;
+    constexpr int TL = KEEP ? TC : 2 * TC;  // rows per group of the long-window form
+#define SNNLIF_FWD_LAUNCH(ROWS, MULTI)                                                           \
+    launch_forward_rows<S, M, V, ROWS, MULTI, WRITE_U, WRITE_S, KEEP>(x, mem, spike, T, N, alpha,  \
+                                                                      thresh, threads, stream)
+    if (T <= 4 && TC > 4) return SNNLIF_FWD_LAUNCH(4, false);
+    if (T <= TC) return SNNLIF_FWD_LAUNCH(TC, false);
+    if constexpr (!KEEP) {
+        if (T <= TL) return SNNLIF_FWD_LAUNCH(TL, false);
+    }
+    return SNNLIF_FWD_LAUNCH(TL, true);
+#undef SNNLIF_FWD_LAUNCH
+}
+
+// Windows of at most SNNLIF_WIDE_LANE_MAX_T (<= 4) steps: only the 4-row instantiation is needed.
+template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S, bool KEEP>
+int launch_forward_short(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha,
+                         float thresh, hipStream_t stream) {
+    static_assert(SNNLIF_WIDE_LANE_MAX_T <= 4, "the short-window forward holds 4 rows");
+    const int threads =
+        forward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S), KEEP);
+    return launch_forward_rows<S, M, V, 4, false, WRITE_U, WRITE_S, KEEP>(x, mem, spike, T, N, alpha,
+                                                                          thresh, threads, stream);
+}
+
+template <typename S, typename M, bool WRITE_U, bool WRITE_S, bool KEEP>
+int launch_forward_policy(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha,
+                          float thresh, hipStream_t stream) {
     // lanes are sized by the narrower of the two element types; the wider one (the fp32 workspace
     // behind bf16 storage) then moves V of its elements, at most 16 bytes
     constexpr size_t narrowest = sizeof(S) < sizeof(M) ? sizeof(S) : sizeof(M);
@@ -719,28 +788,40 @@ int launch_forward(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alp
         const int wv = pick_vec(widev, N, ptrs, elem, 3);
         return with_vec<widev>(wv, [&](auto vc) {
             constexpr int V = decltype(vc)::value;
-            return launch_forward_short<S, M, V, WRITE_U, WRITE_S>(x, mem, spike, T, N, alpha, thresh,
-                                                                   stream);
+            return launch_forward_short<S, M, V, WRITE_U, WRITE_S, KEEP>(x, mem, spike, T, N, alpha,
+                                                                         thresh, stream);
         });
     }
     const int v = pick_vec(maxv, N, ptrs, elem, 3);
     return with_vec<maxv>(v, [&](auto vc) {
         constexpr int V = decltype(vc)::value;
-        return launch_forward_v<S, M, V, WRITE_U, WRITE_S>(x, mem, spike, T, N, alpha, thresh, stream);
+        return launch_forward_v<S, M, V, WRITE_U, WRITE_S, KEEP>(x, mem, spike, T, N, alpha, thresh,
+                                                                 stream);
     });
+}
+
+// keep_x: what the caller said about x (see the file header); small tensors are always kept.
+template <typename S, typename M, bool WRITE_U, bool WRITE_S>
+int launch_forward(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
+                   SpatialHint keep_x, hipStream_t stream) {
+    if (keep_policy(keep_x, static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S)))
+        return launch_forward_policy<S, M, WRITE_U, WRITE_S, true>(x, mem, spike, T, N, alpha, thresh,
+                                                                   stream);
+    return launch_forward_policy<S, M, WRITE_U, WRITE_S, false>(x, mem, spike, T, N, alpha, thresh,
+                                                                stream);
 }
 
 template <typename S>
 int forward_dispatch(const void* x, void* mem, void* spike, int64_t T, int64_t N, float alpha,
-                     float thresh, hipStream_t stream) {
+                     float thresh, SpatialHint keep_x, hipStream_t stream) {
     const S* xs = static_cast<const S*>(x);
     S* ms = static_cast<S*>(mem);
     S* ss = static_cast<S*>(spike);
     if (mem != nullptr && spike != nullptr)
-        return launch_forward<S, S, true, true>(xs, ms, ss, T, N, alpha, thresh, stream);
+        return launch_forward<S, S, true, true>(xs, ms, ss, T, N, alpha, thresh, keep_x, stream);
     if (mem != nullptr)
-        return launch_forward<S, S, true, false>(xs, ms, nullptr, T, N, alpha, thresh, stream);
-    return launch_forward<S, S, false, true>(xs, nullptr, ss, T, N, alpha, thresh, stream);
+        return launch_forward<S, S, true, false>(xs, ms, nullptr, T, N, alpha, thresh, keep_x, stream);
+    return launch_forward<S, S, false, true>(xs, nullptr, ss, T, N, alpha, thresh, keep_x, stream);
 }
 
 // Register budget of the fused backward: TW*V arithmetic values for u plus two gradient
@@ -755,9 +836,9 @@ constexpr int fused_max_vec() {
     return cap < 1 ? 1 : (cap < hw ? cap : hw);
 }
 
-template <typename S, int TW>
-int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, float alpha,
-                          float thresh, float beta, float interval, hipStream_t stream) {
+template <typename S, int TW, bool KEEP>
+int launch_backward_fused_policy(const S* x, const S* g, S* gx, int64_t T, int64_t N, float alpha,
+                                 float thresh, float beta, float interval, hipStream_t stream) {
     using C = typename Arith<S>::type;
     constexpr int maxv = fused_max_vec<S, TW>();
     const void* ptrs[3] = {x, g, gx};
@@ -771,18 +852,29 @@ int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, f
         constexpr int V = decltype(vc)::value;
         const int64_t nvec = N / V;
         const int threads =
-            backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S));
+            backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S), 64, KEEP);
         const dim3 grid(grid_for(nvec, threads)), block(threads);
         const int Ti = static_cast<int>(T);
         if (exact) {
-            launch_kernel(lif_backward_fused_kernel<S, V, TW, true>, grid, block, 0, stream,
+            launch_kernel(lif_backward_fused_kernel<S, V, TW, true, KEEP>, grid, block, 0, stream,
                                x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval));
         } else if constexpr (can_be_inexact) {
-            launch_kernel(lif_backward_fused_kernel<S, V, TW, false>, grid, block, 0, stream,
+            launch_kernel(lif_backward_fused_kernel<S, V, TW, false, KEEP>, grid, block, 0, stream,
                                x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval));
         }
         return launch_status();
     });
+}
+
+template <typename S, int TW>
+int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, float alpha,
+                          float thresh, float beta, float interval, SpatialHint keep_x,
+                          hipStream_t stream) {
+    if (keep_policy(keep_x, static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S)))
+        return launch_backward_fused_policy<S, TW, true>(x, g, gx, T, N, alpha, thresh, beta, interval,
+                                                         stream);
+    return launch_backward_fused_policy<S, TW, false>(x, g, gx, T, N, alpha, thresh, beta, interval,
+                                                      stream);
 }
 
 template <typename S, int V>
@@ -799,7 +891,7 @@ int launch_backward_stream_v(const typename Arith<S>::type* mem, const S* g, S* 
 
 template <typename S>
 int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int64_t N, float alpha,
-                      float thresh, float beta, float interval, void* workspace,
+                      float thresh, float beta, float interval, SpatialHint keep_x, void* workspace,
                       size_t workspace_bytes, hipStream_t stream) {
     using C = typename Arith<S>::type;
     const S* x = static_cast<const S*>(x_);
@@ -812,7 +904,8 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
     // one in its zero-filled form.
 #define SNNLIF_BWD_WINDOW(TW)                                                                    \
     if (T <= TW)                                                                                 \
-        return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, stream);
+        return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, keep_x, \
+                                            stream);
     SNNLIF_BWD_WINDOW(1)
     SNNLIF_BWD_WINDOW(2)
     SNNLIF_BWD_WINDOW(3)
@@ -836,7 +929,8 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
     // straight-line form: zero-filling a 48-row window for T = 33 is slower than two segments.
 #define SNNLIF_BWD_WIDE_WINDOW(TW)                                                               \
     if (T == TW)                                                                                 \
-        return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, stream);
+        return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, keep_x, \
+                                            stream);
     SNNLIF_BWD_WIDE_WINDOW(40)
     SNNLIF_BWD_WIDE_WINDOW(48)
     SNNLIF_BWD_WIDE_WINDOW(56)
@@ -870,7 +964,7 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
     if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
     if (!aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
     C* mem = static_cast<C*>(workspace);
-    int rc = launch_forward<S, C, true, false>(x, mem, nullptr, T, N, alpha, thresh, stream);
+    int rc = launch_forward<S, C, true, false>(x, mem, nullptr, T, N, alpha, thresh, keep_x, stream);
     if (rc != SNNLIF_OK) return rc;
 
     constexpr int maxv = Arith<S>::kMaxVec < static_cast<int>(16 / sizeof(C))
@@ -890,9 +984,9 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
 // lif_bf16.hip; called from lif_abi.hip).
 #define SNNLIF_DECLARE_DTYPE(NAME)                                                                  \
     int forward_##NAME(const void* x, void* mem, void* spike, int64_t T, int64_t N, float alpha,    \
-                       float thresh, hipStream_t stream);                                           \
+                       float thresh, SpatialHint keep_x, hipStream_t stream);                              \
     int backward_##NAME(const void* x, const void* g, void* gx, int64_t T, int64_t N, float alpha,  \
-                        float thresh, float beta, float interval, void* workspace,                  \
+                        float thresh, float beta, float interval, SpatialHint keep_x, void* workspace,     \
                         size_t workspace_bytes, hipStream_t stream);
 SNNLIF_DECLARE_DTYPE(f32)
 SNNLIF_DECLARE_DTYPE(f64)
@@ -901,14 +995,14 @@ SNNLIF_DECLARE_DTYPE(bf16)
 
 #define SNNLIF_DEFINE_DTYPE(NAME, S)                                                                \
     int forward_##NAME(const void* x, void* mem, void* spike, int64_t T, int64_t N, float alpha,    \
-                       float thresh, hipStream_t stream) {                                          \
-        return forward_dispatch<S>(x, mem, spike, T, N, alpha, thresh, stream);                     \
+                       float thresh, SpatialHint keep_x, hipStream_t stream) {                             \
+        return forward_dispatch<S>(x, mem, spike, T, N, alpha, thresh, keep_x, stream);             \
     }                                                                                               \
     int backward_##NAME(const void* x, const void* g, void* gx, int64_t T, int64_t N, float alpha,  \
-                        float thresh, float beta, float interval, void* workspace,                  \
+                        float thresh, float beta, float interval, SpatialHint keep_x, void* workspace,     \
                         size_t workspace_bytes, hipStream_t stream) {                               \
-        return backward_dispatch<S>(x, g, gx, T, N, alpha, thresh, beta, interval, workspace,       \
-                                    workspace_bytes, stream);                                       \
+        return backward_dispatch<S>(x, g, gx, T, N, alpha, thresh, beta, interval, keep_x,          \
+                                    workspace, workspace_bytes, stream);                            \
     }
 
 }  // namespace snnlif

@@ -12,6 +12,8 @@ PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(PKG_DIR, "lib", "libsnnlif_gfx950.so")
 
 DTYPE_F32, DTYPE_F64, DTYPE_BF16 = 0, 1, 2
+# cache hints, or-ed into dtype: the caller will / will not read `spatial` again soon
+KEEP_SPATIAL, STREAM_SPATIAL = 0x100, 0x200
 OK, ERR_ARG, ERR_DTYPE, ERR_WORKSPACE, ERR_ALIGN, ERR_UNSUPPORTED, ERR_SCRATCH = 0, -1, -2, -3, -4, -5, -6
 STATIC_SCRATCH_BYTES = 16 << 20
 BP_FUSED_MAX_T = 32
@@ -153,18 +155,27 @@ def time_next_kernel(start_event, stop_event):
            "snnlif_time_next_kernel")
 
 
-def fire_s_fp_into(spatial, spike, alpha, thresh):
-    """``snnlif_fire_s_fp`` on torch tensors already resident on the GPU; writes ``spike``."""
+def _hinted(dtype_code, keep_spatial):
+    """``keep_spatial``: True -> SNNLIF_KEEP_SPATIAL, False -> SNNLIF_STREAM_SPATIAL, None -> no hint."""
+    if keep_spatial is None:
+        return dtype_code
+    return dtype_code | (KEEP_SPATIAL if keep_spatial else STREAM_SPATIAL)
+
+
+def fire_s_fp_into(spatial, spike, alpha, thresh, keep_spatial=None):
+    """``snnlif_fire_s_fp`` on torch tensors already resident on the GPU; writes ``spike``.
+    ``keep_spatial`` (True / False / None) selects the cache hint, see ``_hinted``."""
     _require_like(spatial, spike=spike)
     T, N = _dims(spatial)
     _require_dense_gpu(spatial, spike)
-    rc = load().snnlif_fire_s_fp(spatial.data_ptr(), spike.data_ptr(), _torch_dtype_code(spatial),
-                                 T, N, alpha, thresh, _stream_handle(spatial))
+    rc = load().snnlif_fire_s_fp(spatial.data_ptr(), spike.data_ptr(),
+                                 _hinted(_torch_dtype_code(spatial), keep_spatial), T, N, alpha,
+                                 thresh, _stream_handle(spatial))
     _check(rc, "snnlif_fire_s_fp")
     return spike
 
 
-def fire_us_fp_into(spatial, mem, spike, alpha, thresh):
+def fire_us_fp_into(spatial, mem, spike, alpha, thresh, keep_spatial=None):
     """``snnlif_fire_us_fp``; ``mem`` or ``spike`` may be None to skip that output."""
     _require_like(spatial, mem=mem, spike=spike)
     T, N = _dims(spatial)
@@ -172,8 +183,8 @@ def fire_us_fp_into(spatial, mem, spike, alpha, thresh):
     rc = load().snnlif_fire_us_fp(spatial.data_ptr(),
                                   mem.data_ptr() if mem is not None else None,
                                   spike.data_ptr() if spike is not None else None,
-                                  _torch_dtype_code(spatial), T, N, alpha, thresh,
-                                  _stream_handle(spatial))
+                                  _hinted(_torch_dtype_code(spatial), keep_spatial), T, N, alpha,
+                                  thresh, _stream_handle(spatial))
     _check(rc, "snnlif_fire_us_fp")
     return mem, spike
 
@@ -182,7 +193,8 @@ def fire_bp_workspace_bytes(dtype_code, T, N):
     return int(load().snnlif_fire_bp_workspace_bytes(dtype_code, T, N))
 
 
-def fire_bp_into(spatial, grad_spike, grad_spatial, alpha, thresh, beta, interval, workspace=None):
+def fire_bp_into(spatial, grad_spike, grad_spatial, alpha, thresh, beta, interval, workspace=None,
+                 keep_spatial=None):
     """``snnlif_fire_bp``; ``workspace`` is a uint8 device tensor when the shape needs one."""
     _require_like(spatial, grad_spike=grad_spike, grad_spatial=grad_spatial)
     T, N = _dims(spatial)
@@ -192,8 +204,8 @@ def fire_bp_into(spatial, grad_spike, grad_spatial, alpha, thresh, beta, interva
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
     _require_dense_gpu(spatial, grad_spike, grad_spatial, workspace)
     rc = load().snnlif_fire_bp(spatial.data_ptr(), grad_spike.data_ptr(), grad_spatial.data_ptr(),
-                               _torch_dtype_code(spatial), T, N, alpha, thresh, beta, interval,
-                               ws_ptr, ws_bytes, _stream_handle(spatial))
+                               _hinted(_torch_dtype_code(spatial), keep_spatial), T, N, alpha, thresh,
+                               beta, interval, ws_ptr, ws_bytes, _stream_handle(spatial))
     _check(rc, "snnlif_fire_bp")
     return grad_spatial
 

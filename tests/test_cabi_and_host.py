@@ -41,6 +41,9 @@ def test_constants_match_the_header():
     assert int(macros["SNNLIF_DTYPE_F32"]) == lif_cabi.DTYPE_F32
     assert int(macros["SNNLIF_DTYPE_F64"]) == lif_cabi.DTYPE_F64
     assert int(macros["SNNLIF_DTYPE_BF16"]) == lif_cabi.DTYPE_BF16
+    hexes = dict(re.findall(r"#define\s+(SNNLIF_\w+)\s+(0x[0-9a-fA-F]+)", text))
+    assert int(hexes["SNNLIF_KEEP_SPATIAL"], 16) == lif_cabi.KEEP_SPATIAL
+    assert int(hexes["SNNLIF_STREAM_SPATIAL"], 16) == lif_cabi.STREAM_SPATIAL
     assert int(macros["SNNLIF_ERR_ARG"]) == lif_cabi.ERR_ARG
     assert int(macros["SNNLIF_ERR_DTYPE"]) == lif_cabi.ERR_DTYPE
     assert int(macros["SNNLIF_ERR_WORKSPACE"]) == lif_cabi.ERR_WORKSPACE
@@ -80,6 +83,13 @@ def test_host_side_queries_need_no_gpu():
     assert lib.snnlif_fire_bp(None, None, None, f32, 4, 0, 0.25, 0.5, 1.0, 0.5, None, 0, None) == lif_cabi.OK
     assert lib.snnlif_fire_bp(None, None, None, f32, 4, 8, 0.25, 0.5, 1.0, 0.5, None, 0, None) == lif_cabi.ERR_ARG
     assert lib.snnlif_fire_us_fp(None, None, None, f32, 1 << 40, 1 << 40, 0.25, 0.5, None) == lif_cabi.ERR_ARG
+    # cache hints ride in the dtype argument: either one is fine, both or unknown bits are not
+    for hint in (lif_cabi.KEEP_SPATIAL, lif_cabi.STREAM_SPATIAL):
+        assert lib.snnlif_fire_s_fp(None, None, f32 | hint, 0, 8, 0.25, 0.5, None) == lif_cabi.OK
+        assert lif_cabi.fire_bp_workspace_bytes(f64 | hint, 2000, 10) == 2000 * 10 * 8
+    both = lif_cabi.KEEP_SPATIAL | lif_cabi.STREAM_SPATIAL
+    assert lib.snnlif_fire_s_fp(None, None, f32 | both, 0, 8, 0.25, 0.5, None) == lif_cabi.ERR_DTYPE
+    assert lib.snnlif_fire_s_fp(None, None, f32 | 0x1000, 0, 8, 0.25, 0.5, None) == lif_cabi.ERR_DTYPE
 
 
 def test_snnlib_module_surface_and_cpu_rejection():

@@ -36,19 +36,21 @@ def make_inputs(shape, mean, std, seed, dtype=torch.float32):
     return x, g
 
 
-def run_gpu(cabi, x, g, alpha=ALPHA, thresh=THRESH, beta=BETA, interval=INTERVAL):
+def run_gpu(cabi, x, g, alpha=ALPHA, thresh=THRESH, beta=BETA, interval=INTERVAL, keep=None):
+    """`keep`: the cache hint (True: SNNLIF_KEEP_SPATIAL, False: SNNLIF_STREAM_SPATIAL, None: by size);
+    it selects between two instantiations of every kernel, which must give the same bits."""
     xd, gd = x.cuda(), g.cuda()
     mem = torch.empty_like(xd)
     spike_a = torch.empty_like(xd)
     spike_b = torch.empty_like(xd)
     gx = torch.empty_like(xd)
-    cabi.fire_s_fp_into(xd, spike_a, alpha, thresh)
-    cabi.fire_us_fp_into(xd, mem, spike_b, alpha, thresh)
+    cabi.fire_s_fp_into(xd, spike_a, alpha, thresh, keep_spatial=keep)
+    cabi.fire_us_fp_into(xd, mem, spike_b, alpha, thresh, keep_spatial=keep)
     code = {torch.float32: 0, torch.float64: 1, torch.bfloat16: 2}[x.dtype]
     T = x.shape[0]
     ws_bytes = cabi.fire_bp_workspace_bytes(code, T, x.numel() // T)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda") if ws_bytes else None
-    cabi.fire_bp_into(xd, gd, gx, alpha, thresh, beta, interval, workspace=ws)
+    cabi.fire_bp_into(xd, gd, gx, alpha, thresh, beta, interval, workspace=ws, keep_spatial=keep)
     torch.cuda.synchronize()
     return mem.cpu(), spike_a.cpu(), spike_b.cpu(), gx.cpu()
 
@@ -89,19 +91,28 @@ CASES = [
 ]
 
 
+# the cache hint: kept (what tensors this small get by themselves), streamed
+HINTS = pytest.mark.parametrize("keep", [True, False], ids=["kept", "streamed"])
+
+
+@HINTS
 @pytest.mark.parametrize("shape,mean,std", CASES)
-def test_fp32_parity(cabi, oracle, shape, mean, std):
+def test_fp32_parity(cabi, oracle, shape, mean, std, keep):
     x, g = make_inputs(shape, mean, std, seed=1234)
-    assert_parity(oracle, x, g, run_gpu(cabi, x, g))
+    assert_parity(oracle, x, g, run_gpu(cabi, x, g, keep=keep))
+    if keep:   # no hint at all: by size, i.e. kept for these shapes
+        assert_parity(oracle, x, g, run_gpu(cabi, x, g))
 
 
+@HINTS
 @pytest.mark.parametrize("T", list(range(1, 35)))
-def test_fp32_every_window_length(cabi, oracle, T):
+def test_fp32_every_window_length(cabi, oracle, T, keep):
     """Each window length up to 32 maps to its own or the next larger register window; 33 and 34
-    are cut into two segments.  Even and odd N."""
+    are cut into two segments.  Even and odd N.  The streamed forward requests windows of 9 to 16
+    steps whole and longer ones in groups of 16."""
     for n_inner in (256, 77):
         x, g = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=1000 + T)
-        assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
+        assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3, keep=keep), alpha=0.3)
 
 
 @pytest.mark.parametrize("T", [40, 48, 56, 64, 41, 47, 63, 65])
@@ -137,10 +148,12 @@ def test_fp32_parity_hyperparameters(cabi, oracle, alpha, thresh, beta, interval
                   alpha, thresh, beta, interval)
 
 
-@pytest.mark.parametrize("shape", [(8, 4, 16, 8, 8), (6, 3, 7), (33, 2, 10), (100, 2, 33), (1024, 1, 40), (1100, 1, 16)])
-def test_fp64_parity(cabi, oracle, shape):
+@HINTS
+@pytest.mark.parametrize("shape", [(8, 4, 16, 8, 8), (6, 3, 7), (13, 2, 50), (16, 3, 33), (20, 2, 64), (33, 2, 10),
+                                   (100, 2, 33), (1024, 1, 40), (1100, 1, 16)])
+def test_fp64_parity(cabi, oracle, shape, keep):
     x, g = make_inputs(shape, 0.5, 1.0, seed=99, dtype=torch.float64)
-    assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
+    assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3, keep=keep), alpha=0.3)
 
 
 def test_empty_shapes_are_noops(cabi):
@@ -158,6 +171,11 @@ def test_argument_errors(cabi):
     x = torch.zeros(4, 8, device="cuda")
     assert lib.snnlif_fire_s_fp(x.data_ptr(), None, 0, 4, 8, ALPHA, THRESH, None) == cabi.ERR_ARG
     assert lib.snnlif_fire_s_fp(x.data_ptr(), x.data_ptr(), 9, 4, 8, ALPHA, THRESH, None) == cabi.ERR_DTYPE
+    both = cabi.KEEP_SPATIAL | cabi.STREAM_SPATIAL       # contradictory hints, unknown flag bits
+    assert lib.snnlif_fire_s_fp(x.data_ptr(), x.data_ptr(), both, 4, 8, ALPHA, THRESH, None) == cabi.ERR_DTYPE
+    assert lib.snnlif_fire_s_fp(x.data_ptr(), x.data_ptr(), 0x400, 4, 8, ALPHA, THRESH, None) == cabi.ERR_DTYPE
+    assert lib.snnlif_fire_bp(x.data_ptr(), x.data_ptr(), x.data_ptr(), both, 4, 8, ALPHA, THRESH, BETA, INTERVAL,
+                              None, 0, None) == cabi.ERR_DTYPE
     assert lib.snnlif_fire_s_fp(x.data_ptr(), x.data_ptr(), 0, -1, 8, ALPHA, THRESH, None) == cabi.ERR_ARG
     assert lib.snnlif_fire_s_fp(x.data_ptr() + 2, x.data_ptr(), 0, 2, 4, ALPHA, THRESH, None) == cabi.ERR_ALIGN
     big = torch.zeros(1100, 8, device="cuda")
@@ -213,15 +231,16 @@ def test_special_values_follow_ieee_like_the_oracle(cabi, oracle):
     assert (np.abs(mem_o[:, 0, 300:364]) < 1.2e-38).all() and (mem_o[:, 0, 300:364] != 0).any()
 
 
+@HINTS
 @pytest.mark.parametrize("shape", [(8, 3, 255), (5, 1, 1), (16, 2, 4097), (33, 3, 77), (12, 4, 64, 4, 4),
                                    (48, 2, 130), (64, 2, 77), (64, 3, 256), (1024, 1, 128), (1040, 1, 30)])
-def test_bf16_storage_parity_including_odd_sizes(cabi, oracle, shape):
+def test_bf16_storage_parity_including_odd_sizes(cabi, oracle, shape, keep):
     """bf16 storage, fp32 arithmetic: two values per lane when N is even and the bases are 4-byte
     aligned, one otherwise.  Expected = the fp32 oracle on the bf16-rounded inputs, outputs rounded
     once to bf16 (spikes are exact either way)."""
     x32, g32 = make_inputs(shape, 0.5, 1.0, seed=2468)
     x, g = x32.bfloat16(), g32.bfloat16()
-    mem, spike_a, spike_b, gx = run_gpu(cabi, x, g)
+    mem, spike_a, spike_b, gx = run_gpu(cabi, x, g, keep=keep)
     mem_o, spike_o = oracle.fire_forward(x.float().numpy(), ALPHA, THRESH)
     gx_o = oracle.fire_backward(x.float().numpy(), g.float().numpy(), ALPHA, THRESH, BETA, INTERVAL)
     assert np.array_equal(spike_a.float().numpy(), spike_o)

@@ -1,4 +1,4 @@
-"""Seeded random sweep of shapes, window lengths, storage types, hyper-parameters and base-pointer
+"""Seeded random sweep of shapes, window lengths, storage types, hyper-parameters, cache hints and base-pointer
 offsets through the C ABI against the CPU oracle: the cases nobody thought of listing by hand.
 
 fp32 / fp64: spikes, membrane potentials and gradients bit-identical.  bf16 storage: spikes exact,
@@ -36,13 +36,14 @@ def draw_case(rng):
     beta = float(rng.choice([0.7, 1.0, 2.0]))
     interval = float(rng.choice([0.3, 0.5, 1.5]))
     offset = int(rng.integers(0, 4))       # elements by which the base pointers are shifted
-    return T, B, n, dtype, alpha, thresh, beta, interval, offset
+    keep = [None, True, False][int(rng.integers(0, 3))]   # cache hint: by size / kept / streamed
+    return T, B, n, dtype, alpha, thresh, beta, interval, offset, keep
 
 
-@pytest.mark.parametrize("seed", range(160))
+@pytest.mark.parametrize("seed", range(240))
 def test_random_fire_case(cabi, oracle, seed):
     rng = np.random.default_rng(9000 + seed)
-    T, B, n, dtype, alpha, thresh, beta, interval, offset = draw_case(rng)
+    T, B, n, dtype, alpha, thresh, beta, interval, offset, keep = draw_case(rng)
     shape = (T, B, n)
     gen = torch.Generator().manual_seed(seed)
     x = (0.4 + 0.9 * torch.randn(shape, generator=gen)).to(dtype)
@@ -58,13 +59,13 @@ def test_random_fire_case(cabi, oracle, seed):
 
     xd, gd = shifted(x), shifted(g)
     mem, spike, gx = shifted(), shifted(), shifted()
-    cabi.fire_us_fp_into(xd, mem, spike, alpha, thresh)
-    cabi.fire_bp_into(xd, gd, gx, alpha, thresh, beta, interval)
+    cabi.fire_us_fp_into(xd, mem, spike, alpha, thresh, keep_spatial=keep)
+    cabi.fire_bp_into(xd, gd, gx, alpha, thresh, beta, interval, keep_spatial=keep)
     spike_only = shifted()
-    cabi.fire_s_fp_into(xd, spike_only, alpha, thresh)
+    cabi.fire_s_fp_into(xd, spike_only, alpha, thresh, keep_spatial=keep)
     torch.cuda.synchronize()
 
-    what = f"T={T} B={B} n={n} {dtype} a={alpha} th={thresh} b={beta} iv={interval} off={offset}"
+    what = f"T={T} B={B} n={n} {dtype} a={alpha} th={thresh} b={beta} iv={interval} off={offset} keep={keep}"
     if dtype == torch.bfloat16:
         xo, go = x.float().numpy(), g.float().numpy()
         mem_o, spike_o = oracle.fire_forward(xo, alpha, thresh)
