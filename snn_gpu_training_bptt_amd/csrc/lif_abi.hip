@@ -234,6 +234,40 @@ int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const vo
                                MD(spike), /*from_ivar=*/true, T, B, C, HW, 0.f, alpha, thresh, st));
 }
 
+size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW) {
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0 || bn_shape_error(T, B, C, HW) != SNNLIF_OK) return 0;
+    if (T == 0 || B * C * HW == 0) return 0;
+    return snnlif::bn_stats_workspace_elems(T, B, C, HW) * es;
+}
+
+int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64_t T, int64_t B,
+                    int64_t C, int64_t HW, int raw_moments, void* workspace, size_t workspace_bytes,
+                    void* stream) {
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    if (C == 0) return SNNLIF_OK;
+    // a channel without elements has no statistics: refuse rather than divide by zero
+    if (T == 0 || B == 0 || HW == 0) return SNNLIF_ERR_ARG;
+    if (!spatial || !mean || !var) return SNNLIF_ERR_ARG;
+    const void* ptrs[3] = {spatial, mean, var};
+    if (!all_aligned(ptrs, 3, es)) return SNNLIF_ERR_ALIGN;
+    const size_t need = snnlif::bn_stats_workspace_elems(T, B, C, HW) * es;
+    if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
+    if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_stats_f32(CF(spatial), MF(mean), MF(var), raw_moments != 0, T, B, C, HW,
+                             MF(workspace), st),
+        snnlif::bn_stats_f64(CD(spatial), MD(mean), MD(var), raw_moments != 0, T, B, C, HW,
+                             MD(workspace), st));
+}
+
 size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW) {
     int rc = SNNLIF_OK;
     const size_t es = bn_element_size(dtype, &rc);

@@ -40,7 +40,29 @@ inline size_t bn_backward_workspace_elems(int64_t B, int64_t C, int64_t HW) {
     return 2 * bn_partial_count(B, C, HW) + split + static_cast<size_t>(2 * C);
 }
 
+// Batch statistics (lif_bn_stats.h): threads per workgroup of the partial-sum kernels, the number of
+// slices the rows of a small-plane tensor are dealt to (enough workgroups to fill the chip), partial
+// sums per quantity (one per wavefront, or one per (slice, column)), and the workspace in elements.
+constexpr int kStatsBlock = 256;
+inline int bn_stats_row_slices(int64_t rows, int64_t CHW) {
+    const int64_t groups = (CHW + kStatsBlock - 1) / kStatsBlock;
+    int64_t s = (2048 + groups - 1) / groups;
+    if (s > rows) s = rows;
+    if (s > 1024) s = 1024;
+    if (s < 1) s = 1;
+    return static_cast<int>(s);
+}
+inline size_t bn_stats_partial_count(int64_t T, int64_t B, int64_t C, int64_t HW) {
+    if (bn_wave_partials(HW)) return bn_partial_count(B, C, HW);
+    return static_cast<size_t>(bn_stats_row_slices(T * B, C * HW)) * static_cast<size_t>(C * HW);
+}
+inline size_t bn_stats_workspace_elems(int64_t T, int64_t B, int64_t C, int64_t HW) {
+    return 2 * bn_stats_partial_count(T, B, C, HW);
+}
+
 // Per scalar type F (suffix f32 = float, f64 = double):
+//   bn_stats_*           per-channel mean and biased variance (moments = false) or E[x] and E[x^2]
+//                        (moments = true) over (T, B, HW);
 //   bn_forward_*         from_ivar = false: stat is the variance and ivar is written; true: stat is
 //                        the inverse standard deviation and ivar is not touched.
 //   bn_backward_stats_*  sweep 1 + channel reduction: parameter gradients and the two per-channel
@@ -52,6 +74,8 @@ inline size_t bn_backward_workspace_elems(int64_t B, int64_t C, int64_t HW) {
                             const F* mean, F* ivar, F* spike, bool from_ivar, int64_t T,           \
                             int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,\
                             hipStream_t stream);                                                   \
+    int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,      \
+                          int64_t C, int64_t HW, F* workspace, hipStream_t stream);                \
     int bn_backward_stats_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,      \
                                    const F* mean, const F* g, F* grad_weight, F* grad_bias,        \
                                    F* mean_gxhat, F* mean_gxhatx, int64_t T, int64_t B, int64_t C, \

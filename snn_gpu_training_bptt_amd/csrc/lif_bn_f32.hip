@@ -1,4 +1,6 @@
 // Batch-norm + fire kernels for float storage and arithmetic; see lif_bn_launch.h.
 #include "lif_bn_launch.h"
+#include "lif_bn_stats.h"
 
 SNNLIF_DEFINE_BN_DTYPE(f32, float)
+SNNLIF_DEFINE_BN_STATS_DTYPE(f32, float)

@@ -1,4 +1,6 @@
 // Batch-norm + fire kernels for double storage and arithmetic; see lif_bn_launch.h.
 #include "lif_bn_launch.h"
+#include "lif_bn_stats.h"
 
 SNNLIF_DEFINE_BN_DTYPE(f64, double)
+SNNLIF_DEFINE_BN_STATS_DTYPE(f64, double)

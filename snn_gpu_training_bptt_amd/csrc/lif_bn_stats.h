@@ -1,0 +1,203 @@
+// Per-channel batch statistics of a [T, B, C, HW] activation for MI355X: mean and biased variance over
+// (T, B, HW), or the first two raw moments E[x], E[x^2] that a batch sharded over several GPUs
+// all-reduces (F = float or double).
+//
+// Reference: the layers compute these with framework reductions before calling the native op --
+// torch.var_mean(x, dim_bn, unbiased=False) in snnlib/example/snnlib_op.py:36-37, 76-78, 113-115, 175-177
+// and torch.mean(x), torch.mean(x**2) in the sharded layers, snnlib/example/snnlib_op.py:263-264,
+// 326-327, 386-387.  On MI355X the framework's Welford reduction over a [8,64,128,32,32] tensor runs at
+// 0.7 TB/s and costs five times the fused batch-norm + fire forward it feeds, so the statistics get a
+// kernel of their own.
+//
+// One pass over x (4 bytes per neuron-step in fp32), HBM-bound, two kernels:
+//   1. partial sums.  Planes of at least 32 positions: wavefronts are laid over the (batch entry,
+//      channel) planes exactly as in sweep 1 of the batch-norm backward (ceil(HW/64) wavefronts per
+//      plane, all lanes of a wavefront share a channel); a lane adds up its neuron's T values (eight
+//      at a time in the storage type, the groups in double), the wavefront folds the 64 lanes by
+//      shuffles and leaves one pair of sums.  Smaller planes (fully
+//      connected shapes): one lane per (channel, position) column of the [T*B, C*HW] matrix, the rows
+//      dealt round-robin to S slices of workgroups; consecutive lanes read consecutive addresses.
+//   2. one workgroup per channel adds the partial sums in double precision, in an order fixed by the
+//      launch geometry (results are reproducible), and writes the two statistics.
+// Sums are taken of d = x - K[c] with K[c] the channel's first element (t = 0, b = 0, position 0):
+// a shift by any sample of the channel keeps sum(d)^2/n and sum(d^2) of comparable size, so that
+// var = (sum(d^2) - sum(d)^2/n)/n does not cancel even when |mean| >> sqrt(var) (the textbook shifted
+// two-sum formula); mean = K + sum(d)/n.
+#ifndef SNNLIF_LIF_BN_STATS_H
+#define SNNLIF_LIF_BN_STATS_H
+
+#include "lif_bn.h"
+#include "lif_bn_kernels.h"
+
+namespace snnlif {
+
+constexpr int kStatsRows = 8;  // rows requested before the first is consumed
+
+// Planes of at least 32 positions.  part_* indexed [plane][chunk] like the backward's partial sums.
+template <typename F>
+__global__ void __launch_bounds__(kStatsBlock)
+bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restrict__ part_dd, int T,
+                     int64_t N, int64_t C, int64_t HW) {
+    const int64_t G = (HW + 63) / 64;
+    const int64_t lanes = (N / HW) * G * 64;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t pc = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; pc < lanes;
+         pc += stride) {
+        const int64_t wave = pc >> 6;
+        const int64_t plane = wave / G;
+        const int64_t k = (wave - plane * G) * 64 + (pc & 63);
+        const int c = static_cast<int>(plane % C);
+        double acc_d = 0.0, acc_dd = 0.0;
+        if (k < HW) {
+            const F shift = x[static_cast<int64_t>(c) * HW];
+            const F* col = x + plane * HW + k;
+            for (int t0 = 0; t0 < T; t0 += kStatsRows) {
+                F v[kStatsRows];
+#pragma unroll
+                for (int r = 0; r < kStatsRows; ++r) {
+                    v[r] = shift;  // rows past the end contribute d = 0
+                    if (t0 + r < T)
+                        v[r] = load_pack<F, 1, false>(col + static_cast<int64_t>(t0 + r) * N).e[0];
+                }
+                F group_d = F(0), group_dd = F(0);
+#pragma unroll
+                for (int r = 0; r < kStatsRows; ++r) {
+                    const F d = v[r] - shift;
+                    group_d += d;
+                    group_dd += d * d;
+                }
+                acc_d += static_cast<double>(group_d);
+                acc_dd += static_cast<double>(group_dd);
+            }
+        }
+        acc_d = wave_sum(acc_d);
+        acc_dd = wave_sum(acc_dd);
+        if ((pc & 63) == 0) {
+            part_d[wave] = static_cast<F>(acc_d);
+            part_dd[wave] = static_cast<F>(acc_dd);
+        }
+    }
+}
+
+// Planes of fewer than 32 positions: the tensor as a [rows = T*B, CHW] matrix.  Workgroup
+// (blockIdx.x, blockIdx.y = slice s) sums rows s, s+S, s+2S, ... of its 256 columns.
+// part_* indexed [slice][column].
+template <typename F>
+__global__ void __launch_bounds__(kStatsBlock)
+bn_stats_column_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restrict__ part_dd,
+                       int64_t rows, int64_t CHW, int64_t HW, int S) {
+    const int64_t j = static_cast<int64_t>(blockIdx.x) * kStatsBlock + threadIdx.x;
+    if (j >= CHW) return;
+    const int s = blockIdx.y;
+    const F shift = x[(j / HW) * HW];
+    double acc_d = 0.0, acc_dd = 0.0;
+    for (int64_t r0 = s; r0 < rows; r0 += static_cast<int64_t>(S) * kStatsRows) {
+        F v[kStatsRows];
+#pragma unroll
+        for (int q = 0; q < kStatsRows; ++q) {
+            const int64_t r = r0 + static_cast<int64_t>(q) * S;
+            v[q] = shift;
+            if (r < rows) v[q] = load_pack<F, 1, false>(x + r * CHW + j).e[0];
+        }
+        F group_d = F(0), group_dd = F(0);
+#pragma unroll
+        for (int q = 0; q < kStatsRows; ++q) {
+            const F d = v[q] - shift;
+            group_d += d;
+            group_dd += d * d;
+        }
+        acc_d += static_cast<double>(group_d);
+        acc_dd += static_cast<double>(group_dd);
+    }
+    part_d[static_cast<int64_t>(s) * CHW + j] = static_cast<F>(acc_d);
+    part_dd[static_cast<int64_t>(s) * CHW + j] = static_cast<F>(acc_dd);
+}
+
+// One workgroup per channel: adds the channel's partial sums in double and writes
+//   moments == false:  out_a = mean,  out_b = biased variance
+//   moments == true:   out_a = E[x],  out_b = E[x^2]
+// Wave layout: entries (b*C + c)*G + i for b < B, i < G.  Column layout: entries s*CHW + c*HW + i for
+// s < S, i < HW.  Both are "outer" groups of "inner" consecutive entries, outer_stride apart.
+template <typename F>
+__global__ void __launch_bounds__(kReduceBlock)
+bn_stats_finalize_kernel(const F* __restrict__ x, const F* __restrict__ part_d,
+                         const F* __restrict__ part_dd, F* __restrict__ out_a,
+                         F* __restrict__ out_b, int64_t HW, int64_t outer, int64_t inner,
+                         int64_t outer_stride, double count, bool moments) {
+    const int c = blockIdx.x;
+    const int64_t base = static_cast<int64_t>(c) * inner;
+    const int64_t n = outer * inner;
+    double a = 0.0, aa = 0.0;
+    for (int64_t e = threadIdx.x; e < n; e += kReduceBlock) {
+        const int64_t at = (e / inner) * outer_stride + base + (e % inner);
+        a += static_cast<double>(part_d[at]);
+        aa += static_cast<double>(part_dd[at]);
+    }
+    __shared__ double lds[2][kReduceBlock / 64];
+    a = wave_sum(a);
+    aa = wave_sum(aa);
+    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    if (lane == 0) {
+        lds[0][wave] = a;
+        lds[1][wave] = aa;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        double sd = 0.0, sdd = 0.0;
+#pragma unroll
+        for (int w = 0; w < kReduceBlock / 64; ++w) {
+            sd += lds[0][w];
+            sdd += lds[1][w];
+        }
+        const double shift = static_cast<double>(x[static_cast<int64_t>(c) * HW]);
+        const double mean_d = sd / count;
+        double var = (sdd - sd * mean_d) / count;
+        if (var < 0.0) var = 0.0;
+        const double mean = shift + mean_d;
+        out_a[c] = static_cast<F>(mean);
+        out_b[c] = static_cast<F>(moments ? var + mean * mean : var);
+    }
+}
+
+template <typename F>
+int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B, int64_t C,
+             int64_t HW, F* workspace, hipStream_t stream) {
+    const int64_t N = B * C * HW;
+    const size_t P = bn_stats_partial_count(T, B, C, HW);
+    F* part_d = workspace;
+    F* part_dd = workspace + P;
+    const double count = static_cast<double>(T) * static_cast<double>(B) * static_cast<double>(HW);
+    if (bn_wave_partials(HW)) {
+        const int64_t G = (HW + 63) / 64;
+        launch_kernel(bn_stats_wave_kernel<F>, dim3(grid_for(B * C * G * 64, kStatsBlock)),
+                      dim3(kStatsBlock), 0, stream, x, part_d, part_dd, static_cast<int>(T), N, C, HW);
+        int rc = launch_status();
+        if (rc != SNNLIF_OK) return rc;
+        launch_kernel(bn_stats_finalize_kernel<F>, dim3(static_cast<unsigned>(C)), dim3(kReduceBlock),
+                      0, stream, x, part_d, part_dd, out_a, out_b, HW, B, G, C * G, count, moments);
+        return launch_status();
+    }
+    const int64_t rows = T * B, CHW = C * HW;
+    const int S = bn_stats_row_slices(rows, CHW);
+    launch_kernel(bn_stats_column_kernel<F>,
+                  dim3(static_cast<unsigned>((CHW + kStatsBlock - 1) / kStatsBlock), S),
+                  dim3(kStatsBlock), 0, stream, x, part_d, part_dd, rows, CHW, HW, S);
+    int rc = launch_status();
+    if (rc != SNNLIF_OK) return rc;
+    launch_kernel(bn_stats_finalize_kernel<F>, dim3(static_cast<unsigned>(C)), dim3(kReduceBlock), 0,
+                  stream, x, part_d, part_dd, out_a, out_b, HW, static_cast<int64_t>(S), HW, CHW, count,
+                  moments);
+    return launch_status();
+}
+
+}  // namespace snnlif
+
+#define SNNLIF_DEFINE_BN_STATS_DTYPE(SUFFIX, F)                                                    \
+    namespace snnlif {                                                                             \
+    int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,      \
+                          int64_t C, int64_t HW, F* workspace, hipStream_t stream) {               \
+        return bn_stats<F>(x, out_a, out_b, moments, T, B, C, HW, workspace, stream);              \
+    }                                                                                              \
+    }
+
+#endif  // SNNLIF_LIF_BN_STATS_H

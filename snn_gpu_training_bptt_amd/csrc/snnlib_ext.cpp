@@ -16,7 +16,9 @@
 //   bn_fire_fc_fp / bn_fire_fc_bp, bn_fire_conv_fp / bn_fire_conv_bp                snn.cpp:85-101, 484-506, 162-188, 630-660
 //
 // plus fire_us_fp(spatial, alpha, thresh) -> (mem, spike), the public face of the reference's
-// internal fire_us_fp_kernel (snnlib/cuda/snn_kernel_bp.cu:54-93), and the halves that a batch sharded
+// internal fire_us_fp_kernel (snnlib/cuda/snn_kernel_bp.cu:54-93), bn_stats(spatial) -> [var, mean] and
+// bn_moments(spatial) -> [E[x], E[x^2]], the batch statistics the reference's layers take from
+// torch.var_mean / torch.mean (snnlib/example/snnlib_op.py:76-78, 263-264), and the halves that a batch sharded
 // over several GPUs runs on either side of its all-reduce (the all-reduce itself is the caller's):
 //
 //   bn_bp_dist1 / bn_bp_dist2                                                       snn.cpp:317-355
@@ -295,6 +297,39 @@ BnOperands bn_operands(const Tensor& spatial, const Tensor& weight_bn, const Ten
     o.mean = channel_param(mean, o.x, o.d.C, op, "mean");
     return o;
 }
+
+// Per-channel batch statistics over every axis but the channel's (axis 2), on the hand-written
+// reduction behind snnlif_bn_stats: what the layers of snnlib/example/snnlib_op.py obtain from
+// torch.var_mean(x, dim_bn, unbiased=False) (:76-78) or, for a sharded batch, from torch.mean(x) and
+// torch.mean(x**2) (:263-264) before they call a batch-norm op.  Not part of the reference's binding
+// table.  raw_moments = false -> {var (biased), mean}; true -> {E[x], E[x^2]}.
+std::vector<Tensor> batch_statistics(const Tensor& spatial, bool raw_moments, const char* op) {
+    check_input(spatial, op, "spatial");
+    TORCH_CHECK(spatial.scalar_type() == at::kFloat || spatial.scalar_type() == at::kDouble,
+                "snnlib.", op, ": only float32 and float64 are supported, got ",
+                spatial.scalar_type());
+    const int dtype = spatial.scalar_type() == at::kFloat ? SNNLIF_DTYPE_F32 : SNNLIF_DTYPE_F64;
+    const BnDims d = bn_dims_of(spatial, op);
+    TORCH_CHECK(d.C == 0 || (d.T > 0 && d.B > 0 && d.HW > 0), "snnlib.", op,
+                ": no elements per channel in a tensor shaped ", spatial.sizes());
+    const DeviceGuard guard(spatial.device());
+    Tensor x = spatial.contiguous();
+    Tensor first = torch::empty({d.C}, x.options());
+    Tensor second = torch::empty({d.C}, x.options());
+    const size_t ws_bytes = snnlif_bn_stats_workspace_bytes(dtype, d.T, d.B, d.C, d.HW);
+    Tensor workspace =
+        torch::empty({static_cast<int64_t>(ws_bytes)}, x.options().dtype(at::kByte));
+    check_rc(snnlif_bn_stats(x.data_ptr(), first.data_ptr(), second.data_ptr(), dtype, d.T, d.B, d.C,
+                             d.HW, raw_moments ? 1 : 0, ws_bytes ? workspace.data_ptr() : nullptr,
+                             ws_bytes, current_stream()),
+             op);
+    if (raw_moments) return {first, second};
+    return {second, first};  // the order of torch.var_mean
+}
+
+std::vector<Tensor> bn_stats(Tensor spatial) { return batch_statistics(spatial, false, "bn_stats"); }
+
+std::vector<Tensor> bn_moments(Tensor spatial) { return batch_statistics(spatial, true, "bn_moments"); }
 
 std::vector<Tensor> bn_fire_s_fp(Tensor spatial, Tensor weight_bn, Tensor bias_bn, Tensor var,
                                  Tensor mean, float eps_bn, float alpha, float thresh) {
@@ -718,6 +753,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("fire_s_fp", &fire_s_fp, "fire (spike) forward");
     m.def("fire_us_fp", &fire_us_fp, "fire (membrane potential, spike) forward");
     m.def("bn_fire_s_fp", &bn_fire_s_fp, "bn fire (spike) forward");
+
+    m.def("bn_stats", &bn_stats, "per-channel [biased variance, mean] of a [T, B, C, ...] tensor");
+    m.def("bn_moments", &bn_moments, "per-channel [E[x], E[x^2]] of a [T, B, C, ...] tensor");
 
     m.def("bn_fp", &bn_fp, "bn forward");
     m.def("bn_bp", &bn_bp, "bn backward");

@@ -30,6 +30,8 @@ SYMBOLS = {
     "snnlif_fire_us_fp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64]),
     "snnlif_fire_bp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
+    "snnlif_bn_stats_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
+    "snnlif_bn_stats": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "snnlif_bn_fire_s_fp": (_int, [_vp] * 7 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _vp]),
     "snnlif_bn_fire_s_recompute": (_int, [_vp] * 6 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_bn_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
@@ -214,6 +216,26 @@ def _bn_dims(t):
     T, B, C = t.shape[0], t.shape[1], t.shape[2]
     HW = t.numel() // (T * B * C) if T * B * C else 0
     return T, B, C, HW
+
+
+def bn_stats_workspace_bytes(dtype_code, T, B, C, HW):
+    return int(load().snnlif_bn_stats_workspace_bytes(dtype_code, T, B, C, HW))
+
+
+def bn_stats_into(spatial, mean, var, workspace, raw_moments=False):
+    """``snnlif_bn_stats``: per-channel mean and biased variance of ``spatial`` ([T, B, C, ...]) over all
+    axes but the channel's, or E[x] and E[x^2] with ``raw_moments``; writes ``mean`` and ``var`` ([C])."""
+    T, B, C, HW = _bn_dims(spatial)
+    _require_per_channel(spatial, C, mean=mean, var=var)
+    _require_workspace(spatial, workspace,
+                       bn_stats_workspace_bytes(_torch_dtype_code(spatial), T, B, C, HW),
+                       "snnlif_bn_stats")
+    _require_dense_gpu(spatial, mean, var, workspace)
+    rc = load().snnlif_bn_stats(spatial.data_ptr(), mean.data_ptr(), var.data_ptr(),
+                                _torch_dtype_code(spatial), T, B, C, HW, int(bool(raw_moments)),
+                                workspace.data_ptr(), workspace.numel(), _stream_handle(spatial))
+    _check(rc, "snnlif_bn_stats")
+    return mean, var
 
 
 def bn_fire_s_fp_into(spatial, weight, bias, var, mean, ivar, spike, eps, alpha, thresh):

@@ -10,8 +10,9 @@ process group (one rank per GPU): the batch statistics and, in the backward, two
 are all-reduced, so every rank normalises with the statistics of the whole batch.
 
 Batch-norm behaviour shared by the ``Bn*`` modules, as in the reference: ``train_bn`` (not
-``nn.Module.training``) selects batch statistics (``torch.var_mean(..., unbiased=False)`` over
-``dim_bn``) or the running ones; the running statistics are ``nn.Parameter`` objects that are
+``nn.Module.training``) selects batch statistics (biased variance and mean over ``dim_bn``, which the
+reference takes from ``torch.var_mean(..., unbiased=False)`` and this build from its own reduction
+kernel, ``snnlib.bn_stats``) or the running ones; the running statistics are ``nn.Parameter`` objects that are
 *replaced* on every training-mode call (momentum 0.1, variance corrected by n/(n-1), n = elements
 per channel of the first input seen).
 """
@@ -21,6 +22,17 @@ import torch
 import torch.nn as nn
 
 from . import snnlib_func as sf
+
+
+def _channel_major_input(x, dim_bn):
+    """``x`` detached, after checking that ``dim_bn`` names every axis but the channel's (axis 2):
+    the native batch-norm ops, like the reference's, take the channel from axis 2 and reduce over
+    all others, so no other ``dim_bn`` is meaningful for a ``[T, B, C, ...]`` input."""
+    wanted = tuple(d for d in range(x.dim()) if d != 2)
+    if tuple(sorted(d % x.dim() for d in dim_bn)) != wanted:
+        raise ValueError(f"dim_bn={tuple(dim_bn)} must name every axis of a {x.dim()}-d input except "
+                         f"the channel axis 2, i.e. {wanted}")
+    return x.detach()
 
 
 class _BatchStatistics(nn.Module):
@@ -46,7 +58,7 @@ class _BatchStatistics(nn.Module):
             self.running_mean = self.running_mean.to(x.device)
         if not self.train_bn:
             return self.running_var, self.running_mean
-        var, mean = torch.var_mean(x, dim=self.dim_bn, unbiased=False)
+        var, mean = sf.snnlib.bn_stats(_channel_major_input(x, self.dim_bn))
         self.running_var = nn.Parameter(self.running_var * 0.9 + var * (0.1 * self.factor))
         self.running_mean = nn.Parameter(self.running_mean * 0.9 + mean * 0.1)
         return var, mean
@@ -71,8 +83,7 @@ class _ShardedBatchStatistics(_BatchStatistics):
             self.world_size = torch.distributed.get_world_size(self.process_group)
         if not self.train_bn:
             return self.running_var, self.running_mean
-        first = torch.mean(x, dim=self.dim_bn)
-        second = torch.mean(x ** 2, dim=self.dim_bn)
+        first, second = sf.snnlib.bn_moments(_channel_major_input(x, self.dim_bn))
         torch.distributed.all_reduce(first, self.ReduceOp.SUM, self.process_group)
         torch.distributed.all_reduce(second, self.ReduceOp.SUM, self.process_group)
         mean = first / self.world_size

@@ -2,6 +2,7 @@ import os
 import sys
 
 import pytest
+import torch
 
 REPO = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if REPO not in sys.path:
@@ -33,3 +34,26 @@ def pytest_collection_modifyitems(config, items):
 @pytest.fixture(scope="session")
 def hyper():
     return dict(alpha=ALPHA, thresh=THRESH, beta=BETA, interval=INTERVAL)
+
+
+def decision_margin(u, thresh=THRESH, interval=INTERVAL):
+    """Smallest distance of any membrane potential in ``u`` to a point where the fire op's output or
+    its gradient jumps: the threshold (spike / no spike, reset / no reset) and the two edges of the
+    surrogate window."""
+    d = (u - thresh).abs()
+    return float(torch.minimum(d, (d - interval).abs()).min())
+
+
+def seed_clear_of_decision_points(potentials_for_seed, seeds, margin=1e-6, thresh=THRESH, interval=INTERVAL):
+    """First seed whose membrane potentials (as computed by the comparator) all stay at least ``margin``
+    away from every decision point.  Two correct implementations of a batch-norm + fire layer differ
+    in the last bits of the batch statistics (different summation orders); a potential closer than that
+    to a decision point would legitimately come out on either side and turn a rounding difference
+    into a whole spike or gradient term.  Drawing inputs clear of those points lets a layer test
+    compare spikes exactly and gradients tightly, without conditions on the outcome.  The default
+    margin is a few times the difference two fp32 evaluations of the batch statistics leave in a
+    potential of order one."""
+    for seed in seeds:
+        if decision_margin(potentials_for_seed(seed), thresh, interval) > margin:
+            return seed
+    raise AssertionError("no candidate seed keeps the membrane potentials clear of the decision points")

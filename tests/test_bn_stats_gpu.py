@@ -1,0 +1,187 @@
+"""Per-channel batch statistics (``snnlif_bn_stats``) on the GPU, through the C ABI.
+
+What it replaces is a library routine -- ``torch.var_mean(x, dim_bn, unbiased=False)`` in the
+reference's layers (snnlib/example/snnlib_op.py:76-78) and ``torch.mean(x)``, ``torch.mean(x**2)`` in the
+sharded ones (:263-264) -- so that routine, evaluated in float64 on the same values, is the checker:
+fp32 results within 1e-6 of it (relative to the statistic's scale), fp64 within 1e-13.
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+SHAPES = [
+    (6, 2, 8),                # the reference test's fc shape: one position per channel
+    (6, 2, 8, 8, 8),          # the reference test's conv shape
+    (8, 16, 32, 16, 16),      # HW = 256: four wavefronts per plane
+    (4, 5, 7, 7, 7),          # HW = 49: one partly idle wavefront per plane
+    (6, 3, 6, 14, 14),        # HW = 196
+    (5, 2, 3, 4, 8),          # HW = 32: the smallest plane-aligned case
+    (5, 2, 9, 31),            # HW = 31: column layout
+    (13, 3, 20, 5, 3),        # 13 steps: two groups of rows, the second partial
+    (32, 2, 16, 4, 4),
+    (33, 2, 6, 8, 8),
+    (100, 3, 20),
+    (1024, 1, 4, 6, 6),
+    (1, 1, 5, 1),             # a single value per channel: variance 0
+    (8, 64, 1024),            # fully connected, many channels
+    (8, 256, 16),             # fully connected, few channels: many row slices
+    (3, 7, 300, 3, 3),        # HW = 9, more columns than one workgroup holds
+    (8, 32, 128, 32, 32),     # few channels, many positions
+]
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from snn_gpu_training_bptt_amd import lif_cabi
+    lif_cabi.load()
+    return lif_cabi
+
+
+def dims_of(shape):
+    T, B, C = shape[:3]
+    HW = int(np.prod(shape[3:])) if len(shape) > 3 else 1
+    return T, B, C, HW
+
+
+def run_stats(cabi, x, raw_moments=False):
+    T, B, C, HW = dims_of(tuple(x.shape))
+    code = cabi.DTYPE_F32 if x.dtype == torch.float32 else cabi.DTYPE_F64
+    ws = torch.empty(cabi.bn_stats_workspace_bytes(code, T, B, C, HW), dtype=torch.uint8, device="cuda")
+    mean = torch.full((C,), float("nan"), dtype=x.dtype, device="cuda")
+    second = torch.full((C,), float("nan"), dtype=x.dtype, device="cuda")
+    cabi.bn_stats_into(x, mean, second, ws, raw_moments=raw_moments)
+    torch.cuda.synchronize()
+    return mean.cpu(), second.cpu()
+
+
+def make(shape, seed, dtype=torch.float32, offset=0.5):
+    gen = torch.Generator().manual_seed(seed)
+    C = shape[2]
+    per_channel = (C,) + (1,) * (len(shape) - 3)
+    x = offset + torch.randn(per_channel, generator=gen) + torch.randn(shape, generator=gen) * (
+        0.5 + torch.rand(per_channel, generator=gen))
+    return x.to(dtype)
+
+
+def reference(x):
+    dims = tuple(d for d in range(x.dim()) if d != 2)
+    var, mean = torch.var_mean(x.double(), dim=dims, unbiased=False)
+    return mean, var, torch.mean(x.double() ** 2, dim=dims)
+
+
+def assert_close(got, want, scale, tol, what):
+    err = (got.double() - want).abs()
+    assert bool((err <= tol * scale + 1e-300).all()), \
+        f"{what}: max error {err.max().item():.3e} against scale {scale.max().item():.3e} (tolerance {tol})"
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_fp32_statistics_against_float64_var_mean(cabi, shape):
+    x = make(shape, seed=51)
+    mean_ref, var_ref, second_ref = reference(x)
+    spread = var_ref.sqrt() + mean_ref.abs() + 1e-30
+    mean, var = run_stats(cabi, x.cuda())
+    assert_close(mean, mean_ref, spread, 1e-6, "mean")
+    assert_close(var, var_ref, var_ref + 1e-30, 1e-6, "biased variance")
+    first, second = run_stats(cabi, x.cuda(), raw_moments=True)
+    assert torch.equal(first, mean)
+    assert_close(second, second_ref, second_ref + 1e-30, 1e-6, "second raw moment")
+    # fixed summation order: the same bits on every call
+    again = run_stats(cabi, x.cuda())
+    assert torch.equal(again[0], mean) and torch.equal(again[1], var)
+
+
+@pytest.mark.parametrize("shape", [(6, 2, 8), (6, 2, 8, 8, 8), (8, 16, 32, 16, 16), (4, 5, 7, 7, 7), (5, 2, 9, 31),
+                                   (13, 3, 20, 5, 3), (8, 64, 256)])
+def test_fp64_statistics(cabi, shape):
+    x = make(shape, seed=52, dtype=torch.float64)
+    mean_ref, var_ref, second_ref = reference(x)
+    mean, var = run_stats(cabi, x.cuda())
+    assert_close(mean, mean_ref, var_ref.sqrt() + mean_ref.abs() + 1e-300, 1e-13, "mean")
+    assert_close(var, var_ref, var_ref + 1e-300, 1e-13, "biased variance")
+    _, second = run_stats(cabi, x.cuda(), raw_moments=True)
+    assert_close(second, second_ref, second_ref + 1e-300, 1e-13, "second raw moment")
+
+
+@pytest.mark.parametrize("shape", [(8, 16, 8, 16, 16), (8, 64, 32)])
+def test_variance_survives_a_mean_far_from_zero(cabi, shape):
+    """|mean| = 1000 standard deviations: E[x^2] - E[x]^2 in float32 would keep no correct digit; the
+    shifted sums still resolve the variance of the float32 values to 1e-6."""
+    x = make(shape, seed=53, offset=1000.0)
+    mean_ref, var_ref, _ = reference(x)
+    assert float((mean_ref.abs() / var_ref.sqrt()).min()) > 300
+    mean, var = run_stats(cabi, x.cuda())
+    assert_close(mean, mean_ref, mean_ref.abs(), 1e-7, "mean")
+    assert_close(var, var_ref, var_ref, 1e-6, "biased variance")
+
+
+def test_constant_channels_have_zero_variance(cabi):
+    x = torch.full((4, 3, 5, 6, 6), 0.75)
+    x[:, :, 2] = -3.0
+    mean, var = run_stats(cabi, x.cuda())
+    assert torch.equal(var, torch.zeros(5))
+    assert torch.equal(mean, torch.tensor([0.75, 0.75, -3.0, 0.75, 0.75]))
+
+
+def test_full_size_headline_shape(cabi):
+    """[8, 64, 128, 32, 32]: 524 288 values per channel, generated on the device."""
+    gen = torch.Generator(device="cuda").manual_seed(54)
+    x = 0.5 + torch.randn((8, 64, 128, 32, 32), generator=gen, device="cuda")
+    var_ref, mean_ref = torch.var_mean(x.double(), dim=(0, 1, 3, 4), unbiased=False)
+    mean, var = run_stats(cabi, x)
+    assert_close(mean, mean_ref.cpu(), (var_ref.sqrt() + mean_ref.abs()).cpu(), 1e-6, "mean")
+    assert_close(var, var_ref.cpu(), var_ref.cpu(), 1e-6, "biased variance")
+
+
+def test_argument_errors(cabi):
+    lib = cabi.load()
+    x = torch.zeros(4, 2, 8, device="cuda")
+    p = torch.zeros(8, device="cuda")
+    ws = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    f32 = cabi.DTYPE_F32
+    call = lambda dtype, T, B, C, HW, w, n: lib.snnlif_bn_stats(x.data_ptr(), p.data_ptr(), p.data_ptr(), dtype,
+                                                                 T, B, C, HW, 0, w, n, None)
+    assert call(cabi.DTYPE_BF16, 4, 2, 8, 1, ws.data_ptr(), ws.numel()) == cabi.ERR_UNSUPPORTED
+    assert call(9, 4, 2, 8, 1, ws.data_ptr(), ws.numel()) == cabi.ERR_DTYPE
+    assert call(f32, 0, 2, 8, 1, ws.data_ptr(), ws.numel()) == cabi.ERR_ARG       # no elements per channel
+    assert call(f32, 4, 2, 0, 1, ws.data_ptr(), ws.numel()) == cabi.OK            # no channels: nothing to do
+    assert call(f32, 4, 2, 8, 1, None, 0) == cabi.ERR_WORKSPACE
+    assert call(f32, 4, 2, 8, 1, ws.data_ptr(), 8) == cabi.ERR_WORKSPACE
+    assert call(f32, 4, 2, 8, 1, ws.data_ptr() + 4, ws.numel() - 4) == cabi.ERR_ALIGN
+    assert lib.snnlif_bn_stats(None, p.data_ptr(), p.data_ptr(), f32, 4, 2, 8, 1, 0, ws.data_ptr(), ws.numel(),
+                               None) == cabi.ERR_ARG
+    torch.cuda.synchronize()
+
+
+def test_module_ops_and_layer_statistics():
+    """``snnlib.bn_stats`` / ``snnlib.bn_moments`` and the running statistics of a layer that uses them."""
+    import snn_gpu_training_bptt_amd.snnlib_func  # noqa: F401  (registers the module)
+    import snnlib
+    from snn_gpu_training_bptt_amd import snnlib_op as sop
+    x = make((6, 4, 8, 8, 8), seed=55).cuda()
+    mean_ref, var_ref, second_ref = reference(x.cpu())
+    var, mean = snnlib.bn_stats(x)                       # the order of torch.var_mean
+    first, second = snnlib.bn_moments(x)
+    torch.testing.assert_close(mean.cpu().double(), mean_ref, rtol=1e-6, atol=1e-7)
+    torch.testing.assert_close(var.cpu().double(), var_ref, rtol=1e-6, atol=0)
+    torch.testing.assert_close(second.cpu().double(), second_ref, rtol=1e-6, atol=0)
+    assert torch.equal(first, mean)
+    strided = x.transpose(3, 4)                          # made dense inside the op
+    v2, m2 = snnlib.bn_stats(strided)
+    torch.testing.assert_close(m2, mean, rtol=1e-6, atol=1e-7)
+    with pytest.raises(RuntimeError, match="float32 and float64"):
+        snnlib.bn_stats(x.bfloat16())
+    with pytest.raises(RuntimeError, match="ROCm GPU"):
+        snnlib.bn_stats(x.cpu())
+    with pytest.raises(RuntimeError, match="no elements per channel"):
+        snnlib.bn_stats(torch.zeros(0, 2, 3, device="cuda"))
+    layer = sop.Bn(8, (0, 1, 3, 4)).cuda()
+    layer(x.requires_grad_(True))
+    n = x.numel() / 8
+    torch.testing.assert_close(layer.running_mean.detach().cpu().double(), 0.1 * mean_ref, rtol=1e-5, atol=1e-7)
+    torch.testing.assert_close(layer.running_var.detach().cpu().double(), 0.9 + 0.1 * var_ref * n / (n - 1),
+                               rtol=1e-5, atol=0)
+    with pytest.raises(ValueError, match="dim_bn"):
+        sop.Bn(8, (0, 1)).cuda()(x)

@@ -97,7 +97,7 @@ def test_snnlib_module_surface_and_cpu_rejection():
     import snnlib  # registered under the reference's top-level name by the package
     assert snnlib is sf.snnlib
     assert snnlib.__backend__ == "hip-gfx950"
-    for name in ("fire_s_fp", "fire_bp", "fire_us_fp"):
+    for name in ("fire_s_fp", "fire_bp", "fire_us_fp", "bn_stats", "bn_moments"):
         assert callable(getattr(snnlib, name))
     # positional signatures of the reference binding (snnlib/cuda/snn.cpp:11-17, 270-279)
     with pytest.raises(TypeError):
@@ -109,6 +109,8 @@ def test_snnlib_module_surface_and_cpu_rejection():
         snnlib.fire_s_fp(torch.zeros(2, 3), 0.25, 0.5)
     with pytest.raises(RuntimeError, match="ROCm GPU"):
         snnlib.fire_bp(torch.zeros(2, 3), torch.zeros(2, 3), 0.25, 0.5, 1.0, 0.5)
+    with pytest.raises(RuntimeError, match="ROCm GPU"):
+        snnlib.bn_stats(torch.zeros(2, 3, 4))
 
 
 def test_python_interface_mirrors_the_reference():

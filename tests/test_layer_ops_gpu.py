@@ -11,7 +11,7 @@ The spikes feeding them are compared exactly where the test can see them.
 import pytest
 import torch
 
-from conftest import ALPHA, BETA, INTERVAL, THRESH
+from conftest import ALPHA, BETA, INTERVAL, THRESH, seed_clear_of_decision_points
 
 pytestmark = pytest.mark.gpu
 EPS = 1e-5
@@ -128,12 +128,22 @@ def test_conv(mods, shape, cout, stride, padding, bias):
 @pytest.mark.parametrize("train_bn", [True, False])
 def test_bn_fire_fc(mods, shape, dim_bn, cin_bn, cout, train_bn):
     _, sop, gold = mods
-    torch.manual_seed(55)
-    x_cpu = 0.3 + torch.randn(shape)
-    cin = x_cpu[0, 0].numel()
-    layer = sop.BnFireFc(cin, cout, dim_bn, EPS, cin_bn=cin_bn).cuda()
-    randomise_bn(layer, 56)
-    layer.train_bn = train_bn
+
+    def build(seed):
+        torch.manual_seed(seed)
+        x_cpu = 0.3 + torch.randn(shape)
+        layer = sop.BnFireFc(x_cpu[0, 0].numel(), cout, dim_bn, EPS, cin_bn=cin_bn).cuda()
+        randomise_bn(layer, seed + 1)
+        layer.train_bn = train_bn
+        return x_cpu, layer
+
+    def potentials(seed):
+        x_cpu, layer = build(seed)
+        with torch.no_grad():
+            return gold.gold_bn_fire(x_cpu.cuda(), layer.weight_bn, layer.bias_bn, layer.running_mean.clone(),
+                                     layer.running_var.clone(), train_bn, EPS, ALPHA, THRESH, BETA, INTERVAL)[0]
+
+    x_cpu, layer = build(seed_clear_of_decision_points(potentials, range(55, 4055, 100)))
     rm, rv = layer.running_mean.detach().clone(), layer.running_var.detach().clone()
     x = x_cpu.cuda().requires_grad_(True)
     y = layer(x)
@@ -155,11 +165,22 @@ def test_bn_fire_fc(mods, shape, dim_bn, cin_bn, cout, train_bn):
 @pytest.mark.parametrize("train_bn,bias", [(True, True), (False, True), (True, False)])
 def test_bn_fire_conv(mods, shape, cout, stride, train_bn, bias):
     _, sop, gold = mods
-    torch.manual_seed(57)
-    x_cpu = 0.3 + torch.randn(shape)
-    layer = sop.BnFireConv(shape[2], cout, (3, 3), stride, (1, 1), EPS, if_bias_conv=bias).cuda()
-    randomise_bn(layer, 58)
-    layer.train_bn = train_bn
+
+    def build(seed):
+        torch.manual_seed(seed)
+        x_cpu = 0.3 + torch.randn(shape)
+        layer = sop.BnFireConv(shape[2], cout, (3, 3), stride, (1, 1), EPS, if_bias_conv=bias).cuda()
+        randomise_bn(layer, seed + 1)
+        layer.train_bn = train_bn
+        return x_cpu, layer
+
+    def potentials(seed):
+        x_cpu, layer = build(seed)
+        with torch.no_grad():
+            return gold.gold_bn_fire(x_cpu.cuda(), layer.weight_bn, layer.bias_bn, layer.running_mean.clone(),
+                                     layer.running_var.clone(), train_bn, EPS, ALPHA, THRESH, BETA, INTERVAL)[0]
+
+    x_cpu, layer = build(seed_clear_of_decision_points(potentials, range(57, 4057, 100)))
     rm, rv = layer.running_mean.detach().clone(), layer.running_var.detach().clone()
     x = x_cpu.cuda().requires_grad_(True)
     y = layer(x)

@@ -255,10 +255,14 @@ def test_dist_modules_with_one_rank(hyper, monkeypatch, kind):
     out.backward(gout)
     assert rank.calls == 4            # two vectors forward (statistics), two backward (means)
 
-    # the same layer through the single-GPU function with the statistics formed the sharded way
+    # the same layer through the single-GPU function with the statistics formed the sharded way:
+    # E[x] and E[x^2] from the op the layer itself uses, var = E[x^2] - E[x]^2
+    import snnlib
     dim_bn = (0, 1, 3, 4)
-    mean = x.detach().mean(dim=dim_bn)
-    var = (x.detach() ** 2).mean(dim=dim_bn) - mean ** 2
+    mean, second = snnlib.bn_moments(x.detach())
+    var = second - mean ** 2
+    torch.testing.assert_close(mean, x.detach().mean(dim=dim_bn), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(second, (x.detach() ** 2).mean(dim=dim_bn), rtol=1e-5, atol=1e-6)
     x2 = x.detach().clone().requires_grad_(True)
     params = {n: p.detach().clone().requires_grad_(True) for n, p in layer.named_parameters()
               if not n.startswith("running")}
