@@ -36,10 +36,10 @@ spiking CNN on CIFAR-shaped random data (conv / linear / pooling on PyTorch-ROCm
 through ``snnlib_op.Fire``) and reports the end-to-end step time and the share of it spent in the
 fire kernels, measured with events around the ``snnlib.fire_s_fp`` / ``snnlib.fire_bp`` calls.
 
-``--workload bn_fire`` times the batch-norm + fire op (``snnlif_bn_fire_s_fp`` / ``snnlif_bn_fire_bp``)
-at the headline shape through the C ABI: 8 B per neuron-step forward, 20 B backward (two sweeps over
-x and the spike gradient, one write of the input gradient), checked against the CPU oracle on a
-sample of channels.
+``--workload bn_fire`` times the batch-norm + fire layer's training step (``snnlif_bn_stats``,
+``snnlif_bn_fire_s_fp``, ``snnlif_bn_fire_bp``) at the headline shape through the C ABI: 4 B per
+neuron-step for the batch statistics, 8 B forward, 20 B backward (two sweeps over x and the spike
+gradient, one write of the input gradient), checked against the CPU oracle on a sample of channels.
 """
 import argparse
 import json
@@ -312,11 +312,17 @@ def run_bn_fire(args):
     g = torch.randn(shape, generator=gen, device=dev)
     weight = 0.5 + torch.rand(C, generator=gen, device=dev)
     bias = 0.2 * torch.randn(C, generator=gen, device=dev)
-    var, mean = torch.var_mean(x, dim=(0, 1, 3, 4), unbiased=False)
+    var, mean = torch.empty_like(weight), torch.empty_like(weight)
+    stats_ws = torch.empty(lif_cabi.bn_stats_workspace_bytes(lif_cabi.DTYPE_F32, T, B, C, HW),
+                           dtype=torch.uint8, device=dev)
+    lif_cabi.bn_stats_into(x, mean, var, stats_ws)
     ivar, spike = torch.empty_like(var), torch.empty_like(x)
     gx, gw, gb = torch.empty_like(x), torch.empty_like(weight), torch.empty_like(weight)
     ws = torch.empty(lif_cabi.bn_fire_bp_workspace_bytes(lif_cabi.DTYPE_F32, T, B, C, HW),
                      dtype=torch.uint8, device=dev)
+
+    def stats():
+        lif_cabi.bn_stats_into(x, mean, var, stats_ws)
 
     def fwd():
         lif_cabi.bn_fire_s_fp_into(x, weight, bias, var, mean, ivar, spike, eps, ALPHA, THRESH)
@@ -326,25 +332,30 @@ def run_bn_fire(args):
                                  INTERVAL, ws)
 
     for _ in range(args.warmup):
+        stats()
         fwd()
         bwd()
-    # the backward is several kernels: stream markers around each pass (dispatch gaps included)
-    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(args.steps)]
+    # a step is what the layer does in training: batch statistics, forward, backward.  The statistics
+    # and the backward are several kernels each: stream markers around each pass (dispatch gaps included)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for k in range(args.steps):
         ev[k][0].record()
-        fwd()
+        stats()
         ev[k][1].record()
-        bwd()
+        fwd()
         ev[k][2].record()
+        bwd()
+        ev[k][3].record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
-    bwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    stats_ms = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    fwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    bwd_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / args.steps
 
     result = {
-        "metric": "BnFire fwd+bwd neuron-steps/s (next-row op, not the headline metric)",
+        "metric": "BnFire statistics+fwd+bwd neuron-steps/s (next-row op, not the headline metric)",
         "value": ns * args.steps / wall, "unit": "neuron-steps/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3, "higher_is_better": True,
         "dtype": "f32", "data": "synthetic",
@@ -358,7 +369,11 @@ def run_bn_fire(args):
                      "traffic_source": MEASURED_TRAFFIC["bn_fire"]["source"],
                      "fwd": {"algorithmic_bytes_per_launch": 8 * ns, "avg_launch_ms": fwd_ms,
                              "achieved": 8 * ns / (fwd_ms * 1e-3) / 1e9,
-                             "frac": 8 * ns / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
+                             "frac": 8 * ns / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+                     "stats": {"kernel": "bn_stats_wave_kernel + bn_stats_finalize_kernel",
+                               "algorithmic_bytes_per_launch": 4 * ns, "avg_launch_ms": stats_ms,
+                               "achieved": 4 * ns / (stats_ms * 1e-3) / 1e9,
+                               "frac": 4 * ns / (stats_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
     }
     if not args.no_cpu_baseline:
         # CPU leg: the scalar C loops of the oracle on a bounded sample (channels are independent given

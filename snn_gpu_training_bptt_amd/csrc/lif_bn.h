@@ -43,7 +43,10 @@ inline size_t bn_backward_workspace_elems(int64_t B, int64_t C, int64_t HW) {
 // Batch statistics (lif_bn_stats.h): threads per workgroup of the partial-sum kernels, the number of
 // slices the rows of a small-plane tensor are dealt to (enough workgroups to fill the chip), partial
 // sums per quantity (one per wavefront, or one per (slice, column)), and the workspace in elements.
-constexpr int kStatsBlock = 256;
+#ifndef SNNLIF_STATS_BLOCK
+#define SNNLIF_STATS_BLOCK 256
+#endif
+constexpr int kStatsBlock = SNNLIF_STATS_BLOCK;
 inline int bn_stats_row_slices(int64_t rows, int64_t CHW) {
     const int64_t groups = (CHW + kStatsBlock - 1) / kStatsBlock;
     int64_t s = (2048 + groups - 1) / groups;

@@ -31,43 +31,84 @@
 
 namespace snnlif {
 
-constexpr int kStatsRows = 8;  // rows requested before the first is consumed
+// Rows requested before the first is consumed, and wavefronts per SIMD of the partial-sum kernels.
+#ifndef SNNLIF_STATS_ROWS
+#define SNNLIF_STATS_ROWS 8
+#endif
+#ifndef SNNLIF_STATS_WAVES
+#define SNNLIF_STATS_WAVES 8
+#endif
+constexpr int kStatsRows = SNNLIF_STATS_ROWS;
 
-// Planes of at least 32 positions.  part_* indexed [plane][chunk] like the backward's partial sums.
-template <typename F>
-__global__ void __launch_bounds__(kStatsBlock)
+// Bytes per load of a lane of the plane-aligned kernel.  One element per lane, as in the fire
+// kernels: measured on MI355X at [8,64,128,32,32] with nothing cached, dword lanes read at 72 % of
+// the HBM peak, 8-byte lanes at 62 %, 16-byte lanes at 57-68 % depending on the workgroup size.
+#ifndef SNNLIF_STATS_LANE_BYTES
+#define SNNLIF_STATS_LANE_BYTES 4
+#endif
+
+// Adds the group sums of kStatsRows x V values (sum of d and of d*d, d = value - shift, in the storage
+// type) to the running sums in double.
+template <typename F, int V>
+__device__ __forceinline__ void stats_add_group(const Pack<F, V> (&v)[kStatsRows], F shift,
+                                                double& acc_d, double& acc_dd) {
+    F group_d = F(0), group_dd = F(0);
+#pragma unroll
+    for (int r = 0; r < kStatsRows; ++r) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            const F d = v[r].e[j] - shift;
+            group_d += d;
+            group_dd += d * d;
+        }
+    }
+    acc_d += static_cast<double>(group_d);
+    acc_dd += static_cast<double>(group_dd);
+}
+
+template <typename F, int V>
+__device__ __forceinline__ Pack<F, V> stats_fill(F value) {
+    Pack<F, V> p;
+#pragma unroll
+    for (int j = 0; j < V; ++j) p.e[j] = value;
+    return p;
+}
+
+// Planes of at least 32 positions.  A wavefront covers 64*V consecutive positions of one plane
+// (G = ceil(HW / (64*V)) wavefronts per plane; HW is a multiple of V); part_* indexed [plane][chunk].
+template <typename F, int V>
+__global__ void __launch_bounds__(kStatsBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_STATS_WAVES)
 bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restrict__ part_dd, int T,
-                     int64_t N, int64_t C, int64_t HW) {
-    const int64_t G = (HW + 63) / 64;
+                     int64_t N, int64_t C, int64_t HW, int64_t G) {
     const int64_t lanes = (N / HW) * G * 64;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t pc = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; pc < lanes;
          pc += stride) {
         const int64_t wave = pc >> 6;
         const int64_t plane = wave / G;
-        const int64_t k = (wave - plane * G) * 64 + (pc & 63);
+        const int64_t k = ((wave - plane * G) * 64 + (pc & 63)) * V;
         const int c = static_cast<int>(plane % C);
         double acc_d = 0.0, acc_dd = 0.0;
         if (k < HW) {
             const F shift = x[static_cast<int64_t>(c) * HW];
             const F* col = x + plane * HW + k;
-            for (int t0 = 0; t0 < T; t0 += kStatsRows) {
-                F v[kStatsRows];
+            int t0 = 0;
+            for (; t0 + kStatsRows <= T; t0 += kStatsRows) {  // whole groups: straight-line loads
+                Pack<F, V> v[kStatsRows];
+#pragma unroll
+                for (int r = 0; r < kStatsRows; ++r)
+                    v[r] = load_pack<F, V, false>(col + static_cast<int64_t>(t0 + r) * N);
+                stats_add_group<F, V>(v, shift, acc_d, acc_dd);
+            }
+            if (t0 < T) {
+                Pack<F, V> v[kStatsRows];
 #pragma unroll
                 for (int r = 0; r < kStatsRows; ++r) {
-                    v[r] = shift;  // rows past the end contribute d = 0
+                    v[r] = stats_fill<F, V>(shift);  // rows past the end contribute d = 0
                     if (t0 + r < T)
-                        v[r] = load_pack<F, 1, false>(col + static_cast<int64_t>(t0 + r) * N).e[0];
+                        v[r] = load_pack<F, V, false>(col + static_cast<int64_t>(t0 + r) * N);
                 }
-                F group_d = F(0), group_dd = F(0);
-#pragma unroll
-                for (int r = 0; r < kStatsRows; ++r) {
-                    const F d = v[r] - shift;
-                    group_d += d;
-                    group_dd += d * d;
-                }
-                acc_d += static_cast<double>(group_d);
-                acc_dd += static_cast<double>(group_dd);
+                stats_add_group<F, V>(v, shift, acc_d, acc_dd);
             }
         }
         acc_d = wave_sum(acc_d);
@@ -92,22 +133,14 @@ bn_stats_column_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __res
     const F shift = x[(j / HW) * HW];
     double acc_d = 0.0, acc_dd = 0.0;
     for (int64_t r0 = s; r0 < rows; r0 += static_cast<int64_t>(S) * kStatsRows) {
-        F v[kStatsRows];
+        Pack<F, 1> v[kStatsRows];
 #pragma unroll
         for (int q = 0; q < kStatsRows; ++q) {
             const int64_t r = r0 + static_cast<int64_t>(q) * S;
-            v[q] = shift;
-            if (r < rows) v[q] = load_pack<F, 1, false>(x + r * CHW + j).e[0];
+            v[q] = stats_fill<F, 1>(shift);
+            if (r < rows) v[q] = load_pack<F, 1, false>(x + r * CHW + j);
         }
-        F group_d = F(0), group_dd = F(0);
-#pragma unroll
-        for (int q = 0; q < kStatsRows; ++q) {
-            const F d = v[q] - shift;
-            group_d += d;
-            group_dd += d * d;
-        }
-        acc_d += static_cast<double>(group_d);
-        acc_dd += static_cast<double>(group_dd);
+        stats_add_group<F, 1>(v, shift, acc_d, acc_dd);
     }
     part_d[static_cast<int64_t>(s) * CHW + j] = static_cast<F>(acc_d);
     part_dd[static_cast<int64_t>(s) * CHW + j] = static_cast<F>(acc_dd);
@@ -168,10 +201,22 @@ int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,
     F* part_dd = workspace + P;
     const double count = static_cast<double>(T) * static_cast<double>(B) * static_cast<double>(HW);
     if (bn_wave_partials(HW)) {
-        const int64_t G = (HW + 63) / 64;
-        launch_kernel(bn_stats_wave_kernel<F>, dim3(grid_for(B * C * G * 64, kStatsBlock)),
-                      dim3(kStatsBlock), 0, stream, x, part_d, part_dd, static_cast<int>(T), N, C, HW);
-        int rc = launch_status();
+        // widest lanes for which rows, planes and the base address stay aligned and a wavefront
+        // still has work for most of its lanes (the partial-sum arrays are sized for V = 1, the
+        // case with the most wavefronts per plane)
+        constexpr int maxv = SNNLIF_STATS_LANE_BYTES / static_cast<int>(sizeof(F)) < 1
+                                 ? 1
+                                 : SNNLIF_STATS_LANE_BYTES / static_cast<int>(sizeof(F));
+        int v = maxv;
+        while (v > 1 && (HW % v != 0 || HW < 64 * v || !aligned_to(x, sizeof(F) * v))) v >>= 1;
+        const int64_t G = (HW + 64 * v - 1) / (64 * v);
+        const dim3 grid(grid_for(B * C * G * 64, kStatsBlock)), block(kStatsBlock);
+        const int rc = with_vec<maxv>(v, [&](auto vc) {
+            constexpr int V = decltype(vc)::value;
+            launch_kernel(bn_stats_wave_kernel<F, V>, grid, block, 0, stream, x, part_d, part_dd,
+                          static_cast<int>(T), N, C, HW, G);
+            return launch_status();
+        });
         if (rc != SNNLIF_OK) return rc;
         launch_kernel(bn_stats_finalize_kernel<F>, dim3(static_cast<unsigned>(C)), dim3(kReduceBlock),
                       0, stream, x, part_d, part_dd, out_a, out_b, HW, B, G, C * G, count, moments);
