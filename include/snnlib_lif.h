@@ -69,7 +69,7 @@ extern "C" {
 #define SNNLIF_ERR_WORKSPACE  -3 /* workspace missing or smaller than snnlif_fire_bp_workspace_bytes() */
 #define SNNLIF_ERR_ALIGN      -4 /* a pointer is not aligned to its element size */
 #define SNNLIF_ERR_SCRATCH    -6 /* shape needs more than SNNLIF_STATIC_SCRATCH_BYTES (snnlif_bn_fire_bp_static) */
-#define SNNLIF_ERR_UNSUPPORTED -5 /* valid arguments this entry point does not implement (see its comment) */
+#define SNNLIF_ERR_UNSUPPORTED -5 /* valid arguments this entry point does not implement (bf16 in the batch-norm ones) */
 
 /* Every T up to this keeps the whole recomputed membrane potential in registers in the backward
  * (one kernel, 12 bytes per neuron-step in fp32); so do T = 40, 48, 56 and 64 exactly. */
@@ -93,16 +93,21 @@ const char* snnlif_target_arch(void);
 const char* snnlif_strerror(int code);
 
 /*
- * Arms kernel-exact timing for the calling thread: the first kernel that the next snnlif_* entry
- * point called from this thread launches gets the two events (hipEvent_t created with timing enabled,
- * passed as void*; either may be NULL) attached to its dispatch -- `start_event` completes when that
- * kernel begins, `stop_event` when it has finished -- so hipEventElapsedTime(start, stop) is the
+ * Arms timing for the next snnlif_* entry point called from this thread (two hipEvent_t created with
+ * timing enabled, passed as void*; either may be NULL; two NULLs disarm).
+ * Entry points that launch one kernel (snnlif_fire_s_fp, snnlif_fire_us_fp, snnlif_fire_bp up to
+ * SNNLIF_BP_NO_WORKSPACE_MAX_T steps, snnlif_bn_fire_s_fp, snnlif_bn_fire_s_recompute,
+ * snnlif_bn_fire_bp_dist2) get the events attached to that dispatch -- `start_event` completes when
+ * the kernel begins, `stop_event` when it has finished -- so hipEventElapsedTime(start, stop) is the
  * kernel's own duration, without the dispatch gaps an interval between two hipEventRecord markers
- * contains.  The arming is consumed by that one launch; passing two NULLs disarms.  Entry points
- * that launch one kernel (snnlif_fire_s_fp, snnlif_fire_us_fp, snnlif_fire_bp up to
- * SNNLIF_BP_NO_WORKSPACE_MAX_T, snnlif_bn_fire_s_fp, snnlif_bn_fire_s_recompute) are timed whole; of
- * the others only the first kernel is.  Not meant for use under HIP graph capture.  No counterpart in
- * the reference (which has no timing hooks); for benchmarks and profilers built on this ABI.
+ * contains.  Entry points that launch several kernels (snnlif_bn_stats, snnlif_bn_fire_bp and its
+ * _static and _dist1 forms, snnlif_fire_bp beyond SNNLIF_BP_NO_WORKSPACE_MAX_T steps) record
+ * `start_event` on the stream before their first kernel and `stop_event` after their last: the whole
+ * operation, gaps between its kernels included.
+ * The arming is consumed by that one call whatever its outcome: a call that returns an argument error
+ * or finds an empty shape leaves the events unrecorded and the timer disarmed.  Not meant for use under
+ * HIP graph capture.  No counterpart in the reference (which has no timing hooks); for benchmarks and
+ * profilers built on this ABI.
  */
 int snnlif_time_next_kernel(void* start_event, void* stop_event);
 
@@ -203,12 +208,15 @@ int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const vo
 
 /* Bytes of device workspace snnlif_bn_fire_bp needs: two partial sums of the storage type per
  * wavefront of sweep 1 (ceil(HW/64) wavefronts per (batch entry, channel) plane) when HW >= 32, two
- * per neuron otherwise, plus per-channel staging.  0 for invalid arguments. */
+ * per neuron plus their batch-sliced column sums otherwise, per-channel staging, and for
+ * T > SNNLIF_BP_NO_WORKSPACE_MAX_T one membrane potential per 32-step segment and neuron.
+ * 0 for invalid arguments. */
 size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);
 
 /*
- * Batch-norm + fire backward (fp32 or fp64; T <= SNNLIF_BP_NO_WORKSPACE_MAX_T, else
- * SNNLIF_ERR_UNSUPPORTED; windows longer than SNNLIF_BP_FUSED_MAX_T read x twice per sweep).
+ * Batch-norm + fire backward (fp32 or fp64; any T; windows longer than SNNLIF_BP_FUSED_MAX_T are cut
+ * into 32-step segments and read x twice per sweep, with the membrane potential at the segment
+ * boundaries in LDS up to SNNLIF_BP_NO_WORKSPACE_MAX_T steps and in device memory beyond).
  * With u recomputed from scale[c] = weight[c]*ivar[c], gy the fire reverse chain (see
  * snnlif_fire_bp), xhat = (x - mean[c])*ivar[c] and M = T*B*HW:
  *   grad_bias[c] = sum gy;   grad_weight[c] = sum gy*xhat
@@ -248,8 +256,7 @@ int snnlif_bn_fire_bp_static(const void* spatial, const void* weight, const void
 
 /*
  * The same backward in the two halves that a batch sharded over several GPUs runs on either side of
- * an all-reduce (fp32 or fp64, T <= SNNLIF_BP_NO_WORKSPACE_MAX_T, shapes and workspace as snnlif_bn_fire_bp;
- * B is the local batch).
+ * an all-reduce (fp32 or fp64, any T, shapes and workspace as snnlif_bn_fire_bp; B is the local batch).
  *
  * snnlif_bn_fire_bp_dist1: the local parameter gradients and the local per-channel means
  *   mean_gxhat[c]  = weight[c] * (sum gy)      / (T*B*HW)
@@ -260,7 +267,8 @@ int snnlif_bn_fire_bp_static(const void* spatial, const void* weight, const void
  *
  * snnlif_bn_fire_bp_dist2: the input gradient from the two means averaged over all ranks,
  *   grad_spatial = (gy*weight[c])*ivar[c] - ivar[c]*((xhat*grad_xhatx[c]) + grad_xhat[c])
- * Needs no workspace.  Replaces bn_fire_bp_cuda_dist2 (snnlib/cuda/snn_kernel_bp.cu:811-854), bound
+ * Needs no workspace (beyond SNNLIF_BP_NO_WORKSPACE_MAX_T steps it parks the segment boundary potentials in
+ * rows of grad_spatial that it overwrites later in the same call).  Replaces bn_fire_bp_cuda_dist2 (snnlib/cuda/snn_kernel_bp.cu:811-854), bound
  * as snnlib.bn_fire_bp_dist2 (snnlib/cuda/snn.cpp:827).
  *
  * dist1 followed by dist2 on the same arrays is snnlif_bn_fire_bp, bit for bit.  The all-reduce

@@ -15,6 +15,7 @@ static __device__ __align__(256) unsigned char scratch[SNNLIF_STATIC_SCRATCH_BYT
 
 namespace snnlif {
 thread_local KernelTimer tl_kernel_timer;
+thread_local hipError_t tl_launch_error = hipSuccess;
 }  // namespace snnlif
 
 namespace {
@@ -62,6 +63,32 @@ int static_scratch(void** out) {
     return SNNLIF_OK;
 }
 
+// Every entry point that can launch holds one of these: whatever way it returns (argument error,
+// empty shape, launch), a timer armed with snnlif_time_next_kernel() does not outlive the call and
+// cannot end up on a later, unrelated launch.
+struct TimerScope {
+    ~TimerScope() { snnlif::tl_kernel_timer = snnlif::KernelTimer{}; }
+};
+
+// For entry points that launch several kernels: the armed events bracket the whole operation
+// (start recorded on the stream before the first kernel, stop after the last, dispatch gaps
+// included) instead of riding on the first dispatch alone.
+struct OperationTimer {
+    snnlif::KernelTimer timer;
+    hipStream_t stream;
+    // active = false: a single-kernel case of the same entry point; the timer stays armed for the
+    // dispatch itself
+    explicit OperationTimer(hipStream_t st, bool active = true) : stream(st) {
+        if (!active) return;
+        timer = snnlif::tl_kernel_timer;
+        snnlif::tl_kernel_timer = snnlif::KernelTimer{};
+        if (timer.start != nullptr) (void)hipEventRecord(timer.start, stream);
+    }
+    ~OperationTimer() {
+        if (timer.stop != nullptr) (void)hipEventRecord(timer.stop, stream);
+    }
+};
+
 inline int shape_error(int64_t T, int64_t N) {
     if (T < 0 || N < 0) return SNNLIF_ERR_ARG;
     if (T > 0x7fffffff) return SNNLIF_ERR_ARG;
@@ -91,7 +118,7 @@ const char* snnlif_strerror(int code) {
         case SNNLIF_ERR_WORKSPACE: return "snnlif: workspace missing or smaller than snnlif_fire_bp_workspace_bytes()";
         case SNNLIF_ERR_ALIGN: return "snnlif: pointer not aligned to its element size (workspace: 16 bytes)";
         case SNNLIF_ERR_SCRATCH: return "snnlif: this shape needs more scratch memory than the library's fixed array holds (SNNLIF_STATIC_SCRATCH_BYTES); call snnlif_bn_fire_bp with a workspace instead";
-        case SNNLIF_ERR_UNSUPPORTED: return "snnlif: not implemented for these arguments (batch-norm fire: fp32 / fp64 only, backward T <= 1024)";
+        case SNNLIF_ERR_UNSUPPORTED: return "snnlif: not implemented for these arguments (batch-norm entry points take fp32 / fp64 only)";
         default: break;
     }
     if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
@@ -100,6 +127,7 @@ const char* snnlif_strerror(int code) {
 
 int snnlif_fire_us_fp(const void* spatial, void* mem, void* spike, int dtype, int64_t T, int64_t N,
                       float alpha, float thresh, void* stream) {
+    const TimerScope timer_scope;
     if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
     const int se = shape_error(T, N);
     if (se != SNNLIF_OK) return se;
@@ -116,6 +144,7 @@ int snnlif_fire_us_fp(const void* spatial, void* mem, void* spike, int dtype, in
 
 int snnlif_fire_s_fp(const void* spatial, void* spike, int dtype, int64_t T, int64_t N,
                      float alpha, float thresh, void* stream) {
+    const TimerScope timer_scope;
     if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
     const int se = shape_error(T, N);
     if (se != SNNLIF_OK) return se;
@@ -134,6 +163,7 @@ size_t snnlif_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t N) {
 int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spatial, int dtype,
                    int64_t T, int64_t N, float alpha, float thresh, float beta, float interval,
                    void* workspace, size_t workspace_bytes, void* stream) {
+    const TimerScope timer_scope;
     if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
     const int se = shape_error(T, N);
     if (se != SNNLIF_OK) return se;
@@ -141,6 +171,9 @@ int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spati
     if (spatial == nullptr || grad_spike == nullptr || grad_spatial == nullptr) return SNNLIF_ERR_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const snnlif::SpatialHint keep = hint_of(dtype);
+    // one kernel up to SNNLIF_BP_NO_WORKSPACE_MAX_T steps; beyond, a recompute kernel and a reverse kernel
+    const bool two_kernels = T > SNNLIF_BP_NO_WORKSPACE_MAX_T;
+    const OperationTimer whole_operation(st, two_kernels);
     switch (storage_of(dtype)) {
         case SNNLIF_DTYPE_F32:
             return snnlif::backward_f32(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
@@ -194,6 +227,7 @@ static bool all_aligned(const void* const* ptrs, int n, size_t bytes) {
 int snnlif_bn_fire_s_fp(const void* spatial, const void* weight, const void* bias, const void* var,
                         const void* mean, void* ivar, void* spike, int dtype, int64_t T, int64_t B,
                         int64_t C, int64_t HW, float eps, float alpha, float thresh, void* stream) {
+    const TimerScope timer_scope;
     int rc = SNNLIF_OK;
     const size_t es = bn_element_size(dtype, &rc);
     if (es == 0) return rc;
@@ -216,6 +250,7 @@ int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const vo
                                const void* ivar, const void* mean, void* spike, int dtype, int64_t T,
                                int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
                                void* stream) {
+    const TimerScope timer_scope;
     int rc = SNNLIF_OK;
     const size_t es = bn_element_size(dtype, &rc);
     if (es == 0) return rc;
@@ -245,6 +280,7 @@ size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t 
 int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64_t T, int64_t B,
                     int64_t C, int64_t HW, int raw_moments, void* workspace, size_t workspace_bytes,
                     void* stream) {
+    const TimerScope timer_scope;
     int rc = SNNLIF_OK;
     const size_t es = bn_element_size(dtype, &rc);
     if (es == 0) return rc;
@@ -260,6 +296,7 @@ int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64
     if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
     if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const OperationTimer whole_operation(st);
     return SNNLIF_BN_DISPATCH(
         es,
         snnlif::bn_stats_f32(CF(spatial), MF(mean), MF(var), raw_moments != 0, T, B, C, HW,
@@ -273,10 +310,14 @@ size_t snnlif_bn_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_
     const size_t es = bn_element_size(dtype, &rc);
     if (es == 0 || bn_shape_error(T, B, C, HW) != SNNLIF_OK) return 0;
     if (T == 0 || B * C * HW == 0) return 0;
-    return snnlif::bn_backward_workspace_elems(B, C, HW) * es;
+    return snnlif::bn_backward_workspace_elems(T, B, C, HW) * es;
 }
 
 // Shared argument checks of the three backward entry points; `needs_workspace` = sweep 1 runs.
+static_assert(snnlif::kBnLdsBoundaryMaxT == SNNLIF_BP_NO_WORKSPACE_MAX_T &&
+                  snnlif::kBnSegment == snnlif::kSegment,
+              "the batch-norm backward cuts time the way the plain backward does");
+
 static int bn_backward_checks(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW,
                               const void* const* ptrs, int n, bool needs_workspace,
                               const void* workspace, size_t workspace_bytes, size_t* es_out,
@@ -289,12 +330,11 @@ static int bn_backward_checks(int dtype, int64_t T, int64_t B, int64_t C, int64_
     *es_out = es;
     *empty = (T == 0 || B * C * HW == 0);
     if (*empty) return SNNLIF_OK;
-    if (T > SNNLIF_BP_NO_WORKSPACE_MAX_T) return SNNLIF_ERR_UNSUPPORTED;
     for (int i = 0; i < n; ++i)
         if (ptrs[i] == nullptr) return SNNLIF_ERR_ARG;
     if (!all_aligned(ptrs, n, es)) return SNNLIF_ERR_ALIGN;
     if (needs_workspace) {
-        const size_t need = snnlif::bn_backward_workspace_elems(B, C, HW) * es;
+        const size_t need = snnlif::bn_backward_workspace_elems(T, B, C, HW) * es;
         if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
         if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
     }
@@ -306,6 +346,7 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
                       void* grad_weight, void* grad_bias, int dtype, int64_t T, int64_t B, int64_t C,
                       int64_t HW, float alpha, float thresh, float beta, float interval,
                       void* workspace, size_t workspace_bytes, void* stream) {
+    const TimerScope timer_scope;
     const void* ptrs[9] = {spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
                            grad_bias};
     size_t es = 0;
@@ -314,6 +355,7 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
                                       &es, &empty);
     if (rc != SNNLIF_OK || empty) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const OperationTimer whole_operation(st);
     return SNNLIF_BN_DISPATCH(
         es,
         snnlif::bn_backward_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean), CF(grad_spike),
@@ -329,13 +371,14 @@ int snnlif_bn_fire_bp_static(const void* spatial, const void* weight, const void
                              void* grad_spatial, void* grad_weight, void* grad_bias, int dtype,
                              int64_t T, int64_t B, int64_t C, int64_t HW, float alpha, float thresh,
                              float beta, float interval, void* stream) {
+    const TimerScope timer_scope;
     const void* ptrs[9] = {spatial, weight, bias, ivar, mean, grad_spike, grad_spatial, grad_weight,
                            grad_bias};
     size_t es = 0;
     bool empty = false;
     int rc = bn_backward_checks(dtype, T, B, C, HW, ptrs, 9, false, nullptr, 0, &es, &empty);
     if (rc != SNNLIF_OK || empty) return rc;
-    if (snnlif::bn_backward_workspace_elems(B, C, HW) * es > SNNLIF_STATIC_SCRATCH_BYTES)
+    if (snnlif::bn_backward_workspace_elems(T, B, C, HW) * es > SNNLIF_STATIC_SCRATCH_BYTES)
         return SNNLIF_ERR_SCRATCH;
     void* workspace = nullptr;
     rc = static_scratch(&workspace);
@@ -343,6 +386,7 @@ int snnlif_bn_fire_bp_static(const void* spatial, const void* weight, const void
     // Every value the reduction reads from the scratch array is written by sweep 1 of this same call,
     // so nothing has to be cleared between calls.
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const OperationTimer whole_operation(st);
     return SNNLIF_BN_DISPATCH(
         es,
         snnlif::bn_backward_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean), CF(grad_spike),
@@ -359,6 +403,7 @@ int snnlif_bn_fire_bp_dist1(const void* spatial, const void* weight, const void*
                             int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
                             float thresh, float beta, float interval, void* workspace,
                             size_t workspace_bytes, void* stream) {
+    const TimerScope timer_scope;
     const void* ptrs[10] = {spatial, weight, bias, ivar, mean, grad_spike, mean_gxhat, mean_gxhatx,
                             grad_weight, grad_bias};
     size_t es = 0;
@@ -368,6 +413,7 @@ int snnlif_bn_fire_bp_dist1(const void* spatial, const void* weight, const void*
                                       workspace_bytes, &es, &empty);
     if (rc != SNNLIF_OK || empty) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const OperationTimer whole_operation(st);
     return SNNLIF_BN_DISPATCH(
         es,
         snnlif::bn_backward_stats_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean),
@@ -385,6 +431,7 @@ int snnlif_bn_fire_bp_dist2(const void* spatial, const void* weight, const void*
                             const void* grad_xhat, const void* grad_xhatx, void* grad_spatial,
                             int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
                             float thresh, float beta, float interval, void* stream) {
+    const TimerScope timer_scope;
     const void* ptrs[9] = {spatial, weight, bias, ivar, mean, grad_spike, grad_xhat, grad_xhatx,
                            grad_spatial};
     size_t es = 0;

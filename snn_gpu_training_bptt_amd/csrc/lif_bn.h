@@ -10,16 +10,6 @@
 
 namespace snnlif {
 
-// Number of batch slices each channel's reduction is split into (enough workgroups to fill the
-// chip when there are few channels).
-inline int bn_reduce_splits(int64_t B, int64_t C) {
-    int64_t s = 2048 / (C > 0 ? C : 1);
-    if (s < 1) s = 1;
-    if (s > B) s = B;
-    if (s > 65535) s = 65535;
-    return static_cast<int>(s);
-}
-
 // Sweep 1 of the backward lays wavefronts over the (batch entry, channel) planes when a plane has at
 // least this many positions (all lanes of a wavefront then share a channel and fold their sums by
 // shuffles); smaller planes keep one lane per neuron in storage order.
@@ -32,12 +22,36 @@ inline size_t bn_partial_count(int64_t B, int64_t C, int64_t HW) {
     return static_cast<size_t>(B * C * HW);
 }
 
+// Per-neuron partial sums are a [B, C*HW] matrix whose columns are summed over the batch in S slices
+// (enough workgroups of kReduceBlock columns to fill the chip), then folded per channel.
+constexpr int kReduceBlock = 256;
+inline int bn_reduce_splits(int64_t B, int64_t CHW) {
+    const int64_t groups = (CHW + kReduceBlock - 1) / kReduceBlock;
+    int64_t s = (1024 + groups - 1) / groups;
+    if (s > 64) s = 64;
+    if (s > B) s = B;
+    if (s < 1) s = 1;
+    return static_cast<int>(s);
+}
+
+// Windows longer than this keep the membrane potential at the segment boundaries in device memory
+// instead of LDS: sweep 1 in its workspace, sweep 2 in rows of the gradient it has yet to write.
+constexpr int64_t kBnLdsBoundaryMaxT = 1024;
+constexpr int64_t kBnSegment = 32;
+inline size_t bn_boundary_elems(int64_t T, int64_t B, int64_t C, int64_t HW) {
+    if (T <= kBnLdsBoundaryMaxT) return 0;
+    return static_cast<size_t>((T + kBnSegment - 1) / kBnSegment) * static_cast<size_t>(B * C * HW);
+}
+
 // Workspace of the backward in elements of the scalar type:
-// part_gy[P], part_gyx[P], split[2*S*C] (per-neuron partials only), coef[2*C], P = bn_partial_count.
-inline size_t bn_backward_workspace_elems(int64_t B, int64_t C, int64_t HW) {
-    const size_t split =
-        bn_wave_partials(HW) ? 0 : static_cast<size_t>(2) * bn_reduce_splits(B, C) * static_cast<size_t>(C);
-    return 2 * bn_partial_count(B, C, HW) + split + static_cast<size_t>(2 * C);
+// part_gy[P], part_gyx[P], split[2*S*C*HW] (per-neuron partials only), coef[2*C],
+// boundary[ceil(T/32)*N] (T > 1024 only); P = bn_partial_count.
+inline size_t bn_backward_workspace_elems(int64_t T, int64_t B, int64_t C, int64_t HW) {
+    const size_t split = bn_wave_partials(HW)
+                             ? 0
+                             : static_cast<size_t>(2) * bn_reduce_splits(B, C * HW) * static_cast<size_t>(C * HW);
+    return 2 * bn_partial_count(B, C, HW) + split + static_cast<size_t>(2 * C) +
+           bn_boundary_elems(T, B, C, HW);
 }
 
 // Batch statistics (lif_bn_stats.h): threads per workgroup of the partial-sum kernels, the number of

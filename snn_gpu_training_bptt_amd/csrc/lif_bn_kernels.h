@@ -21,15 +21,16 @@
 //   1. lif_bn_backward_partial_kernel: reverse chain per neuron, sums over its T steps, and -- for
 //      planes of at least 32 positions, over which wavefronts are laid so that all 64 lanes share a
 //      channel -- over the wavefront by shuffles: two floats per wavefront (per neuron otherwise);
-//   2. bn_channel_reduce_finalize_kernel (or bn_channel_reduce_kernel + bn_channel_finalize_kernel
+//   2. bn_channel_reduce_finalize_kernel (or bn_column_reduce_kernel + bn_channel_finalize_kernel
 //      for per-neuron partials): per-channel sums of those partials (wavefront shuffles, then LDS
-//      across the waves of a workgroup; the only place in this library where lanes cooperate), in
-//      an order fixed by the launch geometry -> bit-reproducible results;
+//      across the waves of a workgroup, for the per-wavefront form; column sums over the batch
+//      for the per-neuron form), in an order fixed by the launch geometry -> bit-reproducible results;
 //   3. lif_bn_backward_input_kernel: the chain again (x and g re-read: 8 B per neuron-step, the
 //      same as storing and re-loading gy would cost) and the input gradient.
-// Windows of more than 32 steps (up to 1024) run both sweeps in 32-step segments with the membrane
-// potential at the segment boundaries kept in LDS (bn_reverse_segmented): x is then read twice per
-// sweep.
+// Windows of more than 32 steps run both sweeps in 32-step segments with the membrane potential at
+// the segment boundaries kept aside (bn_reverse_segmented): x is then read twice per sweep.  Up to
+// 1024 steps the boundary values live in LDS; beyond, sweep 1 keeps them in its workspace and sweep 2
+// in rows of the input gradient that it has not written yet (a lane only ever touches its own column).
 // HBM traffic: forward 8 B, backward 20 B (+ at most 16/T B) per neuron-step up to 32 steps, 28 B
 // beyond; the reference moves 8 and 36.
 #ifndef SNNLIF_LIF_BN_KERNELS_H
@@ -39,8 +40,6 @@
 #include "lif_kernels.h"
 
 namespace snnlif {
-
-constexpr int kReduceBlock = 256;
 
 __device__ __forceinline__ float real_sqrt(float v) { return sqrtf(v); }
 __device__ __forceinline__ double real_sqrt(double v) { return sqrt(v); }
@@ -174,14 +173,18 @@ __device__ __forceinline__ void bn_reverse_chain(const F* __restrict__ x,
 
 // Time axes longer than one register window, in segments of kSegment steps, the way
 // lif_backward_segmented_kernel does it: forward over all but the last segment keeping the membrane
-// potential at each boundary in this lane's own LDS slots (`boundary`: [segment][blockDim.x] floats
-// of dynamic LDS), then the segments last to first.  emit gets the absolute time step.
+// potential at each boundary in a slot of this lane's own, then the segments last to first.  The slot
+// of segment `seg` (the potential after step seg*kSegment - 1, seg >= 1) is
+// boundary[seg * bstride + boff]: dynamic LDS ([segment][blockDim.x]: bstride = blockDim.x, boff =
+// threadIdx.x) or device memory ([segment][N]: bstride = N, boff = col; or rows of the gradient still
+// to be written).  emit gets the absolute time step.
 template <typename F, typename Emit>
 __device__ __forceinline__ void bn_reverse_segmented(const F* __restrict__ x,
                                                      const F* __restrict__ g, int T, int64_t N,
                                                      int64_t col, F m, F scale, F b,
                                                      F alpha, F thresh, F beta,
-                                                     F interval, F* boundary, Emit&& emit) {
+                                                     F interval, F* boundary, int64_t bstride,
+                                                     int64_t boff, Emit&& emit) {
     const int nseg = (T + kSegment - 1) / kSegment;
     constexpr int ROWS = 8;
     static_assert(kSegment % ROWS == 0, "a segment is a whole number of forward groups");
@@ -198,7 +201,7 @@ __device__ __forceinline__ void bn_reverse_segmented(const F* __restrict__ x,
                 sc = (uc > thresh) ? F(1) : F(0);
             }
         }
-        boundary[(seg + 1) * blockDim.x + threadIdx.x] = uc;
+        boundary[static_cast<int64_t>(seg + 1) * bstride + boff] = uc;
     }
     {
         const int t0 = (nseg - 1) * kSegment;
@@ -208,7 +211,7 @@ __device__ __forceinline__ void bn_reverse_segmented(const F* __restrict__ x,
                                            [&](int t, F gy, F xt) { emit(t0 + t, gy, xt); });
     }
     for (int seg = nseg - 2; seg >= 0; --seg) {
-        uc = seg == 0 ? F(0) : boundary[seg * blockDim.x + threadIdx.x];
+        uc = seg == 0 ? F(0) : boundary[static_cast<int64_t>(seg) * bstride + boff];
         sc = (seg != 0 && uc > thresh) ? F(1) : F(0);
         const int t0 = seg * kSegment;
         const int64_t off = static_cast<int64_t>(t0) * N;
@@ -218,15 +221,24 @@ __device__ __forceinline__ void bn_reverse_segmented(const F* __restrict__ x,
     }
 }
 
-// Dispatch between the two: SEGMENTED kernels are instantiated with TW = kSegment.
-template <typename F, int TW, bool EXACT, bool SEGMENTED, typename Emit>
+// How a kernel instance walks time: the whole window in registers, or in segments with the boundary
+// potentials in LDS or in device memory.
+enum class TimeWalk { window, segments_lds, segments_memory };
+
+// Dispatch between them; segmented kernels are instantiated with TW = kSegment.  `far` is the
+// device-memory boundary array (TimeWalk::segments_memory) with its stride and this lane's offset.
+template <typename F, int TW, bool EXACT, TimeWalk WALK, typename Emit>
 __device__ __forceinline__ void bn_reverse(const F* __restrict__ x, const F* __restrict__ g,
                                            int T, int64_t N, int64_t col, F m, F scale,
                                            F b, F alpha, F thresh, F beta,
-                                           F interval, F* boundary, Emit&& emit) {
-    if constexpr (SEGMENTED) {
-        bn_reverse_segmented<F>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, boundary,
-                             emit);
+                                           F interval, F* lds_boundary, F* far, int64_t far_stride,
+                                           int64_t far_offset, Emit&& emit) {
+    if constexpr (WALK == TimeWalk::segments_lds) {
+        bn_reverse_segmented<F>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, lds_boundary,
+                                static_cast<int64_t>(blockDim.x), static_cast<int64_t>(threadIdx.x), emit);
+    } else if constexpr (WALK == TimeWalk::segments_memory) {
+        bn_reverse_segmented<F>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, far,
+                                far_stride, far_offset, emit);
     } else {
         bn_reverse_chain<F, TW, EXACT>(x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, emit);
     }
@@ -246,16 +258,17 @@ __device__ __forceinline__ F wave_sum(F v) {
 // wavefronts per plane, the last one partly idle when HW is not a multiple of 64 -- so all lanes of
 // a wavefront share a channel and their sums are folded by shuffles: one pair of floats per
 // wavefront, part_* indexed [plane][chunk] (B*C*G entries).
-template <typename F, int TW, bool EXACT, bool WAVE, bool SEGMENTED = false>
+// `far`: [segment][N] boundary potentials in the workspace (TimeWalk::segments_memory only).
+template <typename F, int TW, bool EXACT, bool WAVE, TimeWalk WALK = TimeWalk::window>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
 lif_bn_backward_partial_kernel(const F* __restrict__ x, const F* __restrict__ g,
                                const F* __restrict__ weight, const F* __restrict__ bias,
                                const F* __restrict__ ivar, const F* __restrict__ mean,
-                               F* __restrict__ part_gy, F* __restrict__ part_gyx, int T,
-                               int64_t N, int64_t C, int64_t HW, F alpha, F thresh,
+                               F* __restrict__ part_gy, F* __restrict__ part_gyx, F* __restrict__ far,
+                               int T, int64_t N, int64_t C, int64_t HW, F alpha, F thresh,
                                F beta, F interval) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    F* boundary = reinterpret_cast<F*>(lds_raw);  // used by SEGMENTED only
+    F* boundary = reinterpret_cast<F*>(lds_raw);  // used by TimeWalk::segments_lds only
     const bool small = N <= 0xffffffffll;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     if (WAVE) {
@@ -273,12 +286,12 @@ lif_bn_backward_partial_kernel(const F* __restrict__ x, const F* __restrict__ g,
                 const F m = mean[c], iv = ivar[c];
                 const F scale = weight[c] * iv;
                 const F b = bias[c];
-                bn_reverse<F, TW, EXACT, SEGMENTED>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
-                                                 interval, boundary, [&](int, F gy, F xt) {
-                                                     const F xhat = (xt - m) * iv;
-                                                     acc_gy += gy;
-                                                     acc_gyx += gy * xhat;
-                                                 });
+                bn_reverse<F, TW, EXACT, WALK>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
+                                               interval, boundary, far, N, col, [&](int, F gy, F xt) {
+                                                   const F xhat = (xt - m) * iv;
+                                                   acc_gy += gy;
+                                                   acc_gyx += gy * xhat;
+                                               });
             }
             acc_gy = wave_sum(acc_gy);
             acc_gyx = wave_sum(acc_gyx);
@@ -295,12 +308,12 @@ lif_bn_backward_partial_kernel(const F* __restrict__ x, const F* __restrict__ g,
             const F scale = weight[c] * iv;
             const F b = bias[c];
             F acc_gy = F(0), acc_gyx = F(0);
-            bn_reverse<F, TW, EXACT, SEGMENTED>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
-                                             interval, boundary, [&](int, F gy, F xt) {
-                                                 const F xhat = (xt - m) * iv;
-                                                 acc_gy += gy;
-                                                 acc_gyx += gy * xhat;
-                                             });
+            bn_reverse<F, TW, EXACT, WALK>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
+                                           interval, boundary, far, N, col, [&](int, F gy, F xt) {
+                                               const F xhat = (xt - m) * iv;
+                                               acc_gy += gy;
+                                               acc_gyx += gy * xhat;
+                                           });
             part_gy[col] = acc_gy;
             part_gyx[col] = acc_gyx;
         }
@@ -309,7 +322,10 @@ lif_bn_backward_partial_kernel(const F* __restrict__ x, const F* __restrict__ g,
 
 // Sweep 2: input gradient.  mean_gxhat[C], mean_gxhatx[C]: the per-channel means that sweep 1 and
 // the channel reduction produced (averaged over the ranks first when the batch is sharded).
-template <typename F, int TW, bool EXACT, bool SEGMENTED = false>
+// With TimeWalk::segments_memory the boundary potential of segment seg >= 1 is parked in row
+// seg*kSegment - 1 of gx, column of this lane: that row belongs to segment seg - 1, which this lane
+// writes only after it has consumed the value (segments are swept last to first).
+template <typename F, int TW, bool EXACT, TimeWalk WALK = TimeWalk::window>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
 lif_bn_backward_input_kernel(const F* __restrict__ x, const F* __restrict__ g,
                              const F* __restrict__ weight, const F* __restrict__ bias,
@@ -319,7 +335,7 @@ lif_bn_backward_input_kernel(const F* __restrict__ x, const F* __restrict__ g,
                              int64_t N, int64_t C, int64_t HW, F alpha, F thresh, F beta,
                              F interval) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
-    F* boundary = reinterpret_cast<F*>(lds_raw);  // used by SEGMENTED only
+    F* boundary = reinterpret_cast<F*>(lds_raw);  // used by TimeWalk::segments_lds only
     const bool small = N <= 0xffffffffll;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < N;
@@ -330,9 +346,9 @@ lif_bn_backward_input_kernel(const F* __restrict__ x, const F* __restrict__ g,
         const F scale = wgt * iv;
         const F b = bias[c];
         const F gxhat = mean_gxhat[c], gxhatx = mean_gxhatx[c];
-        bn_reverse<F, TW, EXACT, SEGMENTED>(
-            x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, boundary,
-            [&](int t, F gy, F xt) {
+        bn_reverse<F, TW, EXACT, WALK>(
+            x, g, T, N, col, m, scale, b, alpha, thresh, beta, interval, boundary, gx,
+            static_cast<int64_t>(kSegment) * N, col - N, [&](int t, F gy, F xt) {
                 Pack<F, 1> out;
                 out.e[0] = gy * wgt * iv - iv * ((xt - m) * iv * gxhatx + gxhat);
                 store_pack<F, 1>(gx + static_cast<int64_t>(t) * N + col, out);
@@ -341,58 +357,27 @@ lif_bn_backward_input_kernel(const F* __restrict__ x, const F* __restrict__ g,
 }
 
 // ---------------------------------------------------------------------------------------------
-// Per-channel reduction of the per-neuron partials.  Block (c, s) sums the batch entries
-// [s*bs, min(B, (s+1)*bs)) of channel c; lanes stride over the HW positions of one batch entry
-// (consecutive addresses), so the sum order is fixed by the geometry alone.
-// split = {gy[S][C], gyx[S][C]}.
+// Reduction of the per-neuron partials, a [B, CHW] matrix per quantity: workgroup (blockIdx.x,
+// blockIdx.y = s) adds up the batch entries [s*bs, min(B, (s+1)*bs)) of its kReduceBlock columns,
+// one column (channel, position) per lane -- consecutive lanes read consecutive addresses, and the
+// order of the sum is fixed by the geometry alone.  split = {gy[S][CHW], gyx[S][CHW]}.
 // ---------------------------------------------------------------------------------------------
 template <typename F>
 __global__ void __launch_bounds__(kReduceBlock)
-bn_channel_reduce_kernel(const F* __restrict__ part_gy, const F* __restrict__ part_gyx,
-                         F* __restrict__ split, int64_t B, int64_t C, int64_t HW, int64_t bs,
-                         int S) {
-    const int c = blockIdx.x;
+bn_column_reduce_kernel(const F* __restrict__ part_gy, const F* __restrict__ part_gyx,
+                        F* __restrict__ split, int64_t B, int64_t CHW, int64_t bs, int S) {
+    const int64_t j = static_cast<int64_t>(blockIdx.x) * kReduceBlock + threadIdx.x;
+    if (j >= CHW) return;
     const int s = blockIdx.y;
     const int64_t b0 = static_cast<int64_t>(s) * bs;
     const int64_t b1 = (b0 + bs < B) ? (b0 + bs) : B;
-    const int64_t CHW = C * HW;
     F a = F(0), ax = F(0);
-    if (HW >= kReduceBlock / 4) {
-        for (int64_t b = b0; b < b1; ++b) {
-            const int64_t base = b * CHW + static_cast<int64_t>(c) * HW;
-            for (int64_t i = threadIdx.x; i < HW; i += kReduceBlock) {
-                a += part_gy[base + i];
-                ax += part_gyx[base + i];
-            }
-        }
-    } else {  // few positions per channel (fully connected shapes): lanes stride over (b, hw) pairs
-        const int64_t n = (b1 - b0) * HW;
-        for (int64_t e = threadIdx.x; e < n; e += kReduceBlock) {
-            const int64_t b = b0 + e / HW, i = e % HW;
-            const int64_t at = b * CHW + static_cast<int64_t>(c) * HW + i;
-            a += part_gy[at];
-            ax += part_gyx[at];
-        }
+    for (int64_t b = b0; b < b1; ++b) {
+        a += part_gy[b * CHW + j];
+        ax += part_gyx[b * CHW + j];
     }
-    __shared__ F lds[2][kReduceBlock / 64];
-    a = wave_sum(a);
-    ax = wave_sum(ax);
-    const int wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-    if (lane == 0) {
-        lds[0][wave] = a;
-        lds[1][wave] = ax;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        F ta = F(0), tax = F(0);
-#pragma unroll
-        for (int w = 0; w < kReduceBlock / 64; ++w) {
-            ta += lds[0][w];
-            tax += lds[1][w];
-        }
-        split[static_cast<int64_t>(s) * C + c] = ta;
-        split[static_cast<int64_t>(S) * C + static_cast<int64_t>(s) * C + c] = tax;
-    }
+    split[static_cast<int64_t>(s) * CHW + j] = a;
+    split[(static_cast<int64_t>(S) + s) * CHW + j] = ax;
 }
 
 // Whole reduction of one channel in one workgroup, for partials that are few (the wave-summed
@@ -439,20 +424,23 @@ bn_channel_reduce_finalize_kernel(const F* __restrict__ part_gy,
     }
 }
 
-// One lane per channel: fold the S splits in order, emit the parameter gradients and the two
-// coefficients the input-gradient sweep needs.
+// One lane per channel: fold the S slices and the HW positions of the channel in order, emit the
+// parameter gradients and the two coefficients the input-gradient sweep needs.
 template <typename F>
 __global__ void __launch_bounds__(kReduceBlock)
 bn_channel_finalize_kernel(const F* __restrict__ split, const F* __restrict__ weight,
                            F* __restrict__ grad_weight, F* __restrict__ grad_bias,
                            F* __restrict__ mean_gxhat, F* __restrict__ mean_gxhatx,
-                           int64_t C, int S, F count) {
+                           int64_t C, int64_t HW, int S, F count) {
     const int64_t c = static_cast<int64_t>(blockIdx.x) * kReduceBlock + threadIdx.x;
     if (c >= C) return;
+    const int64_t CHW = C * HW;
     F a = F(0), ax = F(0);
     for (int s = 0; s < S; ++s) {
-        a += split[static_cast<int64_t>(s) * C + c];
-        ax += split[static_cast<int64_t>(S) * C + static_cast<int64_t>(s) * C + c];
+        for (int64_t i = 0; i < HW; ++i) {
+            a += split[static_cast<int64_t>(s) * CHW + c * HW + i];
+            ax += split[(static_cast<int64_t>(S) + s) * CHW + c * HW + i];
+        }
     }
     grad_bias[c] = a;
     grad_weight[c] = ax;

@@ -55,28 +55,31 @@ inline size_t bn_segment_lds_bytes(int64_t T, int threads) {
     return static_cast<size_t>((T + kSegment - 1) / kSegment) * threads * sizeof(F);
 }
 
-// Sweep 1 + channel reduction for windows of at most TW steps (SEGMENTED: of any length up to
-// SNNLIF_BP_NO_WORKSPACE_MAX_T, in segments of TW = kSegment steps): parameter gradients and the two
-// per-channel means the input-gradient sweep needs.
-template <typename F, int TW, bool SEGMENTED = false>
+// Sweep 1 + channel reduction for windows of at most TW steps (segmented walks: of any length, in
+// segments of TW = kSegment steps): parameter gradients and the two per-channel means the
+// input-gradient sweep needs.
+template <typename F, int TW, TimeWalk WALK = TimeWalk::window>
 int bn_backward_stats_window(const F* x, const F* weight, const F* bias, const F* ivar,
                              const F* mean, const F* g, F* grad_weight, F* grad_bias, F* mean_gxhat,
                              F* mean_gxhatx, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
                              float thresh, float beta, float interval, F* workspace,
                              hipStream_t stream) {
+    constexpr bool segmented = WALK != TimeWalk::window;
     const int64_t N = B * C * HW;
-    const int S = bn_reduce_splits(B, C);
+    const int S = bn_reduce_splits(B, C * HW);
     const size_t P = bn_partial_count(B, C, HW);
     F* part_gy = workspace;
     F* part_gyx = part_gy + P;
     F* split = part_gyx + P;
+    // boundary potentials of a window too long for LDS: the tail of the workspace, [segment][N]
+    F* far = workspace + bn_backward_workspace_elems(T, B, C, HW) - bn_boundary_elems(T, B, C, HW);
     const int threads =
         backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(F), kBnSmallBlock);
     const dim3 block(threads);
     const int Ti = static_cast<int>(T);
     constexpr bool can_be_inexact = TW > 8;
-    const bool exact = !SEGMENTED && (!can_be_inexact || (T == TW));
-    const size_t lds = SEGMENTED ? bn_segment_lds_bytes<F>(T, threads) : 0;
+    const bool exact = !segmented && (!can_be_inexact || (T == TW));
+    const size_t lds = WALK == TimeWalk::segments_lds ? bn_segment_lds_bytes<F>(T, threads) : 0;
 
     // Planes with few positions (fully connected shapes) would leave most lanes of a plane-aligned
     // wavefront idle; they keep one lane per neuron and per-neuron partials.
@@ -85,10 +88,10 @@ int bn_backward_stats_window(const F* x, const F* weight, const F* bias, const F
     const dim3 grid_partial(wave ? grid_for(B * C * G * 64, threads) : grid_for(N, threads));
     int rc;
 #define SNNLIF_BN_PARTIAL(EXACT_, WAVE_)                                                           \
-    launch_kernel(lif_bn_backward_partial_kernel<F, TW, EXACT_, WAVE_, SEGMENTED>, grid_partial,   \
-                  block, lds, stream, x, g, weight, bias, ivar, mean, part_gy, part_gyx, Ti, N, C, \
+    launch_kernel(lif_bn_backward_partial_kernel<F, TW, EXACT_, WAVE_, WALK>, grid_partial, block,  \
+                  lds, stream, x, g, weight, bias, ivar, mean, part_gy, part_gyx, far, Ti, N, C,  \
                   HW, F(alpha), F(thresh), F(beta), F(interval))
-    if constexpr (SEGMENTED) {
+    if constexpr (segmented) {
         if (wave) SNNLIF_BN_PARTIAL(false, true); else SNNLIF_BN_PARTIAL(false, false);
     } else if (exact) {
         if (wave) SNNLIF_BN_PARTIAL(true, true); else SNNLIF_BN_PARTIAL(true, false);
@@ -106,36 +109,39 @@ int bn_backward_stats_window(const F* x, const F* weight, const F* bias, const F
                       grad_bias, mean_gxhat, mean_gxhatx, B, C, G, count);
         return launch_status();
     }
+    const int64_t CHW = C * HW;
     const int64_t bs = (B + S - 1) / S;
-    launch_kernel(bn_channel_reduce_kernel<F>, dim3(static_cast<unsigned>(C), S),
-                  dim3(kReduceBlock), 0, stream, part_gy, part_gyx, split, B, C, HW, bs, S);
+    launch_kernel(bn_column_reduce_kernel<F>,
+                  dim3(static_cast<unsigned>((CHW + kReduceBlock - 1) / kReduceBlock), S),
+                  dim3(kReduceBlock), 0, stream, part_gy, part_gyx, split, B, CHW, bs, S);
     rc = launch_status();
     if (rc != SNNLIF_OK) return rc;
     launch_kernel(bn_channel_finalize_kernel<F>,
                   dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
                   dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias, mean_gxhat,
-                  mean_gxhatx, C, S, count);
+                  mean_gxhatx, C, HW, S, count);
     return launch_status();
 }
 
-// Sweep 2 for windows of at most TW steps (SEGMENTED: as above).
-template <typename F, int TW, bool SEGMENTED = false>
+// Sweep 2 for windows of at most TW steps (segmented walks: as above).
+template <typename F, int TW, TimeWalk WALK = TimeWalk::window>
 int bn_backward_input_window(const F* x, const F* weight, const F* bias, const F* ivar,
                              const F* mean, const F* g, const F* mean_gxhat, const F* mean_gxhatx,
                              F* gx, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
                              float thresh, float beta, float interval, hipStream_t stream) {
+    constexpr bool segmented = WALK != TimeWalk::window;
     const int64_t N = B * C * HW;
     const int threads =
         backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(F), kBnSmallBlock);
     const dim3 grid(grid_for(N, threads)), block(threads);
     const int Ti = static_cast<int>(T);
     constexpr bool can_be_inexact = TW > 8;
-    const bool exact = !SEGMENTED && (!can_be_inexact || (T == TW));
-    if constexpr (SEGMENTED) {
-        launch_kernel(lif_bn_backward_input_kernel<F, TW, false, true>, grid, block,
-                      bn_segment_lds_bytes<F>(T, threads), stream, x, g, weight, bias, ivar, mean,
-                      mean_gxhat, mean_gxhatx, gx, Ti, N, C, HW, F(alpha), F(thresh), F(beta),
-                      F(interval));
+    const bool exact = !segmented && (!can_be_inexact || (T == TW));
+    if constexpr (segmented) {
+        const size_t lds = WALK == TimeWalk::segments_lds ? bn_segment_lds_bytes<F>(T, threads) : 0;
+        launch_kernel(lif_bn_backward_input_kernel<F, TW, false, WALK>, grid, block, lds, stream, x, g,
+                      weight, bias, ivar, mean, mean_gxhat, mean_gxhatx, gx, Ti, N, C, HW, F(alpha),
+                      F(thresh), F(beta), F(interval));
     } else if (exact) {
         launch_kernel(lif_bn_backward_input_kernel<F, TW, true>, grid, block, 0, stream, x, g, weight,
                       bias, ivar, mean, mean_gxhat, mean_gxhatx, gx, Ti, N, C, HW, F(alpha),
@@ -163,12 +169,13 @@ int bn_backward_stats(const F* x, const F* weight, const F* bias, const F* ivar,
                                                alpha, thresh, beta, interval, workspace, stream);
     SNNLIF_BN_WINDOWS(SNNLIF_BN_WINDOW)
 #undef SNNLIF_BN_WINDOW
-    if (T <= SNNLIF_BP_NO_WORKSPACE_MAX_T)
-        return bn_backward_stats_window<F, kSegment, true>(x, weight, bias, ivar, mean, g,
-                                                           grad_weight, grad_bias, mean_gxhat,
-                                                           mean_gxhatx, T, B, C, HW, alpha, thresh,
-                                                           beta, interval, workspace, stream);
-    return SNNLIF_ERR_UNSUPPORTED;
+    if (T <= kBnLdsBoundaryMaxT)
+        return bn_backward_stats_window<F, kSegment, TimeWalk::segments_lds>(
+            x, weight, bias, ivar, mean, g, grad_weight, grad_bias, mean_gxhat, mean_gxhatx, T, B, C,
+            HW, alpha, thresh, beta, interval, workspace, stream);
+    return bn_backward_stats_window<F, kSegment, TimeWalk::segments_memory>(
+        x, weight, bias, ivar, mean, g, grad_weight, grad_bias, mean_gxhat, mean_gxhatx, T, B, C, HW,
+        alpha, thresh, beta, interval, workspace, stream);
 }
 
 template <typename F>
@@ -183,11 +190,13 @@ int bn_backward_input(const F* x, const F* weight, const F* bias, const F* ivar,
                                                interval, stream);
     SNNLIF_BN_WINDOWS(SNNLIF_BN_WINDOW)
 #undef SNNLIF_BN_WINDOW
-    if (T <= SNNLIF_BP_NO_WORKSPACE_MAX_T)
-        return bn_backward_input_window<F, kSegment, true>(x, weight, bias, ivar, mean, g, mean_gxhat,
-                                                           mean_gxhatx, gx, T, B, C, HW, alpha,
-                                                           thresh, beta, interval, stream);
-    return SNNLIF_ERR_UNSUPPORTED;
+    if (T <= kBnLdsBoundaryMaxT)
+        return bn_backward_input_window<F, kSegment, TimeWalk::segments_lds>(
+            x, weight, bias, ivar, mean, g, mean_gxhat, mean_gxhatx, gx, T, B, C, HW, alpha, thresh,
+            beta, interval, stream);
+    return bn_backward_input_window<F, kSegment, TimeWalk::segments_memory>(
+        x, weight, bias, ivar, mean, g, mean_gxhat, mean_gxhatx, gx, T, B, C, HW, alpha, thresh, beta,
+        interval, stream);
 }
 
 template <typename F>
@@ -195,8 +204,9 @@ int bn_backward(const F* x, const F* weight, const F* bias, const F* ivar, const
                 F* gx, F* grad_weight, F* grad_bias, int64_t T, int64_t B, int64_t C, int64_t HW,
                 float alpha, float thresh, float beta, float interval, F* workspace,
                 hipStream_t stream) {
-    // the two per-channel means live at the end of the workspace between the sweeps
-    F* coef = workspace + bn_backward_workspace_elems(B, C, HW) - 2 * C;
+    // the two per-channel means live behind the partial sums in the workspace between the sweeps
+    F* coef = workspace + bn_backward_workspace_elems(T, B, C, HW) - bn_boundary_elems(T, B, C, HW) -
+              2 * C;
     const int rc = bn_backward_stats<F>(x, weight, bias, ivar, mean, g, grad_weight, grad_bias, coef,
                                         coef + C, T, B, C, HW, alpha, thresh, beta, interval,
                                         workspace, stream);

@@ -66,6 +66,7 @@
 
 #include <cstddef>
 #include <cstdint>
+#include <tuple>
 #include <type_traits>
 
 #include "snnlib_lif.h"
@@ -664,16 +665,27 @@ struct KernelTimer {
 };
 extern thread_local KernelTimer tl_kernel_timer;  // defined in lif_abi.hip
 
-template <typename Kernel, typename... Args>
-inline void launch_kernel(Kernel kernel, dim3 grid, dim3 block, size_t lds_bytes,
+// Status of the most recent launch_kernel() of this thread (what the launch call itself returned,
+// not the runtime's sticky last-error slot, which an unrelated earlier call may have filled).
+extern thread_local hipError_t tl_launch_error;  // defined in lif_abi.hip
+
+// Launches `kernel` with `args` converted to its parameter types; a pending KernelTimer of this
+// thread is attached to the dispatch and consumed.
+template <typename... Params, typename... Args>
+inline void launch_kernel(void (*kernel)(Params...), dim3 grid, dim3 block, size_t lds_bytes,
                           hipStream_t stream, Args... args) {
-    KernelTimer timer = tl_kernel_timer;
+    static_assert(sizeof...(Params) == sizeof...(Args), "one argument per kernel parameter");
+    std::tuple<Params...> converted{static_cast<Params>(args)...};
+    void* slots[sizeof...(Params) > 0 ? sizeof...(Params) : 1];
+    std::apply([&](auto&... a) { int i = 0; ((slots[i++] = static_cast<void*>(&a)), ...); }, converted);
+    const KernelTimer timer = tl_kernel_timer;
     if (timer.start != nullptr || timer.stop != nullptr) {
         tl_kernel_timer = KernelTimer{};
-        hipExtLaunchKernelGGL(kernel, grid, block, static_cast<uint32_t>(lds_bytes), stream,
-                              timer.start, timer.stop, 0, args...);
+        tl_launch_error = hipExtLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, slots,
+                                             lds_bytes, stream, timer.start, timer.stop, 0);
     } else {
-        hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args...);
+        tl_launch_error = hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, slots,
+                                          lds_bytes, stream);
     }
 }
 
@@ -705,7 +717,7 @@ inline int pick_vec(int maxv, int64_t N, const void* const* ptrs, const size_t* 
 }
 
 inline int launch_status() {
-    return static_cast<int>(hipGetLastError());
+    return static_cast<int>(tl_launch_error);
 }
 
 // Calls f(std::integral_constant<int, v>) for the runtime vector width v in {MAXV, MAXV/2, .., 1}.

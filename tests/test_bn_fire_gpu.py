@@ -58,9 +58,13 @@ SHAPES = [
     (64, 2, 8, 4, 8),         # two full segments, plane-aligned wavefronts
     (70, 2, 5, 31),           # three segments, one lane per neuron
     (100, 3, 20),             # fully connected shape, four segments
-    (1024, 1, 4, 6, 6),       # the longest window: 32 segments of LDS boundary values
-    (8, 64, 1024),            # fully connected, many channels
-    (8, 32, 128, 32, 32),     # few channels, many positions: exercises the split reduction
+    (1024, 1, 4, 6, 6),       # the longest window with its boundary values in LDS: 32 segments
+    (1030, 1, 4, 6, 6),       # beyond it: boundary values in the workspace (sweep 1) and in gx rows (sweep 2)
+    (1100, 2, 20),            # the same, fully connected: one lane per neuron
+    (1057, 1, 3, 8, 8),       # 34 segments, the last of one step, plane-aligned wavefronts
+    (8, 64, 1024),            # fully connected, many channels: 64 batch slices of one entry each
+    (6, 200, 4, 3, 3),        # HW = 9, few channels, large batch: 64 batch slices of 4 entries, 9 positions per channel
+    (8, 32, 128, 32, 32),     # few channels, many positions: 16 wavefront partials per plane
 ]
 
 
@@ -167,6 +171,47 @@ def test_bn_fire_layer_like_reference_test(shape, dim_bn, train_bn):
         sf.alpha, sf.thresh, sf.beta, sf.interval = saved
 
 
+def test_bn_fire_layer_with_a_window_beyond_1024_steps():
+    """The layer accepts any window length in both directions (the reference's bn_fire_bp has no limit
+    either, snnlib/cuda/snn_kernel_bp.cu:680-750): forward and backward of a 1030-step window against
+    autograd through batch_norm + the gold fire loop."""
+    from oracle import gold_fire
+    from snn_gpu_training_bptt_amd import snnlib_func as sf
+    from snn_gpu_training_bptt_amd import snnlib_op as sop
+    saved = (sf.alpha, sf.thresh, sf.beta, sf.interval)
+    sf.alpha, sf.thresh, sf.beta, sf.interval = ALPHA, THRESH, BETA, INTERVAL
+    try:
+        shape, C = (1030, 2, 4, 3), 4
+
+        def draw(seed):
+            torch.manual_seed(seed)
+            return torch.randn(shape), torch.rand(C) + 0.5, torch.randn(C) * 0.2, torch.randn(shape)
+
+        def potentials(seed):
+            x_, w_, b_, _ = (t.cuda() for t in draw(seed))
+            with torch.no_grad():
+                return gold_fire.gold_bn_fire(x_, w_, b_, None, None, True, EPS, ALPHA, THRESH, BETA, INTERVAL)[0]
+
+        x0, w0, b0, g0 = draw(seed_clear_of_decision_points(potentials, range(37, 4037, 100)))
+        layer = sop.BnFire(C, (0, 1, 3), EPS).cuda()
+        with torch.no_grad():
+            layer.weight_bn.copy_(w0)
+            layer.bias_bn.copy_(b0)
+        x = x0.cuda().requires_grad_(True)
+        spikes = layer(x)
+        spikes.backward(g0.cuda())
+        xr = x0.cuda().requires_grad_(True)
+        wr, br = w0.cuda().requires_grad_(True), b0.cuda().requires_grad_(True)
+        _, s_ref = gold_fire.gold_bn_fire(xr, wr, br, None, None, True, EPS, ALPHA, THRESH, BETA, INTERVAL)
+        s_ref.backward(g0.cuda())
+        assert torch.equal(spikes, s_ref), "spikes differ from the gold layer"
+        for got, want, what in ((x.grad, xr.grad, "input"), (layer.weight_bn.grad, wr.grad, "weight"),
+                                (layer.bias_bn.grad, br.grad, "bias")):
+            rel_close(got.cpu().numpy(), want.cpu().numpy(), what + " gradient", tol=5e-5)
+    finally:
+        sf.alpha, sf.thresh, sf.beta, sf.interval = saved
+
+
 def test_bn_fire_errors(cabi):
     import snnlib
     x = torch.zeros(4, 2, 8, device="cuda")
@@ -178,11 +223,10 @@ def test_bn_fire_errors(cabi):
     with pytest.raises(RuntimeError, match="per channel"):
         snnlib.bn_fire_s_fp(x, p[:4], p, p, p, EPS, ALPHA, THRESH)
     lib = cabi.load()
-    big = torch.zeros(1025, 2, 8, device="cuda")      # longer than the segmented backward reaches
-    rc = lib.snnlif_bn_fire_bp(big.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), big.data_ptr(),
-                               big.data_ptr(), p.data_ptr(), p.data_ptr(), 0, 1025, 2, 8, 1, ALPHA, THRESH, BETA, INTERVAL,
-                               None, 0, None)
-    assert rc == cabi.ERR_UNSUPPORTED
+    # windows beyond 1024 steps also keep their segment boundaries in the workspace
+    f32 = cabi.DTYPE_F32
+    assert (cabi.bn_fire_bp_workspace_bytes(f32, 1025, 2, 8, 1) - cabi.bn_fire_bp_workspace_bytes(f32, 1024, 2, 8, 1)
+            == 4 * 33 * 16)
     rc = lib.snnlif_bn_fire_bp(x.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), p.data_ptr(), x.data_ptr(),
                                x.data_ptr(), p.data_ptr(), p.data_ptr(), 0, 4, 2, 8, 1, ALPHA, THRESH, BETA, INTERVAL,
                                None, 0, None)

@@ -304,9 +304,11 @@ def test_batch_norm_workspace_follows_the_partial_sum_layout():
     assert need(f32, 8, 4, 6, 49) == 4 * (2 * 4 * 6 * 1 + 2 * 6)
     assert need(f32, 8, 4, 6, 65) == 4 * (2 * 4 * 6 * 2 + 2 * 6)
     assert need(f64, 8, 4, 6, 65) == 2 * need(f32, 8, 4, 6, 65)
-    # 31 positions: one lane per neuron; S = min(B, 2048 / C) splits of the batch axis
-    assert need(f32, 8, 4, 6, 31) == 4 * (2 * 4 * 6 * 31 + 2 * 4 * 6 + 2 * 6)
-    assert need(f32, 8, 64, 1024, 1) == 4 * (2 * 64 * 1024 + 2 * 2 * 1024 + 2 * 1024)
+    # 31 positions: one lane per neuron; the [B, C*HW] partials are summed in S = min(B, 64, ...) batch slices
+    assert need(f32, 8, 4, 6, 31) == 4 * (2 * 4 * 6 * 31 + 2 * 4 * 6 * 31 + 2 * 6)
+    assert need(f32, 8, 64, 1024, 1) == 4 * (2 * 64 * 1024 + 2 * 64 * 1024 + 2 * 1024)
+    # beyond 1024 steps: one boundary potential per 32-step segment and neuron on top
+    assert need(f32, 1025, 4, 6, 65) == need(f32, 8, 4, 6, 65) + 4 * 33 * 4 * 6 * 65
     assert need(f32, 0, 4, 6, 31) == 0 and need(lif_cabi.DTYPE_BF16, 8, 4, 6, 31) == 0
 
 

@@ -162,6 +162,59 @@ def test_events_attached_to_the_next_kernel(cabi):
     assert np.array_equal(spike.cpu().numpy(), spike_o)
 
 
+def test_an_armed_timer_does_not_outlive_a_failed_call(cabi):
+    """An entry point that returns an argument error consumes the arming: the events must not end up
+    on the next, unrelated launch."""
+    lib = cabi.load()
+    x = (0.5 + torch.randn(8, 8, 64, 32, 32)).cuda()
+    spike = torch.empty_like(x)
+    k0, k1, after = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+    k0.record()
+    k1.record()
+    torch.cuda.synchronize()
+    cabi.time_next_kernel(k0, k1)
+    assert lib.snnlif_fire_s_fp(x.data_ptr(), spike.data_ptr(), 9, 8, x.numel() // 8, ALPHA, THRESH, None) == cabi.ERR_DTYPE
+    for _ in range(3):                                   # were the timer still armed, k1 would now be
+        cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)     # re-recorded at the end of the first of these
+    after.record()
+    torch.cuda.synchronize()
+    first_kernel_end_to_after = k1.elapsed_time(after)
+    cabi.time_next_kernel(k0, k1)
+    cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+    torch.cuda.synchronize()
+    one_kernel = k0.elapsed_time(k1)
+    # k1 kept its original record (before all three launches): all three lie between it and `after`
+    assert first_kernel_end_to_after > 2.5 * one_kernel, (first_kernel_end_to_after, one_kernel)
+
+
+def test_events_bracket_the_whole_of_a_multi_kernel_operation(cabi):
+    """The batch-norm backward is three kernels: the armed events are recorded before the first and
+    after the last, so they cover at least the two sweeps."""
+    shape = (8, 16, 32, 32, 32)
+    T, B, C, HW = 8, 16, 32, 1024
+    x = (0.5 + torch.randn(shape)).cuda()
+    g = torch.randn(shape).cuda()
+    w, b = torch.ones(C, device="cuda"), torch.zeros(C, device="cuda")
+    var, mean = torch.ones(C, device="cuda"), torch.full((C,), 0.5, device="cuda")
+    ivar, spike = torch.empty_like(var), torch.empty_like(x)
+    cabi.bn_fire_s_fp_into(x, w, b, var, mean, ivar, spike, 1e-5, ALPHA, THRESH)
+    gx, gw, gb = torch.empty_like(x), torch.empty_like(w), torch.empty_like(w)
+    ws = torch.empty(cabi.bn_fire_bp_workspace_bytes(cabi.DTYPE_F32, T, B, C, HW), dtype=torch.uint8, device="cuda")
+    e = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+    for ev in e:
+        ev.record()
+    torch.cuda.synchronize()
+    for _ in range(2):
+        cabi.bn_fire_bp_into(x, w, b, ivar, mean, g, gx, gw, gb, ALPHA, THRESH, BETA, INTERVAL, ws)
+    cabi.time_next_kernel(e[0], e[1])
+    cabi.bn_fire_bp_into(x, w, b, ivar, mean, g, gx, gw, gb, ALPHA, THRESH, BETA, INTERVAL, ws)
+    cabi.time_next_kernel(e[2], e[3])
+    cabi.bn_fire_bp_dist2_into(x, w, b, ivar, mean, g, gw, gb, gx, ALPHA, THRESH, BETA, INTERVAL)   # one sweep
+    torch.cuda.synchronize()
+    whole, one_sweep = e[0].elapsed_time(e[1]), e[2].elapsed_time(e[3])
+    assert whole > 1.4 * one_sweep, (whole, one_sweep)
+
+
 def test_layers_captured_with_torch_cuda_graph():
     """A forward + backward through the PyTorch-facing layers (Fire, then BnFire with given statistics,
     whose backward draws its workspace from the caching allocator) captured by torch.cuda.graph and

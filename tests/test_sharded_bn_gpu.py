@@ -63,7 +63,7 @@ def dims_of(shape):
 
 
 SHAPES = [(6, 4, 8), (6, 4, 8, 8, 8), (8, 6, 32, 16, 16), (4, 6, 7, 7, 7), (13, 2, 20, 5, 3), (8, 16, 1024),
-          (40, 2, 6, 8, 8)]
+          (40, 2, 6, 8, 8), (1030, 2, 4, 6, 6), (1100, 2, 12)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
@@ -133,7 +133,7 @@ def test_argument_checks_of_the_halves(cabi):
     assert lib.snnlif_bn_fire_bp_dist1(*[None] * 10, f32, 0, 2, 3, 4, 0.25, 0.5, 1.0, 0.5, None, 0, None) == cabi.OK
     assert lib.snnlif_bn_fire_bp_dist1(*[None] * 10, f32, 4, 2, 3, 4, 0.25, 0.5, 1.0, 0.5, None, 0, None) == cabi.ERR_ARG
     assert lib.snnlif_bn_fire_bp_dist2(*[None] * 9, f32, 4, 2, 3, 4, 0.25, 0.5, 1.0, 0.5, None) == cabi.ERR_ARG
-    assert lib.snnlif_bn_fire_bp_dist2(*[None] * 9, f32, 1025, 2, 3, 4, 0.25, 0.5, 1.0, 0.5, None) == cabi.ERR_UNSUPPORTED
+    assert lib.snnlif_bn_fire_bp_dist2(*[None] * 9, f32, 1025, 2, 3, 4, 0.25, 0.5, 1.0, 0.5, None) == cabi.ERR_ARG
     assert lib.snnlif_bn_fire_bp_dist2(*[None] * 9, cabi.DTYPE_BF16, 4, 2, 3, 4, 0.25, 0.5, 1.0, 0.5, None) == cabi.ERR_UNSUPPORTED
     x, g, w, b, var, mean = make((4, 2, 3, 2, 2), seed=44)
     out = [torch.empty_like(w) for _ in range(4)]

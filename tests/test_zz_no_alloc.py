@@ -57,6 +57,7 @@ SEQUENCES = [
     [(6, 32, 64), (3, 8, 16)],                       # fully connected: one partial per neuron
     [(8, 8, 16, 7, 7), (5, 2, 9, 31), (6, 2, 8)],    # switches between the two layouts
     [(40, 4, 8, 8, 8), (33, 2, 6, 4, 4)],            # segmented windows
+    [(1030, 2, 4, 8, 8), (1025, 1, 6)],              # boundary potentials in the array as well
 ]
 
 
