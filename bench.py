@@ -70,8 +70,12 @@ WORKLOADS = {
 # "hot": the kernel of the step loop (SNNLIF_KEEP_SPATIAL), "cold": the streamed kernel of the cold leg.
 # bn_fire: the three backward kernels together.
 MEASURED_TRAFFIC = {
-    "cfg2": {"hot": 805276475, "cold": None, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt"},
-    "bn_fire": {"hot": 1346500000, "cold": None, "source": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt"},
+    "cfg2": {"hot": 805278669, "cold": 805276863, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt"},
+    "cfg3": {"hot": 805324121, "cold": 805325140, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg3_f32.txt"},
+    "cfg5": {"hot": 3221228509, "cold": 3221196043, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_f32.txt"},
+    "cfg5_bf16": {"hot": 1610664262, "cold": 1610660298,
+                  "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_bf16.txt"},
+    "bn_fire": {"hot": 1346471139, "cold": None, "source": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt"},
 }
 HEADLINE = "cfg2"
 METRIC = "LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T=8,B=64,C=128,32x32"
@@ -335,6 +339,13 @@ def run_bn_fire(args):
         stats()
         fwd()
         bwd()
+    if args.copy_calibration:      # plain device copies of known size, to scale PMC readings by
+        torch.cuda.synchronize()
+        scratch_copy = torch.empty_like(x)
+        for _ in range(3):
+            scratch_copy.copy_(x)
+        torch.cuda.synchronize()
+        del scratch_copy
     # a step is what the layer does in training: batch statistics, forward, backward.  The statistics
     # and the backward are several kernels each: stream markers around each pass (dispatch gaps included)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]

@@ -51,15 +51,18 @@ class SnnlifError(RuntimeError):
 
 
 def load():
-    """Load the library once and type its entry points.  Raises if it has not been built."""
+    """Load the library once and type its entry points.  Raises if it has not been built.
+    ``SNNLIF_LIBRARY`` in the environment names another build of the same library to load instead of
+    the in-tree one (e.g. one compiled with different tuning macros, for A/B measurements)."""
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
+    path = os.environ.get("SNNLIF_LIBRARY") or LIB_PATH
+    if not os.path.exists(path):
         raise ImportError(
-            f"{LIB_PATH} is missing: build it with `python -m snn_gpu_training_bptt_amd.build` "
+            f"{path} is missing: build it with `python -m snn_gpu_training_bptt_amd.build` "
             "(there is no CPU or PyTorch fallback for the LIF fire kernels)")
-    lib = ctypes.CDLL(LIB_PATH)
+    lib = ctypes.CDLL(path)
     for name, (restype, argtypes) in SYMBOLS.items():
         fn = getattr(lib, name)
         fn.restype = restype
