@@ -386,6 +386,49 @@ def run_bn_fire(args):
                                "achieved": 4 * ns / (stats_ms * 1e-3) / 1e9,
                                "frac": 4 * ns / (stats_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
     }
+    if not args.no_cold_leg:
+        # the layer with nothing cached between its forward and its backward: four tensor sets, all
+        # (statistics + forward), then all backwards; events bracket each operation (for the
+        # statistics and the backward: all of their kernels, dispatch gaps included)
+        sets, rounds = 4, 5
+        xs = [x] + [x.clone() for _ in range(sets - 1)]
+        gs = [g] + [g.clone() for _ in range(sets - 1)]
+        spikes = [torch.empty_like(x) for _ in range(sets)]
+        gxs = [torch.empty_like(x) for _ in range(sets)]
+        cev = [[[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(sets)] for _ in range(rounds + 1)]
+        for per_round in cev:
+            for per_set in per_round:
+                for e in per_set:
+                    e.record()
+        torch.cuda.synchronize()
+        for r in range(rounds + 1):
+            for k in range(sets):
+                e = cev[r][k]
+                lif_cabi.time_next_kernel(e[0], e[1])
+                lif_cabi.bn_stats_into(xs[k], mean, var, stats_ws)
+                lif_cabi.time_next_kernel(e[2], e[3])
+                lif_cabi.bn_fire_s_fp_into(xs[k], weight, bias, var, mean, ivar, spikes[k], eps, ALPHA, THRESH)
+            for k in range(sets):
+                e = cev[r][k]
+                lif_cabi.time_next_kernel(e[4], e[5])
+                lif_cabi.bn_fire_bp_into(xs[k], weight, bias, ivar, mean, gs[k], gxs[k], gw, gb, ALPHA, THRESH, BETA,
+                                         INTERVAL, ws)
+        torch.cuda.synchronize()
+        timed = [e for per_round in cev[1:] for e in per_round]
+        avg = lambda a, b: sum(e[a].elapsed_time(e[b]) for e in timed) / len(timed)
+        cs, cf, cb = avg(0, 1), avg(2, 3), avg(4, 5)
+        rate = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+        result["roofline"]["cold"] = {
+            "what": f"{sets} independent tensor sets, all (statistics + forward) then all backwards, {rounds} timed "
+                    "rounds after one untimed; events bracket each operation",
+            "stats": {"avg_ms": cs, "achieved": rate(4 * ns, cs), "frac": rate(4 * ns, cs) / HBM_PEAK_GBPS},
+            "fwd": {"avg_ms": cf, "achieved": rate(8 * ns, cf), "frac": rate(8 * ns, cf) / HBM_PEAK_GBPS},
+            "bwd": {"avg_ms": cb, "achieved": rate(20 * ns, cb), "frac": rate(20 * ns, cb) / HBM_PEAK_GBPS},
+            "outputs_equal_across_sets": bool(all(torch.equal(sp, spikes[0]) for sp in spikes[1:])
+                                              and all(torch.equal(q, gxs[0]) for q in gxs[1:])),
+        }
+        del xs, gs, spikes, gxs
+
     if not args.no_cpu_baseline:
         # CPU leg: the scalar C loops of the oracle on a bounded sample (channels are independent given
         # their statistics; the backward's means are those of the sample), one host thread.  Its
