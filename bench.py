@@ -62,6 +62,9 @@ WORKLOADS = {
     "cfg3": ((32, 32, 256, 16, 16), 0.3, 0.8, "float32"),
     "cfg5": ((16, 128, 512, 16, 16), 0.5, 1.0, "float32"),
     "cfg5_bf16": ((16, 128, 512, 16, 16), 0.5, 1.0, "bfloat16"),
+    # no configuration of the reference: a 96-step window, the longest range of the backward that
+    # still recomputes the whole window in registers (67 239 936 neuron-steps, 257 MiB per tensor)
+    "t96": ((96, 4, 171, 32, 32), 0.5, 1.0, "float32"),
 }
 # HBM bytes per launch of the backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
 # of this file (each counter scaled by its reading for a plain device copy of the same tensor:
@@ -75,6 +78,7 @@ MEASURED_TRAFFIC = {
     "cfg5": {"hot": 3221228509, "cold": 3221196043, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_f32.txt"},
     "cfg5_bf16": {"hot": 1610664262, "cold": 1610660298,
                   "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_bf16.txt"},
+    "t96": {"hot": 807059743, "cold": 807058710, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_t96_f32.txt"},
     "bn_fire": {"hot": 1346471139, "cold": None, "source": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt"},
 }
 HEADLINE = "cfg2"

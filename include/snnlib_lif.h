@@ -72,7 +72,7 @@ extern "C" {
 #define SNNLIF_ERR_UNSUPPORTED -5 /* valid arguments this entry point does not implement (bf16 in the batch-norm ones) */
 
 /* Every T up to this keeps the whole recomputed membrane potential in registers in the backward
- * (one kernel, 12 bytes per neuron-step in fp32); so do T = 40, 48, 56 and 64 exactly. */
+ * (one kernel, 12 bytes per neuron-step in fp32); so do multiples of 8 steps up to 104 (64 in fp64). */
 #define SNNLIF_BP_FUSED_MAX_T 32
 /* Largest T for which snnlif_fire_bp needs no workspace: up to here longer windows are processed
  * in register-sized segments whose boundary potentials live in LDS (16 bytes per neuron-step). */

@@ -53,7 +53,7 @@
 //     element-wise CPU/GPU ops do, which makes spikes, potentials and gradients bit-identical to
 //     the per-op rounded reference arithmetic.
 //
-// Windows of exactly 40, 48, 56 or 64 steps still run as one register window.  Other longer windows
+// Windows of a multiple of 8 steps up to 104 (64 with fp64 arithmetic) still run as one register window.  Other longer windows
 // (32 < T <= 1024) are cut into 32-step segments: one forward pass leaves the
 // membrane potential at the segment boundaries in LDS, then each segment is recomputed into registers
 // and swept in reverse, last segment first (x is read twice, nothing else changes).  Beyond that the
@@ -97,6 +97,14 @@
 // VGPR budget (in 32-bit words) the fused backward may spend on the recomputed membrane potential.
 #ifndef SNNLIF_FUSED_U_WORDS
 #define SNNLIF_FUSED_U_WORDS 128
+#endif
+// Longest window run as one register window when its length is a multiple of 8 steps: with 4-byte
+// arithmetic, and with 8-byte arithmetic (two VGPRs per potential).
+#ifndef SNNLIF_BWD_WIDE_MAX_T
+#define SNNLIF_BWD_WIDE_MAX_T 104
+#endif
+#ifndef SNNLIF_BWD_WIDE_MAX_T_F64
+#define SNNLIF_BWD_WIDE_MAX_T_F64 64
 #endif
 // Column order of the fused backward: 1 = workgroups walk the neuron axis from its end, i.e.
 // opposite to the forward (the cached tail of x is consumed before it can be displaced).
@@ -148,6 +156,7 @@ constexpr int backward_waves(int rows, bool keep = true) {
 #ifdef SNNLIF_BWD_MAX_WAVES
     return SNNLIF_BWD_MAX_WAVES;
 #else
+    if (rows > 64) return 3;  // u alone takes `rows` VGPRs per lane
     if (!keep) return rows <= 8 ? SNNLIF_STREAM_BWD_WAVES_SHORT : SNNLIF_STREAM_BWD_WAVES_LONG;
     return rows <= 8 ? 8 : (rows <= 12 ? 5 : 4);
 #endif
@@ -936,17 +945,30 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
 #undef SNNLIF_BWD_WINDOW
     static_assert(SNNLIF_BP_FUSED_MAX_T == 32, "windows above must cover the fused range");
 
-    // A few longer windows still fit the register file whole (u alone takes T VGPRs per lane) and
-    // then move 12 bytes per neuron-step instead of the segmented kernel's 16 -- but only in
-    // straight-line form: zero-filling a 48-row window for T = 33 is slower than two segments.
+    // Windows of a multiple of 8 steps still fit the register file whole a good way further (u alone
+    // takes T VGPRs per lane with 4-byte arithmetic: 4 wavefronts per SIMD up to 64 steps, 3 up to
+    // 104; at 128 steps a single wavefront is left and the kernel collapses to a fifth of the
+    // segmented kernel's rate).  They move 12 bytes per neuron-step where the segmented kernel
+    // re-reads x; cold-cache backward at 64 Mi elements, fp32: 67-72 % of the HBM peak against
+    // 54-65 %.  Only the exact length qualifies: the zero-filled form of these wide windows runs at
+    // 40-58 %, below the segmented kernel.
+    constexpr int64_t wide_max =
+        sizeof(C) == 4 ? SNNLIF_BWD_WIDE_MAX_T : SNNLIF_BWD_WIDE_MAX_T_F64;
 #define SNNLIF_BWD_WIDE_WINDOW(TW)                                                               \
-    if (T == TW)                                                                                 \
+    if (TW <= wide_max && T == TW)                                                               \
         return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, keep_x, \
                                             stream);
     SNNLIF_BWD_WIDE_WINDOW(40)
     SNNLIF_BWD_WIDE_WINDOW(48)
     SNNLIF_BWD_WIDE_WINDOW(56)
     SNNLIF_BWD_WIDE_WINDOW(64)
+    if constexpr (sizeof(C) == 4) {
+        SNNLIF_BWD_WIDE_WINDOW(72)
+        SNNLIF_BWD_WIDE_WINDOW(80)
+        SNNLIF_BWD_WIDE_WINDOW(88)
+        SNNLIF_BWD_WIDE_WINDOW(96)
+        SNNLIF_BWD_WIDE_WINDOW(104)
+    }
 #undef SNNLIF_BWD_WIDE_WINDOW
 
     // Longer windows, up to what the boundary values of a workgroup fit into 64 KiB of LDS for

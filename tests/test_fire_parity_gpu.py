@@ -125,6 +125,31 @@ def test_windows_between_32_and_64(cabi, oracle, T, dtype):
         assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3), alpha=0.3)
 
 
+@HINTS
+@pytest.mark.parametrize("T,dtype", [(72, torch.float32), (80, torch.float32), (88, torch.float32),
+                                     (96, torch.float32), (104, torch.float32), (95, torch.float32),
+                                     (97, torch.float32), (112, torch.float32), (128, torch.float32),
+                                     (72, torch.float64), (96, torch.float64),
+                                     (40, torch.bfloat16), (64, torch.bfloat16), (72, torch.bfloat16),
+                                     (96, torch.bfloat16), (104, torch.bfloat16), (100, torch.bfloat16)])
+def test_windows_between_64_and_128(cabi, oracle, T, dtype, keep):
+    """With 4-byte arithmetic (fp32 and bf16 storage) windows of 72, 80, 88, 96 and 104 steps still
+    run as one register window; their neighbours, longer multiples of 8 and every fp64 window beyond
+    64 steps run in segments.  Even N (bf16 pairs where the register budget allows) and odd N."""
+    for n_inner in (256, 77):
+        x32, g32 = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=4000 + T)
+        x, g = x32.to(dtype), g32.to(dtype)
+        outs = run_gpu(cabi, x, g, alpha=0.3, keep=keep)
+        if dtype == torch.bfloat16:
+            mem, spike_a, spike_b, gx = outs
+            mem_o, spike_o = oracle.fire_forward(x.float().numpy(), 0.3, THRESH)
+            gx_o = oracle.fire_backward(x.float().numpy(), g.float().numpy(), 0.3, THRESH, BETA, INTERVAL)
+            assert np.array_equal(spike_a.float().numpy(), spike_o)
+            assert torch.equal(gx, torch.from_numpy(gx_o).bfloat16())
+        else:
+            assert_parity(oracle, x, g, outs, alpha=0.3)
+
+
 @pytest.mark.parametrize("T", [1, 2])
 @pytest.mark.parametrize("n_inner", [4096, 4098, 4097, 8])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
