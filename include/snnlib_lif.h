@@ -155,6 +155,25 @@ int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spati
                    int64_t T, int64_t N, float alpha, float thresh, float beta, float interval,
                    void* workspace, size_t workspace_bytes, void* stream);
 
+/*
+ * snnlif_fire_bp for a gradient whose time rows are `grad_row_stride` elements apart instead of N:
+ *   grad_row_stride == N  the dense [T,N] gradient (exactly snnlif_fire_bp);
+ *   grad_row_stride == 0  one row of N values that stands for every time step: what autograd hands to
+ *                         the fire op after `spike.mean(dim=0)` or `spike.sum(dim=0)` (a stride-0
+ *                         expansion over time; the pattern of the reference's own snnlib/test_fire.py:22-30).
+ *                         The reference's binding makes such a gradient dense first
+ *                         (snnlib/cuda/snn.cpp:270-279 requires contiguous inputs); here it is read in
+ *                         place, N values instead of T*N;
+ *   grad_row_stride >  N  rows of a wider tensor.
+ * Any other value (negative, or 0 < stride < N: overlapping rows) is SNNLIF_ERR_ARG.  `grad_spatial` is
+ * dense and must not overlap `grad_spike`.  Everything else as snnlif_fire_bp; same results bit for bit
+ * as snnlif_fire_bp on the gradient made dense.
+ */
+int snnlif_fire_bp_strided(const void* spatial, const void* grad_spike, void* grad_spatial, int dtype,
+                           int64_t T, int64_t N, int64_t grad_row_stride, float alpha, float thresh,
+                           float beta, float interval, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
 /* Bytes of device workspace snnlif_bn_stats needs (partial sums: two of the storage type per wavefront
  * when HW >= 32, two per (row slice, channel position) otherwise).  0 for invalid arguments. */
 size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);

@@ -163,11 +163,22 @@ size_t snnlif_fire_bp_workspace_bytes(int dtype, int64_t T, int64_t N) {
 int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spatial, int dtype,
                    int64_t T, int64_t N, float alpha, float thresh, float beta, float interval,
                    void* workspace, size_t workspace_bytes, void* stream) {
+    return snnlif_fire_bp_strided(spatial, grad_spike, grad_spatial, dtype, T, N, N, alpha, thresh, beta,
+                                  interval, workspace, workspace_bytes, stream);
+}
+
+int snnlif_fire_bp_strided(const void* spatial, const void* grad_spike, void* grad_spatial, int dtype,
+                           int64_t T, int64_t N, int64_t grad_row_stride, float alpha, float thresh,
+                           float beta, float interval, void* workspace, size_t workspace_bytes,
+                           void* stream) {
     const TimerScope timer_scope;
     if (arith_size(dtype) == 0) return SNNLIF_ERR_DTYPE;
     const int se = shape_error(T, N);
     if (se != SNNLIF_OK) return se;
+    const int64_t GN = grad_row_stride;
+    if (GN < 0 || (GN != 0 && GN < N)) return SNNLIF_ERR_ARG;
     if (T == 0 || N == 0) return SNNLIF_OK;
+    if (GN > 0 && (T - 1) > (INT64_MAX / 16 - N) / GN) return SNNLIF_ERR_ARG;  // byte offsets stay in int64
     if (spatial == nullptr || grad_spike == nullptr || grad_spatial == nullptr) return SNNLIF_ERR_ARG;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const snnlif::SpatialHint keep = hint_of(dtype);
@@ -176,11 +187,11 @@ int snnlif_fire_bp(const void* spatial, const void* grad_spike, void* grad_spati
     const OperationTimer whole_operation(st, two_kernels);
     switch (storage_of(dtype)) {
         case SNNLIF_DTYPE_F32:
-            return snnlif::backward_f32(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
+            return snnlif::backward_f32(spatial, grad_spike, grad_spatial, T, N, GN, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
         case SNNLIF_DTYPE_F64:
-            return snnlif::backward_f64(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
+            return snnlif::backward_f64(spatial, grad_spike, grad_spatial, T, N, GN, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
         default:
-            return snnlif::backward_bf16(spatial, grad_spike, grad_spatial, T, N, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
+            return snnlif::backward_bf16(spatial, grad_spike, grad_spatial, T, N, GN, alpha, thresh, beta, interval, keep, workspace, workspace_bytes, st);
     }
 }
 

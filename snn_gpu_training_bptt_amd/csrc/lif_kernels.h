@@ -385,7 +385,8 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 
 // ---------------------------------------------------------------------------------------------
 // One register-resident backward window of at most TW rows, for the neuron(s) at column `col`.
-// Row pointers x, g, gx are those of the window's first row.  On entry uc / sc hold the membrane
+// Row pointers x, g, gx are those of the window's first row; rows of x and gx are N elements apart,
+// rows of g GN elements (GN == N: a dense gradient; GN == 0: one row that stands for every step).  On entry uc / sc hold the membrane
 // potential and spike of the step before the window (zeros at t = 0) and gu the gradient carried
 // in from the step after it (zero at the end of time); on exit gu is the gradient of the window's
 // first step, ready for the window before.
@@ -399,7 +400,8 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 template <typename S, int V, int TW, bool EXACT, bool KEEP = true>
 __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S* __restrict__ g,
                                                 S* __restrict__ gx, int rows, int64_t N,
-                                                int64_t col, typename Arith<S>::type (&uc)[V],
+                                                int64_t GN, int64_t col,
+                                                typename Arith<S>::type (&uc)[V],
                                                 typename Arith<S>::type (&sc)[V],
                                                 typename Arith<S>::type (&gu)[V],
                                                 typename Arith<S>::type alpha,
@@ -427,10 +429,10 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
     for (int t = TW - 1; t >= ((TW - GC) > 0 ? (TW - GC) : 0); --t) {
         const int k = t - ((TW - GC) > 0 ? (TW - GC) : 0);
         if (EXACT) {
-            gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+            gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * GN + col);
         } else {
             gbuf[0][k] = zero_pack<S, V>();
-            if (t < rows) gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+            if (t < rows) gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * GN + col);
         }
     }
 
@@ -455,12 +457,12 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
             for (int t = nhi - 1; t >= nlo; --t) {
                 if (EXACT) {
                     gbuf[(q + 1) & 1][t - nlo] =
-                        load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+                        load_pack<S, V, true>(g + static_cast<int64_t>(t) * GN + col);
                 } else {
                     gbuf[(q + 1) & 1][t - nlo] = zero_pack<S, V>();
                     if (t < rows)
                         gbuf[(q + 1) & 1][t - nlo] =
-                            load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+                            load_pack<S, V, true>(g + static_cast<int64_t>(t) * GN + col);
                 }
             }
         }
@@ -495,9 +497,9 @@ __device__ __forceinline__ int64_t backward_column(int64_t v, int64_t nvec, int 
 template <typename S, int V, int TW, bool EXACT, bool KEEP>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW, KEEP))
 lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
-                          int T, int64_t N, int64_t nvec, typename Arith<S>::type alpha,
-                          typename Arith<S>::type thresh, typename Arith<S>::type beta,
-                          typename Arith<S>::type interval) {
+                          int T, int64_t N, int64_t GN, int64_t nvec,
+                          typename Arith<S>::type alpha, typename Arith<S>::type thresh,
+                          typename Arith<S>::type beta, typename Arith<S>::type interval) {
     using C = typename Arith<S>::type;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < nvec;
@@ -510,8 +512,8 @@ lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* _
             sc[j] = C(0);
             gu[j] = C(0);
         }
-        backward_window<S, V, TW, EXACT, KEEP>(x, g, gx, T, N, col, uc, sc, gu, alpha, thresh, beta,
-                                               interval);
+        backward_window<S, V, TW, EXACT, KEEP>(x, g, gx, T, N, GN, col, uc, sc, gu, alpha, thresh,
+                                               beta, interval);
     }
 }
 
@@ -531,7 +533,7 @@ constexpr int kSegment = 32;
 template <typename S, int V>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(kSegment))
 lif_backward_segmented_kernel(const S* __restrict__ x, const S* __restrict__ g,
-                              S* __restrict__ gx, int T, int64_t N, int64_t nvec,
+                              S* __restrict__ gx, int T, int64_t N, int64_t GN, int64_t nvec,
                               typename Arith<S>::type alpha, typename Arith<S>::type thresh,
                               typename Arith<S>::type beta, typename Arith<S>::type interval) {
     using C = typename Arith<S>::type;
@@ -576,8 +578,9 @@ lif_backward_segmented_kernel(const S* __restrict__ x, const S* __restrict__ g,
         {
             const int t0 = (nseg - 1) * kSegment;
             const int64_t off = static_cast<int64_t>(t0) * N;
-            backward_window<S, V, kSegment, false>(x + off, g + off, gx + off, T - t0, N, col, uc, sc,
-                                                   gu, alpha, thresh, beta, interval);
+            backward_window<S, V, kSegment, false>(x + off, g + static_cast<int64_t>(t0) * GN, gx + off,
+                                                   T - t0, N, GN, col, uc, sc, gu, alpha, thresh,
+                                                   beta, interval);
         }
         for (int seg = nseg - 2; seg >= 0; --seg) {
 #pragma unroll
@@ -587,8 +590,9 @@ lif_backward_segmented_kernel(const S* __restrict__ x, const S* __restrict__ g,
                 sc[j] = (seg != 0 && uc[j] > thresh) ? C(1) : C(0);
             }
             const int64_t off = static_cast<int64_t>(seg) * kSegment * N;
-            backward_window<S, V, kSegment, true>(x + off, g + off, gx + off, kSegment, N, col, uc, sc,
-                                                  gu, alpha, thresh, beta, interval);
+            backward_window<S, V, kSegment, true>(x + off, g + static_cast<int64_t>(seg) * kSegment * GN,
+                                                  gx + off, kSegment, N, GN, col, uc, sc, gu, alpha,
+                                                  thresh, beta, interval);
         }
     }
 }
@@ -601,7 +605,7 @@ template <typename S, int V, int TC>
 __global__ void __launch_bounds__(kBwdBlock)
 lif_backward_stream_kernel(const typename Arith<S>::type* __restrict__ mem,
                            const S* __restrict__ g, S* __restrict__ gx, int T, int64_t N,
-                           int64_t nvec, typename Arith<S>::type alpha,
+                           int64_t GN, int64_t nvec, typename Arith<S>::type alpha,
                            typename Arith<S>::type thresh, typename Arith<S>::type beta,
                            typename Arith<S>::type interval) {
     using C = typename Arith<S>::type;
@@ -624,16 +628,16 @@ lif_backward_stream_kernel(const typename Arith<S>::type* __restrict__ mem,
             gcur[k] = zero_pack<S, V>();
             if (t < T) {
                 mcur[k] = load_pack<C, V, true>(mem + static_cast<int64_t>(t) * N + col);
-                gcur[k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * N + col);
+                gcur[k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * GN + col);
             }
         }
         for (int c = ngroups - 1; c >= 0; --c) {
             if (c > 0) {
 #pragma unroll
                 for (int k = TC - 1; k >= 0; --k) {
-                    const int64_t off = static_cast<int64_t>((c - 1) * TC + k) * N + col;
-                    mnxt[k] = load_pack<C, V, true>(mem + off);
-                    gnxt[k] = load_pack<S, V, true>(g + off);
+                    const int64_t row = static_cast<int64_t>((c - 1) * TC + k);
+                    mnxt[k] = load_pack<C, V, true>(mem + row * N + col);
+                    gnxt[k] = load_pack<S, V, true>(g + row * GN + col);
                 }
             }
 #pragma unroll
@@ -712,12 +716,14 @@ inline bool aligned_to(const void* p, size_t bytes) {
     return p == nullptr || (reinterpret_cast<uintptr_t>(p) % bytes) == 0;
 }
 
-// Largest power-of-two V <= maxv such that rows (N elements apart) and the bases of all given
-// pointers stay aligned to V elements.  elem[i] is the element size behind ptrs[i].
-inline int pick_vec(int maxv, int64_t N, const void* const* ptrs, const size_t* elem, int n) {
+// Largest power-of-two V <= maxv such that rows (N elements apart, and GN for a tensor with a row
+// pitch of its own) and the bases of all given pointers stay aligned to V elements.  elem[i] is the
+// element size behind ptrs[i].
+inline int pick_vec(int maxv, int64_t N, const void* const* ptrs, const size_t* elem, int n,
+                    int64_t GN = 0) {
     int v = maxv;
     while (v > 1) {
-        bool ok = (N % v) == 0;
+        bool ok = (N % v) == 0 && (GN % v) == 0;
         for (int i = 0; ok && i < n; ++i) ok = aligned_to(ptrs[i], elem[i] * v);
         if (ok) break;
         v >>= 1;
@@ -858,13 +864,14 @@ constexpr int fused_max_vec() {
 }
 
 template <typename S, int TW, bool KEEP>
-int launch_backward_fused_policy(const S* x, const S* g, S* gx, int64_t T, int64_t N, float alpha,
-                                 float thresh, float beta, float interval, hipStream_t stream) {
+int launch_backward_fused_policy(const S* x, const S* g, S* gx, int64_t T, int64_t N, int64_t GN,
+                                 float alpha, float thresh, float beta, float interval,
+                                 hipStream_t stream) {
     using C = typename Arith<S>::type;
     constexpr int maxv = fused_max_vec<S, TW>();
     const void* ptrs[3] = {x, g, gx};
     const size_t elem[3] = {sizeof(S), sizeof(S), sizeof(S)};
-    const int v = pick_vec(maxv, N, ptrs, elem, 3);
+    const int v = pick_vec(maxv, N, ptrs, elem, 3, GN);
     // Every window of at most 8 rows has an instantiation of its own, so only the longer ones
     // are ever entered with T < TW; windows beyond the fused range are entered with T == TW only.
     constexpr bool can_be_inexact = TW > 8 && TW <= SNNLIF_BP_FUSED_MAX_T;
@@ -878,42 +885,42 @@ int launch_backward_fused_policy(const S* x, const S* g, S* gx, int64_t T, int64
         const int Ti = static_cast<int>(T);
         if (exact) {
             launch_kernel(lif_backward_fused_kernel<S, V, TW, true, KEEP>, grid, block, 0, stream,
-                               x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval));
+                               x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
         } else if constexpr (can_be_inexact) {
             launch_kernel(lif_backward_fused_kernel<S, V, TW, false, KEEP>, grid, block, 0, stream,
-                               x, g, gx, Ti, N, nvec, C(alpha), C(thresh), C(beta), C(interval));
+                               x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
         }
         return launch_status();
     });
 }
 
 template <typename S, int TW>
-int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, float alpha,
-                          float thresh, float beta, float interval, SpatialHint keep_x,
+int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, int64_t GN,
+                          float alpha, float thresh, float beta, float interval, SpatialHint keep_x,
                           hipStream_t stream) {
     if (keep_policy(keep_x, static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S)))
-        return launch_backward_fused_policy<S, TW, true>(x, g, gx, T, N, alpha, thresh, beta, interval,
-                                                         stream);
-    return launch_backward_fused_policy<S, TW, false>(x, g, gx, T, N, alpha, thresh, beta, interval,
-                                                      stream);
+        return launch_backward_fused_policy<S, TW, true>(x, g, gx, T, N, GN, alpha, thresh, beta,
+                                                         interval, stream);
+    return launch_backward_fused_policy<S, TW, false>(x, g, gx, T, N, GN, alpha, thresh, beta,
+                                                      interval, stream);
 }
 
 template <typename S, int V>
 int launch_backward_stream_v(const typename Arith<S>::type* mem, const S* g, S* gx, int64_t T,
-                             int64_t N, float alpha, float thresh, float beta, float interval,
-                             hipStream_t stream) {
+                             int64_t N, int64_t GN, float alpha, float thresh, float beta,
+                             float interval, hipStream_t stream) {
     using C = typename Arith<S>::type;
     const int64_t nvec = N / V;
     launch_kernel(lif_backward_stream_kernel<S, V, 8>, dim3(grid_for(nvec, kBwdBlock)),
-                       dim3(kBwdBlock), 0, stream, mem, g, gx, static_cast<int>(T), N, nvec,
+                       dim3(kBwdBlock), 0, stream, mem, g, gx, static_cast<int>(T), N, GN, nvec,
                        C(alpha), C(thresh), C(beta), C(interval));
     return launch_status();
 }
 
 template <typename S>
-int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int64_t N, float alpha,
-                      float thresh, float beta, float interval, SpatialHint keep_x, void* workspace,
-                      size_t workspace_bytes, hipStream_t stream) {
+int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int64_t N, int64_t GN,
+                      float alpha, float thresh, float beta, float interval, SpatialHint keep_x,
+                      void* workspace, size_t workspace_bytes, hipStream_t stream) {
     using C = typename Arith<S>::type;
     const S* x = static_cast<const S*>(x_);
     const S* g = static_cast<const S*>(g_);
@@ -925,8 +932,8 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
     // one in its zero-filled form.
 #define SNNLIF_BWD_WINDOW(TW)                                                                    \
     if (T <= TW)                                                                                 \
-        return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, keep_x, \
-                                            stream);
+        return launch_backward_fused<S, TW>(x, g, gx, T, N, GN, alpha, thresh, beta, interval,     \
+                                            keep_x, stream);
     SNNLIF_BWD_WINDOW(1)
     SNNLIF_BWD_WINDOW(2)
     SNNLIF_BWD_WINDOW(3)
@@ -956,8 +963,8 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
         sizeof(C) == 4 ? SNNLIF_BWD_WIDE_MAX_T : SNNLIF_BWD_WIDE_MAX_T_F64;
 #define SNNLIF_BWD_WIDE_WINDOW(TW)                                                               \
     if (TW <= wide_max && T == TW)                                                               \
-        return launch_backward_fused<S, TW>(x, g, gx, T, N, alpha, thresh, beta, interval, keep_x, \
-                                            stream);
+        return launch_backward_fused<S, TW>(x, g, gx, T, N, GN, alpha, thresh, beta, interval,     \
+                                            keep_x, stream);
     SNNLIF_BWD_WIDE_WINDOW(40)
     SNNLIF_BWD_WIDE_WINDOW(48)
     SNNLIF_BWD_WIDE_WINDOW(56)
@@ -977,7 +984,7 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
         constexpr int maxv = fused_max_vec<S, kSegment>();
         const void* ptrs[3] = {x, g, gx};
         const size_t elem[3] = {sizeof(S), sizeof(S), sizeof(S)};
-        const int v = pick_vec(maxv, N, ptrs, elem, 3);
+        const int v = pick_vec(maxv, N, ptrs, elem, 3, GN);
         return with_vec<maxv>(v, [&](auto vc) {
             constexpr int V = decltype(vc)::value;
             const int64_t nvec = N / V;
@@ -987,7 +994,7 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
                 backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S), 128);
             const size_t lds = static_cast<size_t>(nseg) * threads * V * sizeof(C);
             launch_kernel(lif_backward_segmented_kernel<S, V>, dim3(grid_for(nvec, threads)),
-                               dim3(threads), lds, stream, x, g, gx, static_cast<int>(T), N, nvec,
+                               dim3(threads), lds, stream, x, g, gx, static_cast<int>(T), N, GN, nvec,
                                C(alpha), C(thresh), C(beta), C(interval));
             return launch_status();
         });
@@ -1006,10 +1013,10 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
                              : static_cast<int>(16 / sizeof(C));
     const void* ptrs[3] = {mem, g, gx};
     const size_t elem[3] = {sizeof(C), sizeof(S), sizeof(S)};
-    const int v = pick_vec(maxv, N, ptrs, elem, 3);
+    const int v = pick_vec(maxv, N, ptrs, elem, 3, GN);
     return with_vec<maxv>(v, [&](auto vc) {
         constexpr int V = decltype(vc)::value;
-        return launch_backward_stream_v<S, V>(mem, g, gx, T, N, alpha, thresh, beta, interval,
+        return launch_backward_stream_v<S, V>(mem, g, gx, T, N, GN, alpha, thresh, beta, interval,
                                               stream);
     });
 }
@@ -1019,9 +1026,9 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
 #define SNNLIF_DECLARE_DTYPE(NAME)                                                                  \
     int forward_##NAME(const void* x, void* mem, void* spike, int64_t T, int64_t N, float alpha,    \
                        float thresh, SpatialHint keep_x, hipStream_t stream);                              \
-    int backward_##NAME(const void* x, const void* g, void* gx, int64_t T, int64_t N, float alpha,  \
-                        float thresh, float beta, float interval, SpatialHint keep_x, void* workspace,     \
-                        size_t workspace_bytes, hipStream_t stream);
+    int backward_##NAME(const void* x, const void* g, void* gx, int64_t T, int64_t N, int64_t GN,   \
+                        float alpha, float thresh, float beta, float interval, SpatialHint keep_x,  \
+                        void* workspace, size_t workspace_bytes, hipStream_t stream);
 SNNLIF_DECLARE_DTYPE(f32)
 SNNLIF_DECLARE_DTYPE(f64)
 SNNLIF_DECLARE_DTYPE(bf16)
@@ -1032,10 +1039,10 @@ SNNLIF_DECLARE_DTYPE(bf16)
                        float thresh, SpatialHint keep_x, hipStream_t stream) {                             \
         return forward_dispatch<S>(x, mem, spike, T, N, alpha, thresh, keep_x, stream);             \
     }                                                                                               \
-    int backward_##NAME(const void* x, const void* g, void* gx, int64_t T, int64_t N, float alpha,  \
-                        float thresh, float beta, float interval, SpatialHint keep_x, void* workspace,     \
-                        size_t workspace_bytes, hipStream_t stream) {                               \
-        return backward_dispatch<S>(x, g, gx, T, N, alpha, thresh, beta, interval, keep_x,          \
+    int backward_##NAME(const void* x, const void* g, void* gx, int64_t T, int64_t N, int64_t GN,   \
+                        float alpha, float thresh, float beta, float interval, SpatialHint keep_x,  \
+                        void* workspace, size_t workspace_bytes, hipStream_t stream) {              \
+        return backward_dispatch<S>(x, g, gx, T, N, GN, alpha, thresh, beta, interval, keep_x,      \
                                     workspace, workspace_bytes, stream);                            \
     }
 

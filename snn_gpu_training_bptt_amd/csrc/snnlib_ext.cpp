@@ -251,9 +251,20 @@ Tensor fire_bp(Tensor spatial, Tensor grad_spike, float alpha, float thresh, flo
     const int dtype = storage_dtype(spatial, "fire_bp");
     const DeviceGuard guard(spatial.device());
     Tensor x = spatial.contiguous();
-    Tensor g = grad_spike.contiguous();
     Tensor grad_spatial = torch::empty_like(x, at::MemoryFormat::Contiguous);
     const Dims d = dims_of(x);
+    // A gradient that is one [N] row expanded over time (stride 0 on the time axis: what autograd
+    // hands over after `spike.sum(dim=0)`) is read in place, N values instead of T*N; any other
+    // layout is made dense, as the reference's binding requires of its caller.
+    Tensor g;
+    int64_t grad_row_stride = d.N;
+    if (grad_spike.dim() >= 2 && grad_spike.size(0) > 1 && grad_spike.stride(0) == 0 &&
+        grad_spike.select(0, 0).is_contiguous()) {
+        g = grad_spike.select(0, 0);
+        grad_row_stride = 0;
+    } else {
+        g = grad_spike.contiguous();
+    }
 
     // Windows longer than SNNLIF_BP_FUSED_MAX_T stage the recomputed membrane potential in a
     // workspace from the caching allocator; it goes back to the allocator on return and stays
@@ -265,8 +276,9 @@ Tensor fire_bp(Tensor spatial, Tensor grad_spike, float alpha, float thresh, flo
         workspace = torch::empty({static_cast<int64_t>(ws_bytes)}, x.options().dtype(at::kByte));
         ws_ptr = workspace.data_ptr();
     }
-    check_rc(snnlif_fire_bp(x.data_ptr(), g.data_ptr(), grad_spatial.data_ptr(), dtype, d.T, d.N,
-                            alpha, thresh, beta, interval, ws_ptr, ws_bytes, current_stream()),
+    check_rc(snnlif_fire_bp_strided(x.data_ptr(), g.data_ptr(), grad_spatial.data_ptr(), dtype, d.T,
+                                    d.N, grad_row_stride, alpha, thresh, beta, interval, ws_ptr,
+                                    ws_bytes, current_stream()),
              "fire_bp");
     return grad_spatial;
 }

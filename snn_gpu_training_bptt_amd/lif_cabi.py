@@ -30,6 +30,8 @@ SYMBOLS = {
     "snnlif_fire_us_fp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64]),
     "snnlif_fire_bp": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
+    "snnlif_fire_bp_strided": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp,
+                                      _sz, _vp]),
     "snnlif_bn_stats_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "snnlif_bn_stats": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
     "snnlif_bn_fire_s_fp": (_int, [_vp] * 7 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _vp]),
@@ -198,20 +200,46 @@ def fire_bp_workspace_bytes(dtype_code, T, N):
     return int(load().snnlif_fire_bp_workspace_bytes(dtype_code, T, N))
 
 
+def _grad_row_stride(grad_spike, N):
+    """Elements between consecutive time rows of ``grad_spike`` as ``snnlif_fire_bp_strided`` takes
+    them: N for a dense tensor, 0 for one row expanded over time, more than N for rows of a wider
+    tensor.  Each row itself must be dense."""
+    if grad_spike.is_contiguous():
+        return N
+    if grad_spike.dim() >= 2 and grad_spike[0].is_contiguous():
+        stride = grad_spike.stride(0)
+        if stride == 0 or stride >= N:
+            return stride
+    raise ValueError("grad_spike: dense time rows required (the time axis may have any stride >= N, or 0)")
+
+
 def fire_bp_into(spatial, grad_spike, grad_spatial, alpha, thresh, beta, interval, workspace=None,
                  keep_spatial=None):
-    """``snnlif_fire_bp``; ``workspace`` is a uint8 device tensor when the shape needs one."""
+    """``snnlif_fire_bp_strided`` (``snnlif_fire_bp`` for a dense gradient); ``workspace`` is a uint8
+    device tensor when the shape needs one.  ``grad_spike`` may be a stride-0 expansion over time
+    (``row.expand(T, ...)``): it is read in place."""
     _require_like(spatial, grad_spike=grad_spike, grad_spatial=grad_spatial)
     T, N = _dims(spatial)
     _require_workspace(spatial, workspace, fire_bp_workspace_bytes(_torch_dtype_code(spatial), T, N),
                        "snnlif_fire_bp")
     ws_ptr = workspace.data_ptr() if workspace is not None else None
     ws_bytes = workspace.numel() * workspace.element_size() if workspace is not None else 0
-    _require_dense_gpu(spatial, grad_spike, grad_spatial, workspace)
-    rc = load().snnlif_fire_bp(spatial.data_ptr(), grad_spike.data_ptr(), grad_spatial.data_ptr(),
-                               _hinted(_torch_dtype_code(spatial), keep_spatial), T, N, alpha, thresh,
-                               beta, interval, ws_ptr, ws_bytes, _stream_handle(spatial))
-    _check(rc, "snnlif_fire_bp")
+    grad_row_stride = _grad_row_stride(grad_spike, N)
+    if not grad_spike.is_cuda:
+        raise ValueError("device tensor required")
+    _require_dense_gpu(spatial, grad_spatial, workspace)
+    if grad_row_stride == N:
+        rc = load().snnlif_fire_bp(spatial.data_ptr(), grad_spike.data_ptr(), grad_spatial.data_ptr(),
+                                   _hinted(_torch_dtype_code(spatial), keep_spatial), T, N, alpha,
+                                   thresh, beta, interval, ws_ptr, ws_bytes, _stream_handle(spatial))
+        _check(rc, "snnlif_fire_bp")
+    else:
+        rc = load().snnlif_fire_bp_strided(spatial.data_ptr(), grad_spike.data_ptr(),
+                                           grad_spatial.data_ptr(),
+                                           _hinted(_torch_dtype_code(spatial), keep_spatial), T, N,
+                                           grad_row_stride, alpha, thresh, beta, interval, ws_ptr,
+                                           ws_bytes, _stream_handle(spatial))
+        _check(rc, "snnlif_fire_bp_strided")
     return grad_spatial
 
 

@@ -60,8 +60,8 @@ class FireFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad_spike):
         (spatial,) = ctx.saved_tensors
-        # the native op makes both operands dense itself (the upstream gradient is often a
-        # stride-0 expansion, e.g. after a mean over time)
+        # the native op reads a gradient that is one row expanded over time (stride 0 on axis 0, as
+        # after ``spike.sum(dim=0)``) in place and makes any other non-dense operand dense itself
         return snnlib.fire_bp(spatial, grad_spike, *_surrogate())
 
 

@@ -289,3 +289,80 @@ def test_bf16_misaligned_base_takes_single_lanes(cabi, oracle):
     gx_o = oracle.fire_backward(x.float().numpy(), g.float().numpy(), ALPHA, THRESH, BETA, INTERVAL)
     assert np.array_equal(spike.float().cpu().numpy(), spike_o)
     assert torch.equal(gx.cpu(), torch.from_numpy(gx_o).bfloat16())
+
+
+def _backward_with_gradient_layout(cabi, x, g_rows, alpha, keep=None):
+    """Backward through the C ABI with ``g_rows`` (a device tensor of x's shape, any time-axis layout)."""
+    xd = x.cuda()
+    gx = torch.empty_like(xd)
+    code = {torch.float32: 0, torch.float64: 1, torch.bfloat16: 2}[x.dtype]
+    T = x.shape[0]
+    ws_bytes = cabi.fire_bp_workspace_bytes(code, T, x.numel() // T)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda") if ws_bytes else None
+    cabi.fire_bp_into(xd, g_rows, gx, alpha, THRESH, BETA, INTERVAL, workspace=ws, keep_spatial=keep)
+    torch.cuda.synchronize()
+    return gx.cpu()
+
+
+@HINTS
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("T", [1, 2, 8, 9, 16, 31, 32, 50, 64, 96, 130, 1030])
+def test_gradient_expanded_over_time_is_read_in_place(cabi, oracle, T, dtype, keep):
+    """A gradient that is one [N] row for every time step (stride 0 on the time axis, what autograd
+    hands over after ``spike.sum(dim=0)``) goes to ``snnlif_fire_bp_strided`` as it is.  The result
+    must be the oracle's on the gradient made dense, and the bits of the dense call: every kernel
+    form of the backward (register windows exact and zero-filled, wide windows, segments, workspace
+    stream) takes the row stride.  Even N (pairs of bf16 per lane) and odd N."""
+    for n_inner in (256, 77):
+        x32, g32 = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=5000 + T)
+        x = x32.to(dtype)
+        row = g32[0].to(dtype)
+        g_dense = row.unsqueeze(0).expand(T, 2, n_inner).contiguous()
+        g_view = row.cuda().unsqueeze(0).expand(T, 2, n_inner)
+        assert T == 1 or g_view.stride(0) == 0
+        gx = _backward_with_gradient_layout(cabi, x, g_view, 0.3, keep)
+        gx_dense = _backward_with_gradient_layout(cabi, x, g_dense.cuda(), 0.3, keep)
+        assert torch.equal(gx, gx_dense)
+        wide = torch.float64 if dtype == torch.float64 else torch.float32
+        gx_o = oracle.fire_backward(x.to(wide).numpy(), g_dense.to(wide).numpy(), 0.3, THRESH, BETA, INTERVAL)
+        if dtype == torch.bfloat16:
+            assert torch.equal(gx, torch.from_numpy(gx_o).bfloat16())
+        else:
+            np.testing.assert_allclose(gx.numpy(), gx_o, rtol=RTOL, atol=0)
+            assert np.array_equal(gx.numpy(), gx_o)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,pad", [(8, 1), (8, 64), (20, 3), (96, 2), (50, 5)])
+def test_gradient_rows_of_a_wider_tensor(cabi, oracle, T, pad, dtype):
+    """Time rows further apart than N (a slice of a wider tensor).  An odd pitch forces single bf16
+    lanes even for even N."""
+    n_inner = 128
+    x32, g32 = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=6000 + T)
+    x, g = x32.to(dtype), g32.to(dtype)
+    N = 2 * n_inner
+    backing = torch.full((T, N + pad), float("nan"), dtype=dtype, device="cuda")
+    backing[:, :N] = g.reshape(T, N).cuda()
+    g_view = backing[:, :N].unflatten(1, (2, n_inner))
+    assert g_view.stride(0) == N + pad and not g_view.is_contiguous()
+    gx = _backward_with_gradient_layout(cabi, x, g_view, 0.3)
+    gx_dense = _backward_with_gradient_layout(cabi, x, g.cuda(), 0.3)
+    assert torch.equal(gx, gx_dense)
+    assert not torch.isnan(gx.float()).any()
+
+
+def test_gradient_row_stride_is_validated(cabi):
+    lib = cabi.load()
+    x = torch.zeros(4, 64, device="cuda")
+    g = torch.zeros(4, 64, device="cuda")
+    gx = torch.empty(4, 64, device="cuda")
+    args = (x.data_ptr(), g.data_ptr(), gx.data_ptr(), 0, 4, 64)
+    tail = (0.25, 0.5, 1.0, 0.5, None, 0, None)
+    assert lib.snnlif_fire_bp_strided(*args, -1, *tail) == cabi.ERR_ARG
+    assert lib.snnlif_fire_bp_strided(*args, 63, *tail) == cabi.ERR_ARG      # rows would overlap
+    assert lib.snnlif_fire_bp_strided(*args, 1, *tail) == cabi.ERR_ARG
+    assert lib.snnlif_fire_bp_strided(*args, 64, *tail) == cabi.OK
+    assert lib.snnlif_fire_bp_strided(*args, 0, *tail) == cabi.OK
+    torch.cuda.synchronize()
+    with pytest.raises(ValueError):   # rows that are not dense themselves
+        cabi.fire_bp_into(x, torch.zeros(4, 128, device="cuda")[:, ::2], gx, 0.25, 0.5, 1.0, 0.5)

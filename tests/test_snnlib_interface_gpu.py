@@ -88,7 +88,7 @@ def test_hyperparameters_are_read_at_call_time(mods):
 
 def test_strided_input_and_expanded_gradient(mods):
     """Forward gets a non-contiguous view; backward gets a stride-0 expansion over T (what
-    ``mean(dim=0)`` produces) -- both must behave as if dense."""
+    ``sum(dim=0)`` produces; the module reads it in place) -- both must behave as if dense."""
     sf, sop, gold = mods
     sf.thresh = 0.5
     gen = torch.Generator().manual_seed(13)
@@ -104,6 +104,32 @@ def test_strided_input_and_expanded_gradient(mods):
     _, s_ref, gx_ref = gold.gold_fire_fwd_bwd(x_cpu.contiguous(), g_cpu.contiguous(), sf.alpha, sf.thresh, sf.beta, sf.interval)
     assert torch.equal(s.detach().cpu(), s_ref)
     assert torch.equal(x.grad.cpu(), gx_ref)
+
+
+@pytest.mark.parametrize("T", [6, 20, 50])
+def test_rate_decoding_by_a_sum_over_time(mods, T):
+    """``spike.sum(dim=0) / T`` ahead of the loss: autograd hands the fire backward one row expanded
+    over time.  Same spikes and the same input gradient as the gold fire under the same graph."""
+    sf, sop, gold = mods
+    sf.thresh = 0.5
+    gen = torch.Generator().manual_seed(17)
+    x_cpu = 0.5 + torch.randn((T, 4, 12, 5), generator=gen)
+    w_cpu = torch.randn((4, 12, 5), generator=gen)
+    seen = []
+
+    x = x_cpu.cuda().requires_grad_(True)
+    s = sop.Fire()(x)
+    s.register_hook(lambda grad: seen.append(grad.stride()))
+    ((s.sum(dim=0) / T) * w_cpu.cuda()).sum().backward()
+    assert seen and seen[0][0] == 0, "autograd no longer expands the gradient of a sum: test needs another graph"
+
+    # the gold fire on the same device: the graph around the fire op is then the same kernels on both
+    # sides (a division by a scalar is a multiplication by its reciprocal on the GPU), so bits must agree
+    xg = x_cpu.cuda().requires_grad_(True)
+    _, s_ref = gold.gold_fire(xg, sf.alpha, sf.thresh, sf.beta, sf.interval)
+    ((s_ref.sum(dim=0) / T) * w_cpu.cuda()).sum().backward()
+    assert torch.equal(s.detach(), s_ref.detach())
+    assert torch.equal(x.grad, xg.grad)
 
 
 @pytest.mark.parametrize("T", [40, 1100])
