@@ -129,6 +129,13 @@
 #ifndef SNNLIF_STREAM_FWD_WAVES_LONG
 #define SNNLIF_STREAM_FWD_WAVES_LONG 4
 #endif
+// ... and of the forward for a window of exactly 8 rows on a tensor of at most so many bytes.
+#ifndef SNNLIF_STREAM_FWD_WAVES_8
+#define SNNLIF_STREAM_FWD_WAVES_8 5
+#endif
+#ifndef SNNLIF_STREAM_FWD_CAPPED_BYTES
+#define SNNLIF_STREAM_FWD_CAPPED_BYTES (size_t(256) << 20)
+#endif
 // Rows of x the forward requests before consuming the first (windows longer than this are
 // streamed with the next group of rows in flight).
 #ifndef SNNLIF_FWD_ROWS
@@ -163,11 +170,18 @@ constexpr int backward_waves(int rows, bool keep = true) {
 }
 
 // The forward keeps `rows` (twice that when the window is streamed in groups) requests per wavefront
-// in flight; only long streamed windows gain from a cap.
-constexpr int forward_waves(int rows, bool keep) {
+// in flight; long streamed windows gain from a cap, and so does (`capped`) the streamed 8-step window
+// on tensors of up to SNNLIF_STREAM_FWD_CAPPED_BYTES: there the 16 row streams of the kernel sit a
+// power of two apart in the usual shapes, and with all 8 wavefronts resident the rate depends on
+// where the output tensor lies relative to the input (66 % of the HBM peak with the output right
+// behind the input, 78 % one tensor further; capped: 77-79 % either way; plain copies of 8 rows in
+// that layout behave the same: 68 / 76 % uncapped, 79 / 80 % at 4 wavefronts).  Windows of 5-7 steps
+// share the kernel but lose 2-10 points under the cap, larger tensors 2-3, so neither is capped.
+constexpr int forward_waves(int rows, bool keep, bool capped = false) {
 #ifdef SNNLIF_FWD_MAX_WAVES
     return SNNLIF_FWD_MAX_WAVES;
 #else
+    if (capped) return SNNLIF_STREAM_FWD_WAVES_8;
     return (!keep && rows > 8) ? SNNLIF_STREAM_FWD_WAVES_LONG : 8;
 #endif
 }
@@ -324,8 +338,9 @@ __device__ __forceinline__ void lif_reverse_step(C& gu, C u, C g, C alpha, C thr
 // flight while the current ones are processed.  KEEP: x is loaded with the default cache policy
 // (see the file header); otherwise with the non-temporal hint.
 // ---------------------------------------------------------------------------------------------
-template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP>
-__global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(forward_waves(TC, KEEP))
+template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP,
+          bool CAPPED = false>
+__global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(forward_waves(TC, KEEP, CAPPED))
 lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__ spike, int T,
                    int64_t N, int64_t nvec, typename Arith<S>::type alpha,
                    typename Arith<S>::type thresh) {
@@ -751,12 +766,13 @@ inline int with_vec(int v, F&& f) {
 }
 
 // One forward launch with TC rows per group.
-template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP>
+template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP,
+          bool CAPPED = false>
 int launch_forward_rows(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
                         int threads, hipStream_t stream) {
     using C = typename Arith<S>::type;
     const int64_t nvec = N / V;
-    launch_kernel(lif_forward_kernel<S, M, V, TC, MULTI, WRITE_U, WRITE_S, KEEP>,
+    launch_kernel(lif_forward_kernel<S, M, V, TC, MULTI, WRITE_U, WRITE_S, KEEP, CAPPED>,
                   dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
                   static_cast<int>(T), N, nvec, C(alpha), C(thresh));
     return launch_status();
@@ -777,6 +793,12 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
     launch_forward_rows<S, M, V, ROWS, MULTI, WRITE_U, WRITE_S, KEEP>(x, mem, spike, T, N, alpha,  \
                                                                       thresh, threads, stream)
     if (T <= 4 && TC > 4) return SNNLIF_FWD_LAUNCH(4, false);
+    if constexpr (!KEEP && TC == 8) {
+        if (T == TC && static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S) <=
+                           static_cast<size_t>(SNNLIF_STREAM_FWD_CAPPED_BYTES))
+            return launch_forward_rows<S, M, V, TC, false, WRITE_U, WRITE_S, KEEP, true>(
+                x, mem, spike, T, N, alpha, thresh, threads, stream);
+    }
     if (T <= TC) return SNNLIF_FWD_LAUNCH(TC, false);
     if constexpr (!KEEP) {
         if (T <= TL) return SNNLIF_FWD_LAUNCH(TL, false);
