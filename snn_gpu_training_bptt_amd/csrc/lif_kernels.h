@@ -116,7 +116,7 @@
 #define SNNLIF_RESIDENT_TENSOR_BYTES (size_t(32) << 20)
 #endif
 // Streamed policy: workgroup size of both kernels, wavefronts per SIMD of the backward for windows
-// of at most 8 rows / longer ones, of the forward for windows of more than 8 rows.
+// of at most 8 rows / longer ones, of the forward for windows of 9 to 16 rows / longer ones.
 #ifndef SNNLIF_STREAM_BLOCK
 #define SNNLIF_STREAM_BLOCK 256
 #endif
@@ -126,8 +126,26 @@
 #ifndef SNNLIF_STREAM_BWD_WAVES_LONG
 #define SNNLIF_STREAM_BWD_WAVES_LONG 4
 #endif
+#ifndef SNNLIF_STREAM_BWD_WAVES_3  // windows of exactly 3 / 4 rows
+#define SNNLIF_STREAM_BWD_WAVES_3 8
+#endif
+#ifndef SNNLIF_STREAM_BWD_WAVES_4
+#define SNNLIF_STREAM_BWD_WAVES_4 7
+#endif
+#ifndef SNNLIF_STREAM_FWD_WAVES_MID
+#define SNNLIF_STREAM_FWD_WAVES_MID 4
+#endif
 #ifndef SNNLIF_STREAM_FWD_WAVES_LONG
-#define SNNLIF_STREAM_FWD_WAVES_LONG 4
+#define SNNLIF_STREAM_FWD_WAVES_LONG 3
+#endif
+// Rows the streamed forward requests at once: windows of 9 rows up to the first run whole in that
+// instantiation, windows of at least three quarters of the second and up to it whole in that one;
+// all others go in groups of the first.
+#ifndef SNNLIF_STREAM_FWD_ROWS_MID
+#define SNNLIF_STREAM_FWD_ROWS_MID 16
+#endif
+#ifndef SNNLIF_STREAM_FWD_ROWS_LONG
+#define SNNLIF_STREAM_FWD_ROWS_LONG 32
 #endif
 // ... and of the forward for a window of exactly 8 rows on a tensor of at most so many bytes.
 #ifndef SNNLIF_STREAM_FWD_WAVES_8
@@ -157,14 +175,20 @@ namespace snnlif {
 // Kept x (part of the traffic served by the memory-side cache): past roughly 100 requests per SIMD the
 // streams of different wavefronts start to evict each other's DRAM pages (-4 % at 16 rows and -9 % at
 // 32 rows with all 8 wavefronts resident; windows of up to 8 rows are best left uncapped).
-// Streamed x (everything from HBM): fewer wavefronts already pay for short windows (8 rows: 84 % of
-// peak at 5 wavefronts against 78 % at 8).  SNNLIF_BWD_MAX_WAVES overrides both.
+// Streamed x (everything from HBM): fewer wavefronts already pay for windows of 5 to 8 rows (8 rows:
+// 84 % of peak at 5 wavefronts against 78 % at 8), while windows of 3 and 4 rows need 8 and 7 to keep
+// enough requests going (cold, 256 MiB tensors: 3 rows 71 -> 83 %, 4 rows 76 -> 84 % against 5
+// wavefronts; 5 rows and more lose 1-6 points beyond 5).  SNNLIF_BWD_MAX_WAVES overrides both.
 constexpr int backward_waves(int rows, bool keep = true) {
 #ifdef SNNLIF_BWD_MAX_WAVES
     return SNNLIF_BWD_MAX_WAVES;
 #else
     if (rows > 64) return 3;  // u alone takes `rows` VGPRs per lane
-    if (!keep) return rows <= 8 ? SNNLIF_STREAM_BWD_WAVES_SHORT : SNNLIF_STREAM_BWD_WAVES_LONG;
+    if (!keep) {
+        if (rows == 3) return SNNLIF_STREAM_BWD_WAVES_3;
+        if (rows == 4) return SNNLIF_STREAM_BWD_WAVES_4;
+        return rows <= 8 ? SNNLIF_STREAM_BWD_WAVES_SHORT : SNNLIF_STREAM_BWD_WAVES_LONG;
+    }
     return rows <= 8 ? 8 : (rows <= 12 ? 5 : 4);
 #endif
 }
@@ -182,7 +206,8 @@ constexpr int forward_waves(int rows, bool keep, bool capped = false) {
     return SNNLIF_FWD_MAX_WAVES;
 #else
     if (capped) return SNNLIF_STREAM_FWD_WAVES_8;
-    return (!keep && rows > 8) ? SNNLIF_STREAM_FWD_WAVES_LONG : 8;
+    if (!keep && rows > SNNLIF_STREAM_FWD_ROWS_MID) return SNNLIF_STREAM_FWD_WAVES_LONG;
+    return (!keep && rows > 8) ? SNNLIF_STREAM_FWD_WAVES_MID : 8;  // groups of SNNLIF_STREAM_FWD_ROWS_MID too
 #endif
 }
 
@@ -780,15 +805,18 @@ int launch_forward_rows(const S* x, M* mem, S* spike, int64_t T, int64_t N, floa
 
 // Rows per group by window length.  Kept x: the whole window up to SNNLIF_FWD_ROWS rows, longer ones
 // streamed in groups of that many.  Streamed x: windows of up to 16 rows are requested whole (a
-// window of 9-16 rows as one group measures +5-8 points over two groups of 8), longer ones go in
-// groups of 16.
+// window of 9-16 rows as one group measures +5-8 points over two groups of 8), and so are windows
+// of 24-32 rows, in a 32-row instantiation at 3 wavefronts per SIMD (+3-5 points over two groups of
+// 16; a 20-row window zero-filled to 32 loses 4-8, so 17-23 rows stay in groups).  Everything else
+// goes in groups of 16 (groups of 32 gain 3-4 points at 48 and 64 rows and lose 1-7 from 96 on).
 template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S, bool KEEP>
 int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
                      hipStream_t stream) {
     const int threads =
         forward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S), KEEP);
     constexpr int TC = SNNLIF_FWD_ROWS;
-    constexpr int TL = KEEP ? TC : 2 * TC;  // rows per group of the long-window form
+    constexpr int TM = KEEP ? TC : SNNLIF_STREAM_FWD_ROWS_MID;  // rows per group of the long-window form
+    constexpr int TL = SNNLIF_STREAM_FWD_ROWS_LONG;
 #define SNNLIF_FWD_LAUNCH(ROWS, MULTI)                                                           \
     launch_forward_rows<S, M, V, ROWS, MULTI, WRITE_U, WRITE_S, KEEP>(x, mem, spike, T, N, alpha,  \
                                                                       thresh, threads, stream)
@@ -801,9 +829,10 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
     }
     if (T <= TC) return SNNLIF_FWD_LAUNCH(TC, false);
     if constexpr (!KEEP) {
-        if (T <= TL) return SNNLIF_FWD_LAUNCH(TL, false);
+        if (T <= TM) return SNNLIF_FWD_LAUNCH(TM, false);
+        if (T <= TL && T >= TL - TL / 4) return SNNLIF_FWD_LAUNCH(TL, false);
     }
-    return SNNLIF_FWD_LAUNCH(TL, true);
+    return SNNLIF_FWD_LAUNCH(TM, true);
 #undef SNNLIF_FWD_LAUNCH
 }
 
