@@ -120,6 +120,12 @@
 #ifndef SNNLIF_STREAM_BLOCK
 #define SNNLIF_STREAM_BLOCK 256
 #endif
+#ifndef SNNLIF_STREAM_SMALL_BLOCK  // ... for tensors of at most SNNLIF_STREAM_SMALL_BYTES
+#define SNNLIF_STREAM_SMALL_BLOCK 128
+#endif
+#ifndef SNNLIF_STREAM_SMALL_BYTES
+#define SNNLIF_STREAM_SMALL_BYTES (size_t(128) << 20)
+#endif
 #ifndef SNNLIF_STREAM_BWD_WAVES_SHORT
 #define SNNLIF_STREAM_BWD_WAVES_SHORT 5
 #endif
@@ -240,12 +246,21 @@ inline bool keep_policy(SpatialHint hint, size_t tensor_bytes) {
     if (hint == SpatialHint::stream) return false;
     return tensor_bytes <= kResidentTensorBytes;
 }
+// Workgroup size of the streamed shape: 256 threads, 128 for tensors of at most
+// SNNLIF_STREAM_SMALL_BYTES (cold, 64-128 MiB tensors: forward +1-15 points, backward 0-8; 256 MiB
+// tensors lose 4-7 points with 128 threads, except at row pitches of 4 MiB).
+inline int stream_block(size_t tensor_bytes, int limit) {
+    const int block = tensor_bytes <= static_cast<size_t>(SNNLIF_STREAM_SMALL_BYTES)
+                          ? SNNLIF_STREAM_SMALL_BLOCK
+                          : SNNLIF_STREAM_BLOCK;
+    return block < limit ? block : limit;
+}
 inline int forward_block(size_t tensor_bytes, bool keep = true) {
-    if (!keep) return SNNLIF_STREAM_BLOCK < kFwdBlock ? SNNLIF_STREAM_BLOCK : kFwdBlock;
+    if (!keep) return stream_block(tensor_bytes, kFwdBlock);
     return (tensor_bytes <= kSmallTensorBytesFwd && kFwdBlock > 128) ? 128 : kFwdBlock;
 }
 inline int backward_block(size_t tensor_bytes, int small = 64, bool keep = true) {
-    if (!keep) return SNNLIF_STREAM_BLOCK < kBwdBlock ? SNNLIF_STREAM_BLOCK : kBwdBlock;
+    if (!keep) return stream_block(tensor_bytes, kBwdBlock);
     return (tensor_bytes <= kSmallTensorBytes && kBwdBlock > small) ? small : kBwdBlock;
 }
 
