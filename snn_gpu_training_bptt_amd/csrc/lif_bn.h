@@ -69,6 +69,18 @@ inline int bn_stats_row_slices(int64_t rows, int64_t CHW) {
     if (s < 1) s = 1;
     return static_cast<int>(s);
 }
+// Row slices of the plane-aligned statistics kernel: one per batch entry, fewer for windows shorter
+// than the kernel's group of rows (so that every lane still sums a whole group).
+#ifndef SNNLIF_STATS_ROWS
+#define SNNLIF_STATS_ROWS 8
+#endif
+inline int64_t bn_stats_wave_slices(int64_t T, int64_t B) {
+    if (T >= SNNLIF_STATS_ROWS || B > 0x7fffffff / SNNLIF_STATS_ROWS) return B;  // (row counts stay in int)
+    int64_t s = (T * B) / SNNLIF_STATS_ROWS;
+    if (s > B) s = B;
+    if (s < 1) s = 1;
+    return s;
+}
 inline size_t bn_stats_partial_count(int64_t T, int64_t B, int64_t C, int64_t HW) {
     if (bn_wave_partials(HW)) return bn_partial_count(B, C, HW);
     return static_cast<size_t>(bn_stats_row_slices(T * B, C * HW)) * static_cast<size_t>(C * HW);

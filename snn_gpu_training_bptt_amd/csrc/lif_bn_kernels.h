@@ -61,8 +61,11 @@ __device__ __forceinline__ int channel_of(int64_t col, int64_t C, int64_t HW, bo
 // published (how the backward of the fused layers recomputes the spikes, as the reference's
 // bn_fire_us_fp_kernel does, snnlib/cuda/snn_kernel_bp.cu:481-530).
 // ---------------------------------------------------------------------------------------------
+#ifndef SNNLIF_BN_FWD_WAVES
+#define SNNLIF_BN_FWD_WAVES 8
+#endif
 template <typename F, int TC, bool MULTI, bool FROM_IVAR>
-__global__ void __launch_bounds__(kFwdBlock)
+__global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_BN_FWD_WAVES)
 lif_bn_forward_kernel(const F* __restrict__ x, const F* __restrict__ weight,
                       const F* __restrict__ bias, const F* __restrict__ stat,
                       const F* __restrict__ mean, F* __restrict__ ivar,

@@ -11,10 +11,11 @@
 //
 // One pass over x (4 bytes per neuron-step in fp32), HBM-bound, two kernels:
 //   1. partial sums.  Planes of at least 32 positions: wavefronts are laid over the (batch entry,
-//      channel) planes exactly as in sweep 1 of the batch-norm backward (ceil(HW/64) wavefronts per
-//      plane, all lanes of a wavefront share a channel); a lane adds up its neuron's T values (eight
-//      at a time in the storage type, the groups in double), the wavefront folds the 64 lanes by
-//      shuffles and leaves one pair of sums.  Smaller planes (fully
+//      channel) planes as in sweep 1 of the batch-norm backward (ceil(HW/64) wavefronts per plane,
+//      all lanes of a wavefront share a channel); a lane adds up its neuron's T values (eight at a
+//      time in the storage type, the groups in double; windows of fewer than eight steps: the values
+//      of several batch entries, so that eight requests are in flight all the same), the wavefront
+//      folds the 64 lanes by shuffles and leaves one pair of sums.  Smaller planes (fully
 //      connected shapes): one lane per (channel, position) column of the [T*B, C*HW] matrix, the rows
 //      dealt round-robin to S slices of workgroups; consecutive lanes read consecutive addresses.
 //   2. one workgroup per channel adds the partial sums in double precision, in an order fixed by the
@@ -32,9 +33,7 @@
 namespace snnlif {
 
 // Rows requested before the first is consumed, and wavefronts per SIMD of the partial-sum kernels.
-#ifndef SNNLIF_STATS_ROWS
-#define SNNLIF_STATS_ROWS 8
-#endif
+// (SNNLIF_STATS_ROWS: lif_bn.h, which also sizes the row slices by it.)
 #ifndef SNNLIF_STATS_WAVES
 #define SNNLIF_STATS_WAVES 8
 #endif
@@ -74,39 +73,49 @@ __device__ __forceinline__ Pack<F, V> stats_fill(F value) {
     return p;
 }
 
-// Planes of at least 32 positions.  A wavefront covers 64*V consecutive positions of one plane
-// (G = ceil(HW / (64*V)) wavefronts per plane; HW is a multiple of V); part_* indexed [plane][chunk].
-template <typename F, int V>
+// Planes of at least 32 positions.  A wavefront covers 64*V consecutive positions of one channel
+// (G = ceil(HW / (64*V)) wavefronts per plane; HW is a multiple of V) and sums a set of rows of the
+// [rows = T*B, C*HW] matrix (row t*B + b) there; part_* indexed [slice][channel][chunk].
+//   SLICED = false (windows of at least kStatsRows steps): S = B slices, slice b = the T rows of
+//       batch entry b, `step` = B*C*HW elements apart, kStatsRows at a time;
+//   SLICED = true (shorter windows): the rows are dealt round-robin to S = rows / kStatsRows slices
+//       (rows s, s+S, s+2S, ... belong to slice s), so that a lane still has kStatsRows requests in
+//       flight: it sums the values of several batch entries.  `step` = C*HW.
+// (Two forms of the row loop because the general one measures 25 % slower where the first applies.)
+template <typename F, int V, bool SLICED>
 __global__ void __launch_bounds__(kStatsBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_STATS_WAVES)
-bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restrict__ part_dd, int T,
-                     int64_t N, int64_t C, int64_t HW, int64_t G) {
-    const int64_t lanes = (N / HW) * G * 64;
+bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restrict__ part_dd,
+                     int rows, int64_t step, int64_t C, int64_t HW, int64_t G, int64_t S) {
+    const int64_t lanes = S * C * G * 64;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t pc = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; pc < lanes;
          pc += stride) {
         const int64_t wave = pc >> 6;
-        const int64_t plane = wave / G;
+        const int64_t plane = wave / G;  // slice * C + channel
         const int64_t k = ((wave - plane * G) * 64 + (pc & 63)) * V;
         const int c = static_cast<int>(plane % C);
         double acc_d = 0.0, acc_dd = 0.0;
         if (k < HW) {
             const F shift = x[static_cast<int64_t>(c) * HW];
+            // first row of the slice; its further rows are `hop` elements apart
             const F* col = x + plane * HW + k;
+            const int64_t hop = SLICED ? S * step : step;
+            const int count = SLICED ? static_cast<int>((rows - plane / C + S - 1) / S) : rows;
             int t0 = 0;
-            for (; t0 + kStatsRows <= T; t0 += kStatsRows) {  // whole groups: straight-line loads
+            for (; t0 + kStatsRows <= count; t0 += kStatsRows) {  // whole groups: straight-line loads
                 Pack<F, V> v[kStatsRows];
 #pragma unroll
                 for (int r = 0; r < kStatsRows; ++r)
-                    v[r] = load_pack<F, V, false>(col + static_cast<int64_t>(t0 + r) * N);
+                    v[r] = load_pack<F, V, false>(col + static_cast<int64_t>(t0 + r) * hop);
                 stats_add_group<F, V>(v, shift, acc_d, acc_dd);
             }
-            if (t0 < T) {
+            if (t0 < count) {
                 Pack<F, V> v[kStatsRows];
 #pragma unroll
                 for (int r = 0; r < kStatsRows; ++r) {
                     v[r] = stats_fill<F, V>(shift);  // rows past the end contribute d = 0
-                    if (t0 + r < T)
-                        v[r] = load_pack<F, V, false>(col + static_cast<int64_t>(t0 + r) * N);
+                    if (t0 + r < count)
+                        v[r] = load_pack<F, V, false>(col + static_cast<int64_t>(t0 + r) * hop);
                 }
                 stats_add_group<F, V>(v, shift, acc_d, acc_dd);
             }
@@ -210,16 +219,21 @@ int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,
         int v = maxv;
         while (v > 1 && (HW % v != 0 || HW < 64 * v || !aligned_to(x, sizeof(F) * v))) v >>= 1;
         const int64_t G = (HW + 64 * v - 1) / (64 * v);
-        const dim3 grid(grid_for(B * C * G * 64, kStatsBlock)), block(kStatsBlock);
+        const int64_t S = bn_stats_wave_slices(T, B);
+        const dim3 grid(grid_for(S * C * G * 64, kStatsBlock)), block(kStatsBlock);
         const int rc = with_vec<maxv>(v, [&](auto vc) {
             constexpr int V = decltype(vc)::value;
-            launch_kernel(bn_stats_wave_kernel<F, V>, grid, block, 0, stream, x, part_d, part_dd,
-                          static_cast<int>(T), N, C, HW, G);
+            if (S == B)  // slice b = batch entry b: its T rows, N elements apart
+                launch_kernel(bn_stats_wave_kernel<F, V, false>, grid, block, 0, stream, x, part_d,
+                              part_dd, static_cast<int>(T), N, C, HW, G, S);
+            else  // row s of the [T*B, C*HW] matrix starts slice s
+                launch_kernel(bn_stats_wave_kernel<F, V, true>, grid, block, 0, stream, x, part_d,
+                              part_dd, static_cast<int>(T * B), C * HW, C, HW, G, S);
             return launch_status();
         });
         if (rc != SNNLIF_OK) return rc;
         launch_kernel(bn_stats_finalize_kernel<F>, dim3(static_cast<unsigned>(C)), dim3(kReduceBlock),
-                      0, stream, x, part_d, part_dd, out_a, out_b, HW, B, G, C * G, count, moments);
+                      0, stream, x, part_d, part_dd, out_a, out_b, HW, S, G, C * G, count, moments);
         return launch_status();
     }
     const int64_t rows = T * B, CHW = C * HW;
