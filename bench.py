@@ -333,7 +333,9 @@ def run_bn_fire(args):
         lif_cabi.bn_stats_into(x, mean, var, stats_ws)
 
     def fwd():
-        lif_cabi.bn_fire_s_fp_into(x, weight, bias, var, mean, ivar, spike, eps, ALPHA, THRESH)
+        # the backward follows straight on the same tensors: x is worth keeping in the cache
+        lif_cabi.bn_fire_s_fp_into(x, weight, bias, var, mean, ivar, spike, eps, ALPHA, THRESH,
+                                   keep_spatial=True)
 
     def bwd():
         lif_cabi.bn_fire_bp_into(x, weight, bias, ivar, mean, g, gx, gw, gb, ALPHA, THRESH, BETA,

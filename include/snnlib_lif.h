@@ -46,8 +46,9 @@ extern "C" {
 #define SNNLIF_DTYPE_BF16 2 /* bfloat16 storage, fp32 arithmetic, round-to-nearest-even stores */
 
 /*
- * Cache hints, or-ed into the `dtype` argument of snnlif_fire_s_fp, snnlif_fire_us_fp and snnlif_fire_bp
- * (accepted and without effect elsewhere; both at once: SNNLIF_ERR_DTYPE).  Results never depend on them.
+ * Cache hints, or-ed into the `dtype` argument of snnlif_fire_s_fp, snnlif_fire_us_fp, snnlif_fire_bp,
+ * snnlif_fire_bp_strided, snnlif_bn_fire_s_fp and snnlif_bn_fire_s_recompute (accepted and without effect
+ * elsewhere; both at once: SNNLIF_ERR_DTYPE).  Results never depend on them.
  * No counterpart in the reference.
  *   SNNLIF_KEEP_SPATIAL    the caller will read `spatial` again soon -- the backward runs straight after
  *       the forward, or the same input current is used step after step.  `spatial` is loaded with the

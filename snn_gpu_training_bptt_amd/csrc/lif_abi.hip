@@ -215,7 +215,7 @@ static size_t bn_element_size(int dtype, int* rc) {
         *rc = SNNLIF_ERR_DTYPE;
         return 0;
     }
-    // the cache hints are accepted and have no effect: both sweeps of the backward read x anyway
+    // the cache hints steer the forward kernels only: both sweeps of the backward read x anyway
     if (storage_of(dtype) == SNNLIF_DTYPE_F32) return sizeof(float);
     if (storage_of(dtype) == SNNLIF_DTYPE_F64) return sizeof(double);
     *rc = SNNLIF_ERR_UNSUPPORTED;
@@ -252,9 +252,9 @@ int snnlif_bn_fire_s_fp(const void* spatial, const void* weight, const void* bia
     return SNNLIF_BN_DISPATCH(
         es,
         snnlif::bn_forward_f32(CF(spatial), CF(weight), CF(bias), CF(var), CF(mean), MF(ivar),
-                               MF(spike), /*from_ivar=*/false, T, B, C, HW, eps, alpha, thresh, st),
+                               MF(spike), /*from_ivar=*/false, T, B, C, HW, eps, alpha, thresh, hint_of(dtype), st),
         snnlif::bn_forward_f64(CD(spatial), CD(weight), CD(bias), CD(var), CD(mean), MD(ivar),
-                               MD(spike), /*from_ivar=*/false, T, B, C, HW, eps, alpha, thresh, st));
+                               MD(spike), /*from_ivar=*/false, T, B, C, HW, eps, alpha, thresh, hint_of(dtype), st));
 }
 
 int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const void* bias,
@@ -275,9 +275,9 @@ int snnlif_bn_fire_s_recompute(const void* spatial, const void* weight, const vo
     return SNNLIF_BN_DISPATCH(
         es,
         snnlif::bn_forward_f32(CF(spatial), CF(weight), CF(bias), CF(ivar), CF(mean), nullptr,
-                               MF(spike), /*from_ivar=*/true, T, B, C, HW, 0.f, alpha, thresh, st),
+                               MF(spike), /*from_ivar=*/true, T, B, C, HW, 0.f, alpha, thresh, hint_of(dtype), st),
         snnlif::bn_forward_f64(CD(spatial), CD(weight), CD(bias), CD(ivar), CD(mean), nullptr,
-                               MD(spike), /*from_ivar=*/true, T, B, C, HW, 0.f, alpha, thresh, st));
+                               MD(spike), /*from_ivar=*/true, T, B, C, HW, 0.f, alpha, thresh, hint_of(dtype), st));
 }
 
 size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW) {

@@ -89,11 +89,14 @@ inline size_t bn_stats_workspace_elems(int64_t T, int64_t B, int64_t C, int64_t 
     return 2 * bn_stats_partial_count(T, B, C, HW);
 }
 
+enum class SpatialHint;  // lif_kernels.h
+
 // Per scalar type F (suffix f32 = float, f64 = double):
 //   bn_stats_*           per-channel mean and biased variance (moments = false) or E[x] and E[x^2]
 //                        (moments = true) over (T, B, HW);
 //   bn_forward_*         from_ivar = false: stat is the variance and ivar is written; true: stat is
-//                        the inverse standard deviation and ivar is not touched.
+//                        the inverse standard deviation and ivar is not touched.  keep_x: the caller's
+//                        cache hint for x (lif_kernels.h).
 //   bn_backward_stats_*  sweep 1 + channel reduction: parameter gradients and the two per-channel
 //                        means (what a batch sharded over several GPUs runs before its all-reduce);
 //   bn_backward_input_*  sweep 2: the input gradient from those means (after the all-reduce);
@@ -102,7 +105,7 @@ inline size_t bn_stats_workspace_elems(int64_t T, int64_t B, int64_t C, int64_t 
     int bn_forward_##SUFFIX(const F* x, const F* weight, const F* bias, const F* stat,             \
                             const F* mean, F* ivar, F* spike, bool from_ivar, int64_t T,           \
                             int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,\
-                            hipStream_t stream);                                                   \
+                            SpatialHint keep_x, hipStream_t stream);                               \
     int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,      \
                           int64_t C, int64_t HW, F* workspace, hipStream_t stream);                \
     int bn_backward_stats_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,      \

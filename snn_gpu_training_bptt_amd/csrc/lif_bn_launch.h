@@ -8,7 +8,7 @@
 
 namespace snnlif {
 
-template <typename F, bool FROM_IVAR>
+template <typename F, bool FROM_IVAR, bool KEEP>
 int bn_forward_launch(const F* x, const F* weight, const F* bias, const F* stat, const F* mean,
                       F* ivar, F* spike, int64_t T, int64_t B, int64_t C, int64_t HW, float eps,
                       float alpha, float thresh, hipStream_t stream) {
@@ -18,14 +18,15 @@ int bn_forward_launch(const F* x, const F* weight, const F* bias, const F* stat,
     const int Ti = static_cast<int>(T);
     constexpr int TC = SNNLIF_FWD_ROWS;
     if (T <= 4 && TC > 4) {
-        launch_kernel(lif_bn_forward_kernel<F, 4, false, FROM_IVAR>, grid, block, 0, stream, x, weight,
-                      bias, stat, mean, ivar, spike, Ti, N, C, HW, F(eps), F(alpha), F(thresh));
+        launch_kernel(lif_bn_forward_kernel<F, 4, false, FROM_IVAR, KEEP>, grid, block, 0, stream, x,
+                      weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, F(eps), F(alpha),
+                      F(thresh));
     } else if (T <= TC) {
-        launch_kernel(lif_bn_forward_kernel<F, TC, false, FROM_IVAR>, grid, block, 0, stream, x,
+        launch_kernel(lif_bn_forward_kernel<F, TC, false, FROM_IVAR, KEEP>, grid, block, 0, stream, x,
                       weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, F(eps), F(alpha),
                       F(thresh));
     } else {
-        launch_kernel(lif_bn_forward_kernel<F, TC, true, FROM_IVAR>, grid, block, 0, stream, x,
+        launch_kernel(lif_bn_forward_kernel<F, TC, true, FROM_IVAR, KEEP>, grid, block, 0, stream, x,
                       weight, bias, stat, mean, ivar, spike, Ti, N, C, HW, F(eps), F(alpha),
                       F(thresh));
     }
@@ -33,16 +34,20 @@ int bn_forward_launch(const F* x, const F* weight, const F* bias, const F* stat,
 }
 
 // from_ivar = false: stat is the variance and ivar is written; true: stat is the inverse standard
-// deviation and ivar is not touched.
+// deviation and ivar is not touched.  keep_x: the caller's cache hint; without one, tensors the
+// memory-side cache is likely to hold anyway are kept and larger ones streamed, as in the plain fire.
 template <typename F>
 int bn_forward(const F* x, const F* weight, const F* bias, const F* stat, const F* mean, F* ivar,
                F* spike, bool from_ivar, int64_t T, int64_t B, int64_t C, int64_t HW, float eps,
-               float alpha, float thresh, hipStream_t stream) {
-    if (from_ivar)
-        return bn_forward_launch<F, true>(x, weight, bias, stat, mean, ivar, spike, T, B, C, HW, eps,
-                                          alpha, thresh, stream);
-    return bn_forward_launch<F, false>(x, weight, bias, stat, mean, ivar, spike, T, B, C, HW, eps,
-                                       alpha, thresh, stream);
+               float alpha, float thresh, SpatialHint keep_x, hipStream_t stream) {
+    const bool keep = keep_policy(
+        keep_x, static_cast<size_t>(T) * static_cast<size_t>(B * C * HW) * sizeof(F));
+#define SNNLIF_BN_FWD(FROM_IVAR, KEEP)                                                            \
+    bn_forward_launch<F, FROM_IVAR, KEEP>(x, weight, bias, stat, mean, ivar, spike, T, B, C, HW, eps, \
+                                          alpha, thresh, stream)
+    if (from_ivar) return keep ? SNNLIF_BN_FWD(true, true) : SNNLIF_BN_FWD(true, false);
+    return keep ? SNNLIF_BN_FWD(false, true) : SNNLIF_BN_FWD(false, false);
+#undef SNNLIF_BN_FWD
 }
 
 // Small workgroup of the two backward sweeps (see backward_block): the sweeps carry more state per
@@ -223,9 +228,9 @@ int bn_backward(const F* x, const F* weight, const F* bias, const F* ivar, const
     int bn_forward_##SUFFIX(const F* x, const F* weight, const F* bias, const F* stat,             \
                             const F* mean, F* ivar, F* spike, bool from_ivar, int64_t T,           \
                             int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,\
-                            hipStream_t stream) {                                                  \
+                            SpatialHint keep_x, hipStream_t stream) {                              \
         return bn_forward<F>(x, weight, bias, stat, mean, ivar, spike, from_ivar, T, B, C, HW, eps,\
-                             alpha, thresh, stream);                                               \
+                             alpha, thresh, keep_x, stream);                                       \
     }                                                                                              \
     int bn_backward_stats_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,      \
                                    const F* mean, const F* g, F* grad_weight, F* grad_bias,        \

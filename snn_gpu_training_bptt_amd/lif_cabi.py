@@ -269,21 +269,22 @@ def bn_stats_into(spatial, mean, var, workspace, raw_moments=False):
     return mean, var
 
 
-def bn_fire_s_fp_into(spatial, weight, bias, var, mean, ivar, spike, eps, alpha, thresh):
-    """``snnlif_bn_fire_s_fp`` on fp32 device tensors; writes ``ivar`` ([C]) and ``spike``."""
+def bn_fire_s_fp_into(spatial, weight, bias, var, mean, ivar, spike, eps, alpha, thresh, keep_spatial=None):
+    """``snnlif_bn_fire_s_fp`` on fp32 / fp64 device tensors; writes ``ivar`` ([C]) and ``spike``.
+    ``keep_spatial``: the cache hint as in the fire helpers (True / False / None = by size)."""
     T, B, C, HW = _bn_dims(spatial)
     _require_like(spatial, spike=spike)
     _require_per_channel(spatial, C, weight=weight, bias=bias, var=var, mean=mean, ivar=ivar)
     _require_dense_gpu(spatial, weight, bias, var, mean, ivar, spike)
     rc = load().snnlif_bn_fire_s_fp(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                     var.data_ptr(), mean.data_ptr(), ivar.data_ptr(),
-                                    spike.data_ptr(), _torch_dtype_code(spatial), T, B, C, HW, eps,
-                                    alpha, thresh, _stream_handle(spatial))
+                                    spike.data_ptr(), _hinted(_torch_dtype_code(spatial), keep_spatial),
+                                    T, B, C, HW, eps, alpha, thresh, _stream_handle(spatial))
     _check(rc, "snnlif_bn_fire_s_fp")
     return ivar, spike
 
 
-def bn_fire_s_recompute_into(spatial, weight, bias, ivar, mean, spike, alpha, thresh):
+def bn_fire_s_recompute_into(spatial, weight, bias, ivar, mean, spike, alpha, thresh, keep_spatial=None):
     """``snnlif_bn_fire_s_recompute``: spikes from saved ``ivar`` / ``mean`` (backward-side scale)."""
     T, B, C, HW = _bn_dims(spatial)
     _require_like(spatial, spike=spike)
@@ -291,8 +292,8 @@ def bn_fire_s_recompute_into(spatial, weight, bias, ivar, mean, spike, alpha, th
     _require_dense_gpu(spatial, weight, bias, ivar, mean, spike)
     rc = load().snnlif_bn_fire_s_recompute(spatial.data_ptr(), weight.data_ptr(), bias.data_ptr(),
                                            ivar.data_ptr(), mean.data_ptr(), spike.data_ptr(),
-                                           _torch_dtype_code(spatial), T, B, C, HW, alpha, thresh,
-                                           _stream_handle(spatial))
+                                           _hinted(_torch_dtype_code(spatial), keep_spatial), T, B, C,
+                                           HW, alpha, thresh, _stream_handle(spatial))
     _check(rc, "snnlif_bn_fire_s_recompute")
     return spike
 

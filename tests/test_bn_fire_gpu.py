@@ -79,6 +79,11 @@ def test_bn_fire_against_oracle(cabi, shape):
     ivar = torch.empty_like(vd)
     spike = torch.empty_like(xd)
     cabi.bn_fire_s_fp_into(xd, wd, bd, vd, md, ivar, spike, EPS, ALPHA, THRESH)
+    # the cache hint selects between two instantiations of the forward: same bits from both
+    for keep in (True, False):
+        ivar_h, spike_h = torch.empty_like(vd), torch.empty_like(xd)
+        cabi.bn_fire_s_fp_into(xd, wd, bd, vd, md, ivar_h, spike_h, EPS, ALPHA, THRESH, keep_spatial=keep)
+        assert torch.equal(ivar_h, ivar) and torch.equal(spike_h, spike), f"hint keep={keep} changes the result"
     gx, gw, gb = torch.empty_like(xd), torch.empty_like(wd), torch.empty_like(wd)
     ws = torch.empty(cabi.bn_fire_bp_workspace_bytes(cabi.DTYPE_F32, T, B, C, HW), dtype=torch.uint8, device="cuda")
     cabi.bn_fire_bp_into(xd, wd, bd, ivar, md, gd, gx, gw, gb, ALPHA, THRESH, BETA, INTERVAL, ws)
@@ -251,6 +256,10 @@ def test_bn_fire_double_precision_against_oracle(cabi, shape):
     cabi.bn_fire_s_fp_into(xd, wd, bd, vd, md, ivar, spike, EPS, ALPHA, THRESH)
     again = torch.empty_like(xd)
     cabi.bn_fire_s_recompute_into(xd, wd, bd, ivar, md, again, ALPHA, THRESH)
+    for keep in (True, False):
+        hinted = torch.empty_like(xd)
+        cabi.bn_fire_s_recompute_into(xd, wd, bd, ivar, md, hinted, ALPHA, THRESH, keep_spatial=keep)
+        assert torch.equal(hinted, again)
     gx, gw, gb = torch.empty_like(xd), torch.empty_like(wd), torch.empty_like(wd)
     ws_bytes = cabi.bn_fire_bp_workspace_bytes(cabi.DTYPE_F64, T, B, C, HW)
     assert ws_bytes == 2 * cabi.bn_fire_bp_workspace_bytes(cabi.DTYPE_F32, T, B, C, HW)

@@ -107,7 +107,8 @@ def test_random_bn_fire_case(cabi, oracle, seed):
     var = var + 0.05          # also meaningful when T*B*HW == 1
     xd, gd, wd, bd, vd, md = (t.cuda() for t in (x, g, w, b, var, mean))
     ivar, spike = torch.empty_like(vd), torch.empty_like(xd)
-    cabi.bn_fire_s_fp_into(xd, wd, bd, vd, md, ivar, spike, eps, alpha, thresh)
+    cabi.bn_fire_s_fp_into(xd, wd, bd, vd, md, ivar, spike, eps, alpha, thresh,
+                           keep_spatial=(None, True, False)[seed % 3])
     gx, gw, gb = torch.empty_like(xd), torch.empty_like(wd), torch.empty_like(wd)
     code = cabi.DTYPE_F64 if dtype == torch.float64 else cabi.DTYPE_F32
     ws = torch.empty(cabi.bn_fire_bp_workspace_bytes(code, T, B, C, HW), dtype=torch.uint8, device="cuda")
