@@ -71,8 +71,11 @@ inline int bn_stats_row_slices(int64_t rows, int64_t CHW) {
 }
 // Row slices of the plane-aligned statistics kernel: one per batch entry, fewer for windows shorter
 // than the kernel's group of rows (so that every lane still sums a whole group).
+// Rows of x a lane of the statistics kernels requests before it consumes the first: a read-only
+// pass needs about twice as many requests in flight as the fire kernels (cold, [8,64,128,32,32]:
+// 68 us with 8 rows, 55 us with 16; [8,128,128,32,32]: 131 / 99 us).
 #ifndef SNNLIF_STATS_ROWS
-#define SNNLIF_STATS_ROWS 8
+#define SNNLIF_STATS_ROWS 16
 #endif
 inline int64_t bn_stats_wave_slices(int64_t T, int64_t B) {
     if (T >= SNNLIF_STATS_ROWS || B > 0x7fffffff / SNNLIF_STATS_ROWS) return B;  // (row counts stay in int)

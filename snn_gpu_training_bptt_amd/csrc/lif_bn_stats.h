@@ -12,9 +12,9 @@
 // One pass over x (4 bytes per neuron-step in fp32), HBM-bound, two kernels:
 //   1. partial sums.  Planes of at least 32 positions: wavefronts are laid over the (batch entry,
 //      channel) planes as in sweep 1 of the batch-norm backward (ceil(HW/64) wavefronts per plane,
-//      all lanes of a wavefront share a channel); a lane adds up its neuron's T values (eight at a
-//      time in the storage type, the groups in double; windows of fewer than eight steps: the values
-//      of several batch entries, so that eight requests are in flight all the same), the wavefront
+//      all lanes of a wavefront share a channel); a lane adds up its neuron's T values (sixteen at
+//      a time in the storage type, the groups in double; windows of fewer than sixteen steps: the
+//      values of several batch entries, so that sixteen requests are in flight all the same), the wavefront
 //      folds the 64 lanes by shuffles and leaves one pair of sums.  Smaller planes (fully
 //      connected shapes): one lane per (channel, position) column of the [T*B, C*HW] matrix, the rows
 //      dealt round-robin to S slices of workgroups; consecutive lanes read consecutive addresses.
@@ -81,7 +81,6 @@ __device__ __forceinline__ Pack<F, V> stats_fill(F value) {
 //   SLICED = true (shorter windows): the rows are dealt round-robin to S = rows / kStatsRows slices
 //       (rows s, s+S, s+2S, ... belong to slice s), so that a lane still has kStatsRows requests in
 //       flight: it sums the values of several batch entries.  `step` = C*HW.
-// (Two forms of the row loop because the general one measures 25 % slower where the first applies.)
 template <typename F, int V, bool SLICED>
 __global__ void __launch_bounds__(kStatsBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_STATS_WAVES)
 bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restrict__ part_dd,

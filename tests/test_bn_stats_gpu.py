@@ -29,12 +29,15 @@ SHAPES = [
     (8, 256, 16),             # fully connected, few channels: many row slices
     (3, 7, 300, 3, 3),        # HW = 9, more columns than one workgroup holds
     (8, 32, 128, 32, 32),     # few channels, many positions
-    (4, 64, 16, 8, 8),        # 4 steps: a lane sums two batch entries' worth (32 row slices)
-    (2, 6, 5, 8, 8),          # 12 rows: one slice, two groups, the second partial
-    (1, 64, 8, 16, 16),       # a single step: eight batch entries per lane
+    (4, 64, 16, 8, 8),        # 4 steps: a lane sums four batch entries' worth (16 row slices)
+    (2, 6, 5, 8, 8),          # 12 rows: one slice, one partial group
+    (1, 64, 8, 16, 16),       # a single step: sixteen batch entries per lane
     (3, 5, 4, 6, 6),          # 15 rows in one slice
-    (6, 64, 8, 8, 8),         # 384 rows in 48 slices of exactly 8
-    (7, 9, 4, 8, 8),          # 63 rows in 7 slices of 9: one whole group and a one-row tail
+    (6, 64, 8, 8, 8),         # 384 rows in 24 slices of exactly 16
+    (7, 9, 4, 8, 8),          # 63 rows in 3 slices of 21: one whole group and a five-row tail
+    (8, 64, 8, 8, 8),         # the headline window: 32 slices, two batch entries per lane
+    (16, 4, 8, 8, 8),         # 16 steps: one slice per batch entry, one whole group
+    (40, 3, 4, 8, 8),         # 40 steps: two whole groups and an eight-row tail per batch entry
 ]
 
 
