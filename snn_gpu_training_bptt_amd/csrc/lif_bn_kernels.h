@@ -264,9 +264,12 @@ __device__ __forceinline__ F wave_sum(F v) {
 // WAVE = true: wavefronts are laid over the (batch entry, channel) planes -- G = ceil(HW/64)
 // wavefronts per plane, the last one partly idle when HW is not a multiple of 64 -- so all lanes of
 // a wavefront share a channel and their sums are folded by shuffles: one pair of floats per
-// wavefront, part_* indexed [plane][chunk] (B*C*G entries).
+// wavefront, part_* indexed [plane][chunk] (B*C*G entries).  NB > 1 (short windows, B a multiple of
+// NB): a lane takes the same position of NB batch entries B/NB apart, so that a read-only sweep whose
+// window gives a lane fewer than sixteen requests keeps that many in flight all the same; the
+// planes then number (B/NB)*C.
 // `far`: [segment][N] boundary potentials in the workspace (TimeWalk::segments_memory only).
-template <typename F, int TW, bool EXACT, bool WAVE, TimeWalk WALK = TimeWalk::window>
+template <typename F, int TW, bool EXACT, bool WAVE, TimeWalk WALK = TimeWalk::window, int NB = 1>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW))
 lif_bn_backward_partial_kernel(const F* __restrict__ x, const F* __restrict__ g,
                                const F* __restrict__ weight, const F* __restrict__ bias,
@@ -280,7 +283,8 @@ lif_bn_backward_partial_kernel(const F* __restrict__ x, const F* __restrict__ g,
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     if (WAVE) {
         const int64_t G = (HW + 63) / 64;
-        const int64_t lanes = (N / HW) * G * 64;  // padded lane space: planes * G wavefronts
+        const int64_t planes = (N / HW) / NB;     // (B/NB) * C
+        const int64_t lanes = planes * G * 64;    // padded lane space: planes * G wavefronts
         for (int64_t pc = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; pc < lanes;
              pc += stride) {
             const int64_t wave = pc >> 6;
@@ -289,16 +293,20 @@ lif_bn_backward_partial_kernel(const F* __restrict__ x, const F* __restrict__ g,
             const int c = static_cast<int>(plane % C);
             F acc_gy = F(0), acc_gyx = F(0);
             if (k < HW) {
-                const int64_t col = plane * HW + k;
                 const F m = mean[c], iv = ivar[c];
                 const F scale = weight[c] * iv;
                 const F b = bias[c];
-                bn_reverse<F, TW, EXACT, WALK>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
-                                               interval, boundary, far, N, col, [&](int, F gy, F xt) {
-                                                   const F xhat = (xt - m) * iv;
-                                                   acc_gy += gy;
-                                                   acc_gyx += gy * xhat;
-                                               });
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    const int64_t col = (plane + j * planes) * HW + k;
+                    bn_reverse<F, TW, EXACT, WALK>(x, g, T, N, col, m, scale, b, alpha, thresh, beta,
+                                                   interval, boundary, far, N, col,
+                                                   [&](int, F gy, F xt) {
+                                                       const F xhat = (xt - m) * iv;
+                                                       acc_gy += gy;
+                                                       acc_gyx += gy * xhat;
+                                                   });
+                }
             }
             acc_gy = wave_sum(acc_gy);
             acc_gyx = wave_sum(acc_gyx);

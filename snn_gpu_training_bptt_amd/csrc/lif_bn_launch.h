@@ -54,6 +54,14 @@ int bn_forward(const F* x, const F* weight, const F* bias, const F* stat, const 
 // wavefront than the plain backward and single-wavefront groups cost them more than they gain.
 constexpr int kBnSmallBlock = 128;
 
+// Longest window for which a lane of the plane-aligned sweep 1 takes two batch entries (2 * T
+// requests per entry: sixteen or more in flight from 4 steps on; windows of 7 steps and more have
+// them on their own).
+#ifndef SNNLIF_BN_PAIRED_MAX_T
+#define SNNLIF_BN_PAIRED_MAX_T 6
+#endif
+constexpr int kBnPairedMaxT = SNNLIF_BN_PAIRED_MAX_T;
+
 // Dynamic LDS of the segmented sweeps: one boundary value per segment and lane.
 template <typename F>
 inline size_t bn_segment_lds_bytes(int64_t T, int threads) {
@@ -90,20 +98,31 @@ int bn_backward_stats_window(const F* x, const F* weight, const F* bias, const F
     // wavefront idle; they keep one lane per neuron and per-neuron partials.
     const bool wave = bn_wave_partials(HW);
     const int64_t G = (HW + 63) / 64;
-    const dim3 grid_partial(wave ? grid_for(B * C * G * 64, threads) : grid_for(N, threads));
+    // windows of at most kBnPairedMaxT steps: a lane of the plane-aligned sweep takes two batch entries
+    constexpr bool can_pair = !segmented && TW <= kBnPairedMaxT;
+    const int64_t nb = (can_pair && wave && B % 2 == 0) ? 2 : 1;
+    const dim3 grid_partial(wave ? grid_for((B / nb) * C * G * 64, threads) : grid_for(N, threads));
     int rc;
-#define SNNLIF_BN_PARTIAL(EXACT_, WAVE_)                                                           \
-    launch_kernel(lif_bn_backward_partial_kernel<F, TW, EXACT_, WAVE_, WALK>, grid_partial, block,  \
-                  lds, stream, x, g, weight, bias, ivar, mean, part_gy, part_gyx, far, Ti, N, C,  \
-                  HW, F(alpha), F(thresh), F(beta), F(interval))
+#define SNNLIF_BN_PARTIAL_NB(EXACT_, WAVE_, NB_)                                                   \
+    launch_kernel(lif_bn_backward_partial_kernel<F, TW, EXACT_, WAVE_, WALK, NB_>, grid_partial,   \
+                  block, lds, stream, x, g, weight, bias, ivar, mean, part_gy, part_gyx, far, Ti,  \
+                  N, C, HW, F(alpha), F(thresh), F(beta), F(interval))
+#define SNNLIF_BN_PARTIAL(EXACT_, WAVE_) SNNLIF_BN_PARTIAL_NB(EXACT_, WAVE_, 1)
     if constexpr (segmented) {
         if (wave) SNNLIF_BN_PARTIAL(false, true); else SNNLIF_BN_PARTIAL(false, false);
     } else if (exact) {
-        if (wave) SNNLIF_BN_PARTIAL(true, true); else SNNLIF_BN_PARTIAL(true, false);
+        if (nb == 2) {
+            if constexpr (can_pair) SNNLIF_BN_PARTIAL_NB(true, true, 2);
+        } else if (wave) {
+            SNNLIF_BN_PARTIAL(true, true);
+        } else {
+            SNNLIF_BN_PARTIAL(true, false);
+        }
     } else if constexpr (can_be_inexact) {
         if (wave) SNNLIF_BN_PARTIAL(false, true); else SNNLIF_BN_PARTIAL(false, false);
     }
 #undef SNNLIF_BN_PARTIAL
+#undef SNNLIF_BN_PARTIAL_NB
     rc = launch_status();
     if (rc != SNNLIF_OK) return rc;
 
@@ -111,7 +130,7 @@ int bn_backward_stats_window(const F* x, const F* weight, const F* bias, const F
     if (wave) {
         launch_kernel(bn_channel_reduce_finalize_kernel<F>, dim3(static_cast<unsigned>(C)),
                       dim3(kReduceBlock), 0, stream, part_gy, part_gyx, weight, grad_weight,
-                      grad_bias, mean_gxhat, mean_gxhatx, B, C, G, count);
+                      grad_bias, mean_gxhat, mean_gxhatx, B / nb, C, G, count);
         return launch_status();
     }
     const int64_t CHW = C * HW;
