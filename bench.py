@@ -73,13 +73,13 @@ WORKLOADS = {
 # "hot": the kernel of the step loop (SNNLIF_KEEP_SPATIAL), "cold": the streamed kernel of the cold leg.
 # bn_fire: the three backward kernels together.
 MEASURED_TRAFFIC = {
-    "cfg2": {"hot": 805281485, "cold": 805271164, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt"},
-    "cfg3": {"hot": 805412747, "cold": 805351835, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg3_f32.txt"},
-    "cfg5": {"hot": 3221242589, "cold": 3221204207, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_f32.txt"},
-    "cfg5_bf16": {"hot": 1610664335, "cold": 1610663823,
+    "cfg2": {"hot": 805282380, "cold": 805272791, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt"},
+    "cfg3": {"hot": 805382795, "cold": 805351821, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg3_f32.txt"},
+    "cfg5": {"hot": 3221239206, "cold": 3221248806, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_f32.txt"},
+    "cfg5_bf16": {"hot": 1610648811, "cold": 1610648468,
                   "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_bf16.txt"},
-    "t96": {"hot": 807132893, "cold": 807131947, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_t96_f32.txt"},
-    "bn_fire": {"hot": 1346503544, "cold": None, "source": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt"},
+    "t96": {"hot": 807131851, "cold": 807130946, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_t96_f32.txt"},
+    "bn_fire": {"hot": 1346499576, "cold": None, "source": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt"},
 }
 HEADLINE = "cfg2"
 METRIC = "LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T=8,B=64,C=128,32x32"
