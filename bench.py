@@ -65,6 +65,8 @@ WORKLOADS = {
     # no configuration of the reference: a 96-step window, the longest range of the backward that
     # still recomputes the whole window in registers (67 239 936 neuron-steps, 257 MiB per tensor)
     "t96": ((96, 4, 171, 32, 32), 0.5, 1.0, "float32"),
+    # ... and a 100-step one, which the backward cuts into 32-step segments (67 174 400 neuron-steps)
+    "t100": ((100, 4, 164, 32, 32), 0.5, 1.0, "float32"),
 }
 # HBM bytes per launch of the backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
 # of this file (each counter scaled by its reading for a plain device copy of the same tensor:
@@ -79,6 +81,7 @@ MEASURED_TRAFFIC = {
     "cfg5_bf16": {"hot": 1610648811, "cold": 1610648468,
                   "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_bf16.txt"},
     "t96": {"hot": 807131851, "cold": 807130946, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_t96_f32.txt"},
+    "t100": {"hot": 1046477051, "cold": 1046477051, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_t100_f32.txt"},
     "bn_fire": {"hot": 1346499576, "cold": None, "source": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt"},
 }
 HEADLINE = "cfg2"

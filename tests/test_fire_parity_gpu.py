@@ -150,6 +150,28 @@ def test_windows_between_64_and_128(cabi, oracle, T, dtype, keep):
             assert_parity(oracle, x, g, outs, alpha=0.3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("T", [33, 34, 39, 57, 63, 65, 66, 71, 95, 97, 105, 127, 129, 159, 160, 161, 191, 193, 250, 1023])
+def test_segmented_windows(cabi, oracle, T, dtype):
+    """Windows cut into 32-step segments, the last one partial: one step into a new segment (33, 65, 97,
+    129, 161, 193), one short of a full one (63, 95, 127, 159, 191, 1023), whole segments only (160), many
+    segments (250, 1023).  A negative threshold makes a wrong spike flag at the start of the window
+    visible.  Even and odd N."""
+    for n_inner, thresh in ((128, THRESH), (77, -0.25)):
+        x32, g32 = make_inputs((T, 2, n_inner), 0.1, 0.9, seed=7000 + T)
+        x, g = x32.to(dtype), g32.to(dtype)
+        xd = x.cuda()
+        gx = torch.empty_like(xd)
+        cabi.fire_bp_into(xd, g.cuda(), gx, 0.3, thresh, BETA, INTERVAL)
+        torch.cuda.synchronize()
+        wide = torch.float64 if dtype == torch.float64 else torch.float32
+        gx_o = oracle.fire_backward(x.to(wide).numpy(), g.to(wide).numpy(), 0.3, thresh, BETA, INTERVAL)
+        if dtype == torch.bfloat16:
+            assert torch.equal(gx.cpu(), torch.from_numpy(gx_o).bfloat16())
+        else:
+            assert np.array_equal(gx.cpu().numpy(), gx_o)
+
+
 @pytest.mark.parametrize("T", [1, 2])
 @pytest.mark.parametrize("n_inner", [4096, 4098, 4097, 8])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
