@@ -38,7 +38,10 @@
 extern "C" {
 #endif
 
-#define SNNLIF_ABI_VERSION 1
+/* 2: cache hints in `dtype`, snnlif_fire_bp_strided, snnlif_bn_stats, snnlif_bn_fire_bp_static and
+ *    SNNLIF_ERR_SCRATCH, the plain batch-norm entry points (snnlif_bn_fp, snnlif_bn_bp and its halves).
+ *    A library of version 1 rejects hinted dtypes with SNNLIF_ERR_DTYPE and lacks those symbols. */
+#define SNNLIF_ABI_VERSION 2
 
 /* Storage types. */
 #define SNNLIF_DTYPE_F32  0 /* float storage, fp32 arithmetic (the reference's training dtype) */
@@ -256,8 +259,7 @@ int snnlif_bn_fire_bp(const void* spatial, const void* weight, const void* bias,
 /*
  * snnlif_bn_fire_bp for callers that can neither allocate device memory nor hand in a workspace: code
  * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
- * counterpart in the reference (whose bn_fire_bp_cuda allocates five temporaries per call,
- * snnlib/cuda/snn_kernel_bp.cu:700, 711-714).  Same arguments, checks, kernels and results (bit for bit)
+ * counterpart in the reference.  Same arguments, checks, kernels and results (bit for bit)
  * as snnlif_bn_fire_bp, minus the workspace: the partial sums live in a fixed device array of
  * SNNLIF_STATIC_SCRATCH_BYTES that the library holds once per GPU.  Shapes for which
  * snnlif_bn_fire_bp_workspace_bytes() exceeds that size return SNNLIF_ERR_SCRATCH and launch nothing
@@ -306,6 +308,59 @@ int snnlif_bn_fire_bp_dist2(const void* spatial, const void* weight, const void*
                             const void* grad_xhat, const void* grad_xhatx, void* grad_spatial,
                             int dtype, int64_t T, int64_t B, int64_t C, int64_t HW, float alpha,
                             float thresh, float beta, float interval, void* stream);
+
+/*
+ * Plain batch norm of a [T, B, C, HW] activation with given per-channel statistics (fp32 or fp64; bf16:
+ * SNNLIF_ERR_UNSUPPORTED); weight, bias, var, mean, ivar are [C].
+ *   scale[c] = weight[c] / sqrt(var[c] + eps);   ivar[c] = scale[c] / weight[c]
+ *   y_bn = (x_bn - mean[c]) * scale[c] + bias[c]
+ * One pass, 8 bytes per element.  Replaces bn_fp_cuda + bn_fp_kernel (snnlib/cuda/snn_kernel_fp.cu:81-150),
+ * bound as snnlib.bn_fp (snnlib/cuda/snn.cpp:30-40).
+ */
+int snnlif_bn_fp(const void* x_bn, const void* weight, const void* bias, const void* var,
+                 const void* mean, void* ivar, void* y_bn, int dtype, int64_t T, int64_t B, int64_t C,
+                 int64_t HW, float eps, void* stream);
+
+/* Bytes of device workspace snnlif_bn_bp and snnlif_bn_bp_dist1 need: two partial sums of the storage
+ * type per wavefront and row slice of the sums pass when HW >= 32, two per column and row slice
+ * otherwise, and two per-channel means.  0 for invalid arguments. */
+size_t snnlif_bn_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);
+
+/*
+ * Plain batch-norm backward with the statistics the forward saved (fp32 or fp64).  With
+ * xhat = (x_bn - mean[c])*ivar[c] and M = T*B*HW:
+ *   grad_bias[c] = sum grad_y;   grad_weight[c] = sum grad_y*xhat
+ *   grad_x_bn = (grad_y*weight[c])*ivar[c]
+ *               - ivar[c]*((xhat*(weight[c]*grad_weight[c]/M)) + weight[c]*grad_bias[c]/M)
+ * Two passes over (x_bn, grad_y) around a per-channel reduction in a fixed order (reproducible
+ * results): 20 bytes per element.  Replaces bn_bp_cuda with bn_bp_wb_kernel and bn_bp_x_kernel
+ * (snnlib/cuda/snn_kernel_bp.cu:176-345), bound as snnlib.bn_bp (snnlib/cuda/snn.cpp:293-304).  `workspace`:
+ * snnlif_bn_bp_workspace_bytes() bytes, 16-byte aligned, private to the call until the stream has run it.
+ */
+int snnlif_bn_bp(const void* x_bn, const void* weight, const void* ivar, const void* mean,
+                 const void* grad_y_bn, void* grad_x_bn, void* grad_weight, void* grad_bias, int dtype,
+                 int64_t T, int64_t B, int64_t C, int64_t HW, void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+/*
+ * The two halves of snnlif_bn_bp for a batch sharded over several GPUs (B is the local batch):
+ * snnlif_bn_bp_dist1 leaves the local parameter gradients and the local means
+ *   mean_gxhat[c] = weight[c]*(sum grad_y)/(T*B*HW),  mean_gxhatx[c] = weight[c]*(sum grad_y*xhat)/(T*B*HW)
+ * (8 bytes per element); snnlif_bn_bp_dist2 forms the input gradient from the two means averaged over
+ * all ranks (12 bytes per element, no workspace).  dist1 followed by dist2 on the same arrays is
+ * snnlif_bn_bp, bit for bit; the all-reduce between them is the caller's.  Replace bn_bp_cuda_dist1 and
+ * bn_bp_cuda_dist2 (snnlib/cuda/snn_kernel_bp.cu:348-425), bound as snnlib.bn_bp_dist1 / bn_bp_dist2
+ * (snnlib/cuda/snn.cpp:317-355).
+ */
+int snnlif_bn_bp_dist1(const void* x_bn, const void* weight, const void* ivar, const void* mean,
+                       const void* grad_y_bn, void* mean_gxhat, void* mean_gxhatx, void* grad_weight,
+                       void* grad_bias, int dtype, int64_t T, int64_t B, int64_t C, int64_t HW,
+                       void* workspace, size_t workspace_bytes, void* stream);
+
+int snnlif_bn_bp_dist2(const void* x_bn, const void* weight, const void* ivar, const void* mean,
+                       const void* grad_y_bn, const void* grad_xhat, const void* grad_xhatx,
+                       void* grad_x_bn, int dtype, int64_t T, int64_t B, int64_t C, int64_t HW,
+                       void* stream);
 
 #ifdef __cplusplus
 }

@@ -43,6 +43,10 @@ def _load():
         getattr(lib, f"lif_oracle_bn_forward_{sfx}").restype = None
         getattr(lib, f"lif_oracle_bn_backward_{sfx}").argtypes = [ptr] * 9 + [i64] * 4 + [f32] * 4
         getattr(lib, f"lif_oracle_bn_backward_{sfx}").restype = None
+        getattr(lib, f"lif_oracle_plain_bn_forward_{sfx}").argtypes = [ptr] * 7 + [i64] * 4 + [f32]
+        getattr(lib, f"lif_oracle_plain_bn_forward_{sfx}").restype = None
+        getattr(lib, f"lif_oracle_plain_bn_backward_{sfx}").argtypes = [ptr] * 8 + [i64] * 4
+        getattr(lib, f"lif_oracle_plain_bn_backward_{sfx}").restype = None
     _lib = lib
     return lib
 
@@ -131,4 +135,30 @@ def bn_fire_backward(x, weight, bias, ivar, mean, grad_spike, alpha, thresh, bet
     fn = getattr(_load(), "lif_oracle_bn_backward_" + _suffix(x))
     fn(_p(x), _p(weight), _p(bias), _p(ivar), _p(mean), _p(g), _p(gx), _p(gw), _p(gb), T, B, C, hw,
        alpha, thresh, beta, interval)
+    return gx, gw, gb
+
+
+def bn_forward(x, weight, bias, var, mean, eps):
+    """Plain batch norm with given statistics: return ``(ivar, y)`` for fp32 or fp64 ``x`` shaped
+    ``[T, B, C, ...]`` (loops of snnlib/cuda/snn_kernel_fp.cu:102-121)."""
+    real = _bn_real(x)
+    x, weight, bias, var, mean = (np.ascontiguousarray(a, dtype=real) for a in (x, weight, bias, var, mean))
+    T, B, C, hw = _bn_dims(x)
+    ivar = np.empty(C, dtype=real)
+    y = np.empty_like(x)
+    fn = getattr(_load(), "lif_oracle_plain_bn_forward_" + _suffix(x))
+    fn(_p(x), _p(weight), _p(bias), _p(var), _p(mean), _p(ivar), _p(y), T, B, C, hw, eps)
+    return ivar, y
+
+
+def bn_backward(x, weight, ivar, mean, grad_y):
+    """Plain batch-norm backward: return ``(grad_x, grad_weight, grad_bias)`` (loops of
+    snnlib/cuda/snn_kernel_bp.cu:202-234, 263-283)."""
+    real = _bn_real(x)
+    x, weight, ivar, mean, g = (np.ascontiguousarray(a, dtype=real) for a in (x, weight, ivar, mean, grad_y))
+    T, B, C, hw = _bn_dims(x)
+    gx = np.empty_like(x)
+    gw, gb = np.empty(C, dtype=real), np.empty(C, dtype=real)
+    fn = getattr(_load(), "lif_oracle_plain_bn_backward_" + _suffix(x))
+    fn(_p(x), _p(weight), _p(ivar), _p(mean), _p(g), _p(gx), _p(gw), _p(gb), T, B, C, hw)
     return gx, gw, gb

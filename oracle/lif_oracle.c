@@ -216,3 +216,93 @@ void lif_oracle_bn_backward_##SUFFIX(const REAL* spatial, const REAL* weight, co
  * the device code do not narrow them).  Sums across positions: one precision up, rounded once. */
 LIF_ORACLE_BN_DEFINE(f32, float, double, sqrtf)
 LIF_ORACLE_BN_DEFINE(f64, double, long double, sqrt)
+
+/*
+ * Plain batch norm (no fire recurrence), fp32 and fp64, following the reference's kernels:
+ *   forward  : snnlib/cuda/snn_kernel_fp.cu:102-121 (bn_fp_kernel: scale = weight / sqrt(var + eps),
+ *              ivar = scale / weight, y = (x - mean) * scale + bias)
+ *   backward : snnlib/cuda/snn_kernel_bp.cu:202-234 (bn_bp_wb_kernel: partial sums per (c,h,w) over b and
+ *              t, t descending, the two mean-type ones divided by T*B), :263-283 (bn_bp_x_kernel),
+ *              driven as in bn_bp_cuda :288-345 (at::mean / at::sum of the partials over the positions
+ *              of a channel: no defined order in the reference; one precision up here, rounded once).
+ * Parity pinning (tests/test_oracle_pinning.py): the forward against torch.nn.functional.batch_norm
+ * with given statistics, the backward against autograd through the training-mode batch norm in
+ * float64 (the textbook formula), and against hand-computed values on a two-channel case.
+ */
+#define LIF_ORACLE_PLAIN_BN_DEFINE(SUFFIX, REAL, WIDE, SQRT) \
+void lif_oracle_plain_bn_forward_##SUFFIX(const REAL* x, const REAL* weight, const REAL* bias,                        \
+                                     const REAL* var, const REAL* mean, REAL* ivar, REAL* y,                          \
+                                     int64_t T, int64_t B, int64_t C, int64_t HW, float eps_bn) {                     \
+    const int64_t CHW = C * HW, step_stride = B * CHW;                                                                \
+    for (int64_t i = 0; i < CHW; i++) {                                                                               \
+        const int64_t c = i / HW;                                                                                     \
+        const REAL m = mean[c];                                                                                       \
+        const REAL scale = weight[c] / SQRT(var[c] + eps_bn);                                                         \
+        const REAL shift = bias[c];                                                                                   \
+        ivar[c] = scale / weight[c];                                                                                  \
+        for (int64_t b = 0; b < B; b++) {                                                                             \
+            for (int64_t t = 0; t < T; t++) {                                                                         \
+                const int64_t at = t * step_stride + b * CHW + i;                                                     \
+                y[at] = (x[at] - m) * scale + shift;                                                                  \
+            }                                                                                                         \
+        }                                                                                                             \
+    }                                                                                                                 \
+}                                                                                                                     \
+                                                                                                                      \
+void lif_oracle_plain_bn_backward_##SUFFIX(const REAL* x, const REAL* weight, const REAL* ivar,                       \
+                                      const REAL* mean, const REAL* grad_y, REAL* grad_x,                             \
+                                      REAL* grad_weight, REAL* grad_bias, int64_t T, int64_t B,                       \
+                                      int64_t C, int64_t HW) {                                                        \
+    const int64_t CHW = C * HW, step_stride = B * CHW;                                                                \
+    REAL* p_xhat = (REAL*)malloc(sizeof(REAL) * (size_t)CHW);                                                         \
+    REAL* p_xhatx = (REAL*)malloc(sizeof(REAL) * (size_t)CHW);                                                        \
+    REAL* p_w = (REAL*)malloc(sizeof(REAL) * (size_t)CHW);                                                            \
+    REAL* p_b = (REAL*)malloc(sizeof(REAL) * (size_t)CHW);                                                            \
+    for (int64_t i = 0; i < CHW; i++) {                                                                               \
+        const int64_t c = i / HW;                                                                                     \
+        const REAL m = mean[c], w = weight[c], iv = ivar[c];                                                          \
+        REAL sum_b = 0, sum_w = 0, sum_xhat = 0, sum_xhatx = 0;                                                       \
+        for (int64_t b = 0; b < B; b++) {                                                                             \
+            for (int64_t t = T - 1; t >= 0; t--) {                                                                    \
+                const int64_t at = t * step_stride + b * CHW + i;                                                     \
+                const REAL gy = grad_y[at];                                                                           \
+                const REAL x_bn = (x[at] - m) * iv;                                                                   \
+                sum_b += gy;                                                                                          \
+                sum_w += gy * x_bn;                                                                                   \
+                sum_xhat += gy * w;                                                                                   \
+                sum_xhatx += gy * w * x_bn;                                                                           \
+            }                                                                                                         \
+        }                                                                                                             \
+        p_b[i] = sum_b;                                                                                               \
+        p_w[i] = sum_w;                                                                                               \
+        p_xhat[i] = sum_xhat / (T * B);                                                                               \
+        p_xhatx[i] = sum_xhatx / (T * B);                                                                             \
+    }                                                                                                                 \
+    for (int64_t c = 0; c < C; c++) {                                                                                 \
+        WIDE acc_b = 0, acc_w = 0, acc_xhat = 0, acc_xhatx = 0;                                                       \
+        for (int64_t k = 0; k < HW; k++) {                                                                            \
+            acc_b += p_b[c * HW + k];                                                                                 \
+            acc_w += p_w[c * HW + k];                                                                                 \
+            acc_xhat += p_xhat[c * HW + k];                                                                           \
+            acc_xhatx += p_xhatx[c * HW + k];                                                                         \
+        }                                                                                                             \
+        grad_bias[c] = (REAL)acc_b;                                                                                   \
+        grad_weight[c] = (REAL)acc_w;                                                                                 \
+        const REAL g_xhat = (REAL)(acc_xhat / (WIDE)HW);                                                              \
+        const REAL g_xhatx = (REAL)(acc_xhatx / (WIDE)HW);                                                            \
+        const REAL m = mean[c], w = weight[c], iv = ivar[c];                                                          \
+        for (int64_t k = 0; k < HW; k++) {                                                                            \
+            const int64_t i = c * HW + k;                                                                             \
+            for (int64_t b = 0; b < B; b++) {                                                                         \
+                for (int64_t t = T - 1; t >= 0; t--) {                                                                \
+                    const int64_t at = t * step_stride + b * CHW + i;                                                 \
+                    grad_x[at] = grad_y[at] * w * iv - iv * ((x[at] - m) * iv * g_xhatx + g_xhat);                    \
+                }                                                                                                     \
+            }                                                                                                         \
+        }                                                                                                             \
+    }                                                                                                                 \
+    free(p_xhat); free(p_xhatx); free(p_w); free(p_b);                                                                \
+}
+
+LIF_ORACLE_PLAIN_BN_DEFINE(f32, float, double, sqrtf)
+LIF_ORACLE_PLAIN_BN_DEFINE(f64, double, long double, sqrt)

@@ -460,6 +460,131 @@ int snnlif_bn_fire_bp_dist2(const void* spatial, const void* weight, const void*
                                       T, B, C, HW, alpha, thresh, beta, interval, st));
 }
 
+// ---- plain batch norm (no fire recurrence) --------------------------------------------------------
+
+int snnlif_bn_fp(const void* x_bn, const void* weight, const void* bias, const void* var,
+                 const void* mean, void* ivar, void* y_bn, int dtype, int64_t T, int64_t B, int64_t C,
+                 int64_t HW, float eps, void* stream) {
+    const TimerScope timer_scope;
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    if (T == 0 || B * C * HW == 0) return SNNLIF_OK;
+    if (!x_bn || !weight || !bias || !var || !mean || !ivar || !y_bn) return SNNLIF_ERR_ARG;
+    const void* ptrs[7] = {x_bn, weight, bias, var, mean, ivar, y_bn};
+    if (!all_aligned(ptrs, 7, es)) return SNNLIF_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_plain_forward_f32(CF(x_bn), CF(weight), CF(bias), CF(var), CF(mean), MF(ivar),
+                                     MF(y_bn), T, B, C, HW, eps, st),
+        snnlif::bn_plain_forward_f64(CD(x_bn), CD(weight), CD(bias), CD(var), CD(mean), MD(ivar),
+                                     MD(y_bn), T, B, C, HW, eps, st));
+}
+
+size_t snnlif_bn_bp_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW) {
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0 || bn_shape_error(T, B, C, HW) != SNNLIF_OK) return 0;
+    if (T == 0 || B * C * HW == 0) return 0;
+    return snnlif::bn_plain_workspace_elems(T, B, C, HW) * es;
+}
+
+// Shared argument checks of the three plain batch-norm backward entry points.
+static int bn_plain_backward_checks(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW,
+                                    const void* const* ptrs, int n, bool needs_workspace,
+                                    const void* workspace, size_t workspace_bytes, size_t* es_out,
+                                    bool* empty) {
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    *es_out = es;
+    *empty = (T == 0 || B * C * HW == 0);
+    if (*empty) return SNNLIF_OK;
+    for (int i = 0; i < n; ++i)
+        if (ptrs[i] == nullptr) return SNNLIF_ERR_ARG;
+    if (!all_aligned(ptrs, n, es)) return SNNLIF_ERR_ALIGN;
+    if (needs_workspace) {
+        const size_t need = snnlif::bn_plain_workspace_elems(T, B, C, HW) * es;
+        if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
+        if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
+    }
+    return SNNLIF_OK;
+}
+
+int snnlif_bn_bp(const void* x_bn, const void* weight, const void* ivar, const void* mean,
+                 const void* grad_y_bn, void* grad_x_bn, void* grad_weight, void* grad_bias, int dtype,
+                 int64_t T, int64_t B, int64_t C, int64_t HW, void* workspace, size_t workspace_bytes,
+                 void* stream) {
+    const TimerScope timer_scope;
+    const void* ptrs[8] = {x_bn, weight, ivar, mean, grad_y_bn, grad_x_bn, grad_weight, grad_bias};
+    size_t es = 0;
+    bool empty = false;
+    const int rc = bn_plain_backward_checks(dtype, T, B, C, HW, ptrs, 8, true, workspace,
+                                            workspace_bytes, &es, &empty);
+    if (rc != SNNLIF_OK || empty) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const OperationTimer whole_operation(st);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_plain_backward_f32(CF(x_bn), CF(weight), CF(ivar), CF(mean), CF(grad_y_bn),
+                                      MF(grad_x_bn), MF(grad_weight), MF(grad_bias), T, B, C, HW,
+                                      MF(workspace), st),
+        snnlif::bn_plain_backward_f64(CD(x_bn), CD(weight), CD(ivar), CD(mean), CD(grad_y_bn),
+                                      MD(grad_x_bn), MD(grad_weight), MD(grad_bias), T, B, C, HW,
+                                      MD(workspace), st));
+}
+
+int snnlif_bn_bp_dist1(const void* x_bn, const void* weight, const void* ivar, const void* mean,
+                       const void* grad_y_bn, void* mean_gxhat, void* mean_gxhatx, void* grad_weight,
+                       void* grad_bias, int dtype, int64_t T, int64_t B, int64_t C, int64_t HW,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+    const TimerScope timer_scope;
+    const void* ptrs[9] = {x_bn, weight, ivar, mean, grad_y_bn, mean_gxhat, mean_gxhatx, grad_weight,
+                           grad_bias};
+    size_t es = 0;
+    bool empty = false;
+    // an empty batch has no statistics to report: the channel arrays are left untouched
+    const int rc = bn_plain_backward_checks(dtype, T, B, C, HW, ptrs, 9, true, workspace,
+                                            workspace_bytes, &es, &empty);
+    if (rc != SNNLIF_OK || empty) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const OperationTimer whole_operation(st);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_plain_backward_stats_f32(CF(x_bn), CF(weight), CF(ivar), CF(mean), CF(grad_y_bn),
+                                            MF(grad_weight), MF(grad_bias), MF(mean_gxhat),
+                                            MF(mean_gxhatx), T, B, C, HW, MF(workspace), st),
+        snnlif::bn_plain_backward_stats_f64(CD(x_bn), CD(weight), CD(ivar), CD(mean), CD(grad_y_bn),
+                                            MD(grad_weight), MD(grad_bias), MD(mean_gxhat),
+                                            MD(mean_gxhatx), T, B, C, HW, MD(workspace), st));
+}
+
+int snnlif_bn_bp_dist2(const void* x_bn, const void* weight, const void* ivar, const void* mean,
+                       const void* grad_y_bn, const void* grad_xhat, const void* grad_xhatx,
+                       void* grad_x_bn, int dtype, int64_t T, int64_t B, int64_t C, int64_t HW,
+                       void* stream) {
+    const TimerScope timer_scope;
+    const void* ptrs[8] = {x_bn, weight, ivar, mean, grad_y_bn, grad_xhat, grad_xhatx, grad_x_bn};
+    size_t es = 0;
+    bool empty = false;
+    const int rc = bn_plain_backward_checks(dtype, T, B, C, HW, ptrs, 8, false, nullptr, 0, &es, &empty);
+    if (rc != SNNLIF_OK || empty) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_plain_backward_input_f32(CF(x_bn), CF(weight), CF(ivar), CF(mean), CF(grad_y_bn),
+                                            CF(grad_xhat), CF(grad_xhatx), MF(grad_x_bn), T, B, C, HW,
+                                            st),
+        snnlif::bn_plain_backward_input_f64(CD(x_bn), CD(weight), CD(ivar), CD(mean), CD(grad_y_bn),
+                                            CD(grad_xhat), CD(grad_xhatx), MD(grad_x_bn), T, B, C, HW,
+                                            st));
+}
+
 #undef SNNLIF_BN_DISPATCH
 #undef CF
 #undef MF

@@ -92,6 +92,35 @@ inline size_t bn_stats_workspace_elems(int64_t T, int64_t B, int64_t C, int64_t 
     return 2 * bn_stats_partial_count(T, B, C, HW);
 }
 
+// Plain batch norm (lif_bn_plain.h).  Rows of the [T*B, C*HW] matrix a lane of the element-wise passes
+// takes at a time, and a lane of the sums pass (x and g: twice as many requests in flight).
+#ifndef SNNLIF_BN_PLAIN_ROWS
+#define SNNLIF_BN_PLAIN_ROWS 8
+#endif
+#ifndef SNNLIF_BN_PLAIN_SUM_ROWS
+#define SNNLIF_BN_PLAIN_SUM_ROWS 8
+#endif
+constexpr int kBnPlainRows = SNNLIF_BN_PLAIN_ROWS;
+constexpr int kBnPlainSumRows = SNNLIF_BN_PLAIN_SUM_ROWS;
+// Row slices of the sums pass: one group of kBnPlainSumRows rows per lane while that leaves few enough
+// partial sums (at most 2^20 pairs; one per wavefront and slice, or one per column and slice), more
+// rows per lane beyond.
+inline int64_t bn_plain_slices(int64_t R, int64_t C, int64_t HW) {
+    const int64_t per_slice = bn_wave_partials(HW) ? C * ((HW + 63) / 64) : C * HW;
+    int64_t s = (R + kBnPlainSumRows - 1) / kBnPlainSumRows;
+    const int64_t most = per_slice > 0 ? (int64_t(1) << 20) / per_slice : 1;
+    if (s > most) s = most;
+    if (s > 4096) s = 4096;
+    if (s < 1) s = 1;
+    return s;
+}
+// Workspace of the plain batch-norm backward in elements of the scalar type: the two partial-sum
+// arrays ([S][C][ceil(HW/64)] each, or [S][C*HW] each) and the two per-channel means.
+inline size_t bn_plain_workspace_elems(int64_t T, int64_t B, int64_t C, int64_t HW) {
+    const int64_t per_slice = bn_wave_partials(HW) ? C * ((HW + 63) / 64) : C * HW;
+    return static_cast<size_t>(2 * bn_plain_slices(T * B, C, HW) * per_slice + 2 * C);
+}
+
 enum class SpatialHint;  // lif_kernels.h
 
 // Per scalar type F (suffix f32 = float, f64 = double):
@@ -104,6 +133,8 @@ enum class SpatialHint;  // lif_kernels.h
 //                        means (what a batch sharded over several GPUs runs before its all-reduce);
 //   bn_backward_input_*  sweep 2: the input gradient from those means (after the all-reduce);
 //   bn_backward_*        the two back to back, the means staged at the end of the workspace.
+//   bn_plain_*           the batch norm without a fire recurrence: forward (var -> ivar, y), the
+//                        backward's sums + channel reduction, its input gradient, and both back to back.
 #define SNNLIF_DECLARE_BN_DTYPE(SUFFIX, F)                                                         \
     int bn_forward_##SUFFIX(const F* x, const F* weight, const F* bias, const F* stat,             \
                             const F* mean, F* ivar, F* spike, bool from_ivar, int64_t T,           \
@@ -127,9 +158,29 @@ enum class SpatialHint;  // lif_kernels.h
                              float thresh, float beta, float interval, F* workspace,               \
                              hipStream_t stream);
 
+#define SNNLIF_DECLARE_BN_PLAIN_DTYPE(SUFFIX, F)                                                   \
+    int bn_plain_forward_##SUFFIX(const F* x, const F* weight, const F* bias, const F* var,        \
+                                  const F* mean, F* ivar, F* y, int64_t T, int64_t B, int64_t C,   \
+                                  int64_t HW, float eps, hipStream_t stream);                      \
+    int bn_plain_backward_stats_##SUFFIX(const F* x, const F* weight, const F* ivar,               \
+                                         const F* mean, const F* g, F* grad_weight, F* grad_bias,  \
+                                         F* mean_gxhat, F* mean_gxhatx, int64_t T, int64_t B,      \
+                                         int64_t C, int64_t HW, F* workspace, hipStream_t stream); \
+    int bn_plain_backward_input_##SUFFIX(const F* x, const F* weight, const F* ivar,               \
+                                         const F* mean, const F* g, const F* mean_gxhat,           \
+                                         const F* mean_gxhatx, F* gx, int64_t T, int64_t B,        \
+                                         int64_t C, int64_t HW, hipStream_t stream);               \
+    int bn_plain_backward_##SUFFIX(const F* x, const F* weight, const F* ivar, const F* mean,      \
+                                   const F* g, F* gx, F* grad_weight, F* grad_bias, int64_t T,     \
+                                   int64_t B, int64_t C, int64_t HW, F* workspace,                 \
+                                   hipStream_t stream);
+
 SNNLIF_DECLARE_BN_DTYPE(f32, float)
 SNNLIF_DECLARE_BN_DTYPE(f64, double)
+SNNLIF_DECLARE_BN_PLAIN_DTYPE(f32, float)
+SNNLIF_DECLARE_BN_PLAIN_DTYPE(f64, double)
 #undef SNNLIF_DECLARE_BN_DTYPE
+#undef SNNLIF_DECLARE_BN_PLAIN_DTYPE
 
 }  // namespace snnlif
 

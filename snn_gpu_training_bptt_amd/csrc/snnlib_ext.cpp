@@ -26,8 +26,8 @@
 //   bn_fire_fc_bp_dist1, bn_fire_conv_bp_dist1                                      snn.cpp:528-550, 687-716
 //
 // Division of labour: the fire recurrences (with or without the batch norm folded in) run on the
-// hand-written kernels behind the C ABI of libsnnlif_gfx950.so (include/snnlib_lif.h); linear,
-// convolution and the plain batch norm stay on PyTorch-ROCm (rocBLAS / MIOpen through ATen) and are
+// hand-written kernels behind the C ABI of libsnnlif_gfx950.so (include/snnlib_lif.h), and so does the
+// plain batch norm; linear and convolution stay on PyTorch-ROCm (rocBLAS / MIOpen through ATen) and are
 // issued once with the time axis folded into the batch, not once per time step as the reference's
 // host loops do (snnlib/cuda/snn_kernel_fp.cu:314-326, 444-447; snnlib/cuda/snn_kernel_bp.cu:1099-1117,
 // 1382-1390).  As in the reference, backward ops receive only what the forward saved (inputs and
@@ -457,41 +457,79 @@ Tensor bn_fire_bp_dist2(Tensor spatial, Tensor weight_bn, Tensor bias_bn, Tensor
     return grad_spatial;
 }
 
-// ---- layers without fire (ATen only) ------------------------------------------------------------
+// ---- plain batch norm (hand-written kernels behind snnlif_bn_fp / snnlif_bn_bp*) -------------------
+
+struct PlainBnOperands {
+    BnDims d;
+    int dtype;  // SNNLIF_DTYPE_F32 or SNNLIF_DTYPE_F64; the per-channel tensors share it
+    Tensor x;
+};
+
+PlainBnOperands plain_bn_operands(const Tensor& x_bn, const char* op) {
+    check_input(x_bn, op, "x_bn");
+    TORCH_CHECK(x_bn.scalar_type() == at::kFloat || x_bn.scalar_type() == at::kDouble, "snnlib.", op,
+                ": only float32 and float64 are supported, got ", x_bn.scalar_type());
+    PlainBnOperands o;
+    o.dtype = x_bn.scalar_type() == at::kFloat ? SNNLIF_DTYPE_F32 : SNNLIF_DTYPE_F64;
+    o.d = bn_dims_of(x_bn, op);
+    o.x = x_bn.contiguous();
+    return o;
+}
+
+// A gradient shaped, typed and placed like the activation, made dense.
+Tensor dense_gradient(const Tensor& g, const Tensor& like, const char* op, const char* name) {
+    check_input(g, op, name);
+    check_like(g, like, op, name);
+    check_same_shape(like, g, op, "x_bn", name);
+    return g.contiguous();
+}
+
+Tensor byte_workspace(size_t bytes, const Tensor& like) {
+    return torch::empty({static_cast<int64_t>(bytes)}, like.options().dtype(at::kByte));
+}
 
 std::vector<Tensor> bn_fp(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor var, Tensor mean,
                           float eps_bn) {
-    check_input(x_bn, "bn_fp", "x_bn");
-    const BnDims d = bn_dims_of(x_bn, "bn_fp");
-    Tensor w = channel_param(weight_bn, x_bn, d.C, "bn_fp", "weight_bn");
-    Tensor b = channel_param(bias_bn, x_bn, d.C, "bn_fp", "bias_bn");
-    Tensor v = channel_param(var, x_bn, d.C, "bn_fp", "var").detach();
-    Tensor m = channel_param(mean, x_bn, d.C, "bn_fp", "mean").detach();
+    const char* op = "bn_fp";
+    const PlainBnOperands o = plain_bn_operands(x_bn, op);
+    Tensor w = channel_param(weight_bn, o.x, o.d.C, op, "weight_bn");
+    Tensor b = channel_param(bias_bn, o.x, o.d.C, op, "bias_bn");
+    Tensor v = channel_param(var, o.x, o.d.C, op, "var");
+    Tensor m = channel_param(mean, o.x, o.d.C, op, "mean");
     const DeviceGuard guard(x_bn.device());
-    // y = (x - mean) * weight / sqrt(var + eps) + bias with the statistics the caller supplies
-    Tensor y = at::batch_norm(fold_time(x_bn), w, b, m, v, /*training=*/false, /*momentum=*/0.0,
-                              eps_bn, /*cudnn_enabled=*/true);
-    return {at::rsqrt(v + eps_bn), reshaped_result(y, x_bn.sizes())};
+    Tensor ivar = torch::empty_like(v, at::MemoryFormat::Contiguous);
+    Tensor y = torch::empty_like(o.x, at::MemoryFormat::Contiguous);
+    check_rc(snnlif_bn_fp(o.x.data_ptr(), w.data_ptr(), b.data_ptr(), v.data_ptr(), m.data_ptr(),
+                          ivar.data_ptr(), y.data_ptr(), o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW, eps_bn,
+                          current_stream()),
+             op);
+    return {ivar, y};
 }
 
 std::vector<Tensor> bn_bp(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor ivar, Tensor mean,
                           IntList dim_bn, Tensor grad_y_bn) {
-    (void)bias_bn;
-    (void)dim_bn;
-    check_input(x_bn, "bn_bp", "x_bn");
-    check_like(grad_y_bn, x_bn, "bn_bp", "grad_y_bn");
-    check_same_shape(x_bn, grad_y_bn, "bn_bp", "x_bn", "grad_y_bn");
-    const BnDims d = bn_dims_of(x_bn, "bn_bp");
-    Tensor w = channel_param(weight_bn, x_bn, d.C, "bn_bp", "weight_bn");
-    Tensor iv = channel_param(ivar, x_bn, d.C, "bn_bp", "ivar");
-    Tensor m = channel_param(mean, x_bn, d.C, "bn_bp", "mean");
+    (void)bias_bn;  // the gradients do not depend on it
+    (void)dim_bn;   // names the reduced axes ((0,1) or (0,1,3,4)); they follow from the shape here
+    const char* op = "bn_bp";
+    const PlainBnOperands o = plain_bn_operands(x_bn, op);
+    Tensor w = channel_param(weight_bn, o.x, o.d.C, op, "weight_bn");
+    Tensor iv = channel_param(ivar, o.x, o.d.C, op, "ivar");
+    Tensor m = channel_param(mean, o.x, o.d.C, op, "mean");
+    Tensor g = dense_gradient(grad_y_bn, x_bn, op, "grad_y_bn");
     const DeviceGuard guard(x_bn.device());
-    // training-mode batch-norm backward with the saved batch statistics
-    auto grads = at::native_batch_norm_backward(
-        fold_time(grad_y_bn.contiguous()), fold_time(x_bn.contiguous()), w,
-        /*running_mean=*/c10::nullopt, /*running_var=*/c10::nullopt, /*save_mean=*/m,
-        /*save_invstd=*/iv, /*train=*/true, /*eps=*/0.0, {true, true, true});
-    return {reshaped_result(std::get<0>(grads), x_bn.sizes()), std::get<1>(grads), std::get<2>(grads)};
+    Tensor grad_x = torch::empty_like(o.x, at::MemoryFormat::Contiguous);
+    // zeros: a tensor without elements leaves the parameter gradients untouched
+    Tensor grad_weight = torch::zeros_like(w, at::MemoryFormat::Contiguous);
+    Tensor grad_bias = torch::zeros_like(w, at::MemoryFormat::Contiguous);
+    const size_t ws_bytes = snnlif_bn_bp_workspace_bytes(o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW);
+    Tensor workspace = byte_workspace(ws_bytes, o.x);
+    check_rc(snnlif_bn_bp(o.x.data_ptr(), w.data_ptr(), iv.data_ptr(), m.data_ptr(), g.data_ptr(),
+                          grad_x.data_ptr(), grad_weight.data_ptr(), grad_bias.data_ptr(), o.dtype,
+                          o.d.T, o.d.B, o.d.C, o.d.HW, ws_bytes ? workspace.data_ptr() : nullptr,
+                          ws_bytes, current_stream()),
+             op);
+    return {grad_x, reshaped_result(grad_weight, weight_bn.sizes()),
+            reshaped_result(grad_bias, weight_bn.sizes())};
 }
 
 // The two halves of bn_bp for a sharded batch (snnlib/cuda/snn_kernel_bp.cu:348-425): local
@@ -501,26 +539,26 @@ std::vector<Tensor> bn_bp_dist1(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, T
     (void)bias_bn;
     (void)dim_bn;
     const char* op = "bn_bp_dist1";
-    check_input(x_bn, op, "x_bn");
-    check_like(grad_y_bn, x_bn, op, "grad_y_bn");
-    check_same_shape(x_bn, grad_y_bn, op, "x_bn", "grad_y_bn");
-    const BnDims d = bn_dims_of(x_bn, op);
-    Tensor w = channel_param(weight_bn, x_bn, d.C, op, "weight_bn");
-    Tensor iv = channel_param(ivar, x_bn, d.C, op, "ivar");
-    Tensor m = channel_param(mean, x_bn, d.C, op, "mean");
+    const PlainBnOperands o = plain_bn_operands(x_bn, op);
+    Tensor w = channel_param(weight_bn, o.x, o.d.C, op, "weight_bn");
+    Tensor iv = channel_param(ivar, o.x, o.d.C, op, "ivar");
+    Tensor m = channel_param(mean, o.x, o.d.C, op, "mean");
+    Tensor g = dense_gradient(grad_y_bn, x_bn, op, "grad_y_bn");
     const DeviceGuard guard(x_bn.device());
-    if (x_bn.numel() == 0) {
-        Tensor z = torch::zeros_like(w);
-        return {z, z.clone(), z.clone(), z.clone()};
-    }
-    // one pass: sum gy and sum gy*(x - mean) per channel, and the parameter gradients from them
-    auto sums = at::batch_norm_backward_reduce(fold_time(grad_y_bn.contiguous()),
-                                               fold_time(x_bn.contiguous()), m, iv, w,
-                                               /*input_g=*/true, /*weight_g=*/true, /*bias_g=*/true);
-    const Tensor& grad_weight = std::get<2>(sums);
-    const Tensor& grad_bias = std::get<3>(sums);
-    const double count = static_cast<double>(d.T) * d.B * d.HW;
-    return {(grad_bias * w) / count, (grad_weight * w) / count, grad_weight, grad_bias};
+    // zeros: an empty local batch contributes nothing to the all-reduce
+    Tensor mean_gxhat = torch::zeros_like(w, at::MemoryFormat::Contiguous);
+    Tensor mean_gxhatx = torch::zeros_like(w, at::MemoryFormat::Contiguous);
+    Tensor grad_weight = torch::zeros_like(w, at::MemoryFormat::Contiguous);
+    Tensor grad_bias = torch::zeros_like(w, at::MemoryFormat::Contiguous);
+    const size_t ws_bytes = snnlif_bn_bp_workspace_bytes(o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW);
+    Tensor workspace = byte_workspace(ws_bytes, o.x);
+    check_rc(snnlif_bn_bp_dist1(o.x.data_ptr(), w.data_ptr(), iv.data_ptr(), m.data_ptr(),
+                                g.data_ptr(), mean_gxhat.data_ptr(), mean_gxhatx.data_ptr(),
+                                grad_weight.data_ptr(), grad_bias.data_ptr(), o.dtype, o.d.T, o.d.B,
+                                o.d.C, o.d.HW, ws_bytes ? workspace.data_ptr() : nullptr, ws_bytes,
+                                current_stream()),
+             op);
+    return {mean_gxhat, mean_gxhatx, grad_weight, grad_bias};
 }
 
 Tensor bn_bp_dist2(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor ivar, Tensor mean,
@@ -528,24 +566,23 @@ Tensor bn_bp_dist2(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor ivar, T
     (void)bias_bn;
     (void)dim_bn;
     const char* op = "bn_bp_dist2";
-    check_input(x_bn, op, "x_bn");
-    check_like(grad_y_bn, x_bn, op, "grad_y_bn");
-    check_same_shape(x_bn, grad_y_bn, op, "x_bn", "grad_y_bn");
-    const BnDims d = bn_dims_of(x_bn, op);
+    const PlainBnOperands o = plain_bn_operands(x_bn, op);
+    Tensor w = channel_param(weight_bn, o.x, o.d.C, op, "weight_bn");
+    Tensor iv = channel_param(ivar, o.x, o.d.C, op, "ivar");
+    Tensor m = channel_param(mean, o.x, o.d.C, op, "mean");
+    Tensor gxhat = channel_param(grad_xhat, o.x, o.d.C, op, "grad_xhat");
+    Tensor gxhatx = channel_param(grad_xhatx, o.x, o.d.C, op, "grad_xhatx");
+    Tensor g = dense_gradient(grad_y_bn, x_bn, op, "grad_y_bn");
     const DeviceGuard guard(x_bn.device());
-    // per-channel vectors shaped to broadcast over [T, B, C, ...]
-    std::vector<int64_t> shape(static_cast<size_t>(x_bn.dim()), 1);
-    shape[2] = d.C;
-    auto per_channel = [&](const Tensor& p, const char* name) {
-        return channel_param(p, x_bn, d.C, op, name).view(shape);
-    };
-    Tensor w = per_channel(weight_bn, "weight_bn"), iv = per_channel(ivar, "ivar");
-    Tensor m = per_channel(mean, "mean");
-    Tensor gxhat = per_channel(grad_xhat, "grad_xhat"), gxhatx = per_channel(grad_xhatx, "grad_xhatx");
-    // grad_x = gy*w*ivar - ivar*(xhat*grad_xhatx + grad_xhat),  xhat = (x - mean)*ivar
-    Tensor xhat = (x_bn - m) * iv;
-    return (grad_y_bn * w) * iv - iv * (xhat * gxhatx + gxhat);
+    Tensor grad_x = torch::empty_like(o.x, at::MemoryFormat::Contiguous);
+    check_rc(snnlif_bn_bp_dist2(o.x.data_ptr(), w.data_ptr(), iv.data_ptr(), m.data_ptr(),
+                                g.data_ptr(), gxhat.data_ptr(), gxhatx.data_ptr(), grad_x.data_ptr(),
+                                o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW, current_stream()),
+             op);
+    return grad_x;
 }
+
+// ---- dense layers without fire (ATen only) --------------------------------------------------------
 
 Tensor fc_fp(Tensor spatial, Tensor weight_fc, Tensor bias_fc) {
     check_input(spatial, "fc_fp", "spatial");

@@ -41,7 +41,13 @@ SYMBOLS = {
     "snnlif_bn_fire_bp_static": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp]),
     "snnlif_bn_fire_bp_dist1": (_int, [_vp] * 10 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp, _sz, _vp]),
     "snnlif_bn_fire_bp_dist2": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _f32, _vp]),
+    "snnlif_bn_fp": (_int, [_vp] * 7 + [_int, _i64, _i64, _i64, _i64, _f32, _vp]),
+    "snnlif_bn_bp_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
+    "snnlif_bn_bp": (_int, [_vp] * 8 + [_int, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "snnlif_bn_bp_dist1": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "snnlif_bn_bp_dist2": (_int, [_vp] * 8 + [_int, _i64, _i64, _i64, _i64, _vp]),
 }
+ABI_VERSION = 2
 
 _lib = None
 
@@ -151,6 +157,13 @@ def _require_workspace(spatial, workspace, need, what):
         raise ValueError(f"workspace is on {workspace.device}, spatial is on {spatial.device}")
     if workspace.numel() < need:
         raise ValueError(f"workspace holds {workspace.numel()} bytes, {what} needs {need}")
+
+
+def _workspace_args(workspace):
+    """(pointer, bytes) of a uint8 workspace tensor; (NULL, 0) for ``None``."""
+    if workspace is None:
+        return None, 0
+    return workspace.data_ptr(), workspace.numel() * workspace.element_size()
 
 
 def time_next_kernel(start_event, stop_event):
@@ -387,3 +400,71 @@ def bn_fire_bp_dist2_into(spatial, weight, bias, ivar, mean, grad_spike, grad_xh
                                         HW, alpha, thresh, beta, interval, _stream_handle(spatial))
     _check(rc, "snnlif_bn_fire_bp_dist2")
     return grad_spatial
+
+
+def bn_fp_into(x_bn, weight, bias, var, mean, ivar, y_bn, eps):
+    """``snnlif_bn_fp`` on fp32 / fp64 device tensors; writes ``ivar`` ([C]) and ``y_bn``."""
+    T, B, C, HW = _bn_dims(x_bn)
+    _require_like(x_bn, y_bn=y_bn)
+    _require_per_channel(x_bn, C, weight=weight, bias=bias, var=var, mean=mean, ivar=ivar)
+    _require_dense_gpu(x_bn, weight, bias, var, mean, ivar, y_bn)
+    rc = load().snnlif_bn_fp(x_bn.data_ptr(), weight.data_ptr(), bias.data_ptr(), var.data_ptr(),
+                             mean.data_ptr(), ivar.data_ptr(), y_bn.data_ptr(), _torch_dtype_code(x_bn),
+                             T, B, C, HW, eps, _stream_handle(x_bn))
+    _check(rc, "snnlif_bn_fp")
+    return ivar, y_bn
+
+
+def bn_bp_workspace_bytes(dtype_code, T, B, C, HW):
+    return int(load().snnlif_bn_bp_workspace_bytes(dtype_code, T, B, C, HW))
+
+
+def bn_bp_into(x_bn, weight, ivar, mean, grad_y, grad_x, grad_weight, grad_bias, workspace):
+    """``snnlif_bn_bp``: the plain batch-norm backward; ``workspace`` is a uint8 device tensor."""
+    T, B, C, HW = _bn_dims(x_bn)
+    _require_like(x_bn, grad_y=grad_y, grad_x=grad_x)
+    _require_per_channel(x_bn, C, weight=weight, ivar=ivar, mean=mean, grad_weight=grad_weight,
+                         grad_bias=grad_bias)
+    _require_workspace(x_bn, workspace, bn_bp_workspace_bytes(_torch_dtype_code(x_bn), T, B, C, HW),
+                       "snnlif_bn_bp")
+    _require_dense_gpu(x_bn, weight, ivar, mean, grad_y, grad_x, grad_weight, grad_bias, workspace)
+    rc = load().snnlif_bn_bp(x_bn.data_ptr(), weight.data_ptr(), ivar.data_ptr(), mean.data_ptr(),
+                             grad_y.data_ptr(), grad_x.data_ptr(), grad_weight.data_ptr(),
+                             grad_bias.data_ptr(), _torch_dtype_code(x_bn), T, B, C, HW,
+                             *_workspace_args(workspace), _stream_handle(x_bn))
+    _check(rc, "snnlif_bn_bp")
+    return grad_x, grad_weight, grad_bias
+
+
+def bn_bp_dist1_into(x_bn, weight, ivar, mean, grad_y, mean_gxhat, mean_gxhatx, grad_weight, grad_bias,
+                     workspace):
+    """``snnlif_bn_bp_dist1``: the half of the plain batch-norm backward before the all-reduce."""
+    T, B, C, HW = _bn_dims(x_bn)
+    _require_like(x_bn, grad_y=grad_y)
+    _require_per_channel(x_bn, C, weight=weight, ivar=ivar, mean=mean, mean_gxhat=mean_gxhat,
+                         mean_gxhatx=mean_gxhatx, grad_weight=grad_weight, grad_bias=grad_bias)
+    _require_workspace(x_bn, workspace, bn_bp_workspace_bytes(_torch_dtype_code(x_bn), T, B, C, HW),
+                       "snnlif_bn_bp_dist1")
+    _require_dense_gpu(x_bn, weight, ivar, mean, grad_y, mean_gxhat, mean_gxhatx, grad_weight, grad_bias,
+                       workspace)
+    rc = load().snnlif_bn_bp_dist1(x_bn.data_ptr(), weight.data_ptr(), ivar.data_ptr(), mean.data_ptr(),
+                                   grad_y.data_ptr(), mean_gxhat.data_ptr(), mean_gxhatx.data_ptr(),
+                                   grad_weight.data_ptr(), grad_bias.data_ptr(), _torch_dtype_code(x_bn),
+                                   T, B, C, HW, *_workspace_args(workspace), _stream_handle(x_bn))
+    _check(rc, "snnlif_bn_bp_dist1")
+    return mean_gxhat, mean_gxhatx, grad_weight, grad_bias
+
+
+def bn_bp_dist2_into(x_bn, weight, ivar, mean, grad_y, grad_xhat, grad_xhatx, grad_x):
+    """``snnlif_bn_bp_dist2``: the half after the all-reduce."""
+    T, B, C, HW = _bn_dims(x_bn)
+    _require_like(x_bn, grad_y=grad_y, grad_x=grad_x)
+    _require_per_channel(x_bn, C, weight=weight, ivar=ivar, mean=mean, grad_xhat=grad_xhat,
+                         grad_xhatx=grad_xhatx)
+    _require_dense_gpu(x_bn, weight, ivar, mean, grad_y, grad_xhat, grad_xhatx, grad_x)
+    rc = load().snnlif_bn_bp_dist2(x_bn.data_ptr(), weight.data_ptr(), ivar.data_ptr(), mean.data_ptr(),
+                                   grad_y.data_ptr(), grad_xhat.data_ptr(), grad_xhatx.data_ptr(),
+                                   grad_x.data_ptr(), _torch_dtype_code(x_bn), T, B, C, HW,
+                                   _stream_handle(x_bn))
+    _check(rc, "snnlif_bn_bp_dist2")
+    return grad_x

@@ -408,3 +408,69 @@ def test_bn_fire_double_precision_loops(shape):
     assert iv32.dtype == np.float32
     np.testing.assert_allclose(iv32, c_oracle.bn_fire_forward(n(x32.double()), n(w.float().double()), n(b.float().double()),
                                                                n(var32.double()), n(mean32.double()), eps, 0.25, 0.5)[0], rtol=1e-6)
+
+
+# ---- plain batch norm (no fire): lif_oracle_plain_bn_* ----------------------------------------------
+
+@pytest.mark.parametrize("shape", [(6, 4, 8, 8, 8), (6, 16, 8), (3, 2, 5, 7), (1, 6, 3, 5)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+def test_plain_bn_loops_match_the_library_batch_norm_and_its_autograd(shape, dtype):
+    """Forward: torch.nn.functional.batch_norm with given statistics (the textbook affine).  Backward:
+    autograd through the training-mode batch norm evaluated in float64, i.e. the statistics as
+    functions of x -- a derivation independent of the reference kernels' formulae."""
+    eps = 1e-5
+    x, g, w, b, var, mean = (t.to(dtype) for t in _bn_case(shape, 50))
+    dims = (0, 1) + tuple(range(3, len(shape)))
+    var, mean = torch.var_mean(x, dim=dims, unbiased=False)
+    n = lambda t: t.numpy()
+    ivar, y = c_oracle.bn_forward(n(x), n(w), n(b), n(var), n(mean), eps)
+    assert ivar.dtype == y.dtype == n(x).dtype
+    fold = lambda t: t.reshape((shape[0] * shape[1],) + tuple(shape[2:]))
+    y_lib = torch.nn.functional.batch_norm(fold(x.double()), mean.double(), var.double(), w.double(), b.double(),
+                                           False, 0.0, float(np.float32(eps)) if dtype == torch.float64 else eps)
+    tol = 1e-5 if dtype == torch.float32 else 1e-12
+    np.testing.assert_allclose(y.reshape(y_lib.shape), n(y_lib), rtol=tol, atol=tol)
+    np.testing.assert_allclose(ivar, 1.0 / np.sqrt(n(var).astype(np.float64) + np.float64(np.float32(eps))), rtol=tol)
+
+    gx, gw, gb = c_oracle.bn_backward(n(x), n(w), ivar, n(mean), n(g))
+    xr = x.double().clone().requires_grad_(True)
+    wr, br = w.double().clone().requires_grad_(True), b.double().clone().requires_grad_(True)
+    out = torch.nn.functional.batch_norm(fold(xr), None, None, wr, br, True, 0.0, float(np.float32(eps)))
+    out.backward(fold(g.double()))
+    scale = lambda a: np.abs(a).max() + 1e-300
+    btol = 2e-5 if dtype == torch.float32 else 1e-11
+    assert np.abs(gx - n(xr.grad)).max() <= btol * scale(gx)
+    assert np.abs(gw - n(wr.grad)).max() <= btol * scale(gw)
+    assert np.abs(gb - n(br.grad)).max() <= btol * scale(gb)
+
+
+def test_plain_bn_loops_on_a_hand_computed_case():
+    """Two channels, dyadic values, everything exact: channel 0 holds x = (1, 3) with g = (1, 0),
+    channel 1 holds x = (0, 4) with g = (2, 2); statistics given, not derived.
+    Channel 0: mean 2, ivar 1, weight 2 -> xhat = (-1, 1); grad_bias 1, grad_weight -1,
+    gxhat = 2*1/2 = 1, gxhatx = 2*(-1)/2 = -1, gx = g*2 - (xhat*(-1) + 1) = (2 - 2, 0 - 0) = (0, 0).
+    Channel 1: mean 2, ivar 0.5, weight 1 -> xhat = (-1, 1); grad_bias 4, grad_weight 0,
+    gxhat = 2, gxhatx = 0, gx = g*0.5 - 0.5*(0 + 2) = (0, 0)."""
+    x = np.array([[[1.0, 0.0]], [[3.0, 4.0]]], np.float32)        # [T=2, B=1, C=2]
+    g = np.array([[[1.0, 2.0]], [[0.0, 2.0]]], np.float32)
+    w = np.array([2.0, 1.0], np.float32)
+    mean = np.array([2.0, 2.0], np.float32)
+    ivar = np.array([1.0, 0.5], np.float32)
+    gx, gw, gb = c_oracle.bn_backward(x, w, ivar, mean, g)
+    assert np.array_equal(gb, np.array([1.0, 4.0], np.float32))
+    assert np.array_equal(gw, np.array([-1.0, 0.0], np.float32))
+    assert np.array_equal(gx, np.zeros_like(x))
+    # a gradient that is not orthogonal to the projections: g' = g + (1, 0) on channel 1's first element
+    g2 = g.copy()
+    g2[0, 0, 1] = 3.0      # channel 1: g = (3, 2): grad_bias 5, grad_weight -3+2 = -1, gxhat 2.5, gxhatx -0.5
+    gx2, gw2, gb2 = c_oracle.bn_backward(x, w, ivar, mean, g2)
+    assert gb2[1] == 5.0 and gw2[1] == -1.0
+    # gx = g*0.5 - 0.5*(xhat*(-0.5) + 2.5) -> (1.5 - 0.5*3.0, 1.0 - 0.5*2.0) = (0.0, 0.0)
+    assert np.array_equal(gx2[:, 0, 1], np.array([0.0, 0.0], np.float32))
+    # forward with var chosen so that var + eps is exactly 4 (scale = weight / 2)
+    eps = np.float32(1e-5)
+    var = np.full(2, np.float32(4.0) - eps, np.float32)
+    assert np.float32(var[0] + eps) == np.float32(4.0)
+    iv, y = c_oracle.bn_forward(x, w, np.array([0.5, -1.0], np.float32), var, mean, float(eps))
+    assert np.array_equal(iv, np.array([0.5, 0.5], np.float32))
+    assert np.array_equal(y, np.array([[[-0.5, -2.0]], [[1.5, 0.0]]], np.float32))
