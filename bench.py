@@ -1,31 +1,44 @@
 #!/usr/bin/env python3
 """Benchmark of the LIF fire forward+backward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg5_bf16|cfg1]
-                    [--no-cpu-baseline]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg5_bf16|cfg1|t96|t100]
+                    [--no-cpu-baseline] [--no-extra-legs]
     python bench.py --workload train_step [--steps K] [--warmup W]     (context figure, see below)
     python bench.py --workload bn_fire    [--steps K] [--warmup W]     (next-row op, see below)
+    python bench.py --workload bn         [--steps K] [--warmup W]     (next-row op, see below)
 
 One "step" is one forward (spikes from the input current) plus one backward (input gradient from
 the saved input current and the spike gradient) over one synthetic batch that is already resident
-in HBM, launched through the C ABI of ``libsnnlif_gfx950.so`` on PyTorch's current stream with
-pre-allocated outputs.  The default workload is the headline configuration
-``T=8, B=64, C=128, 32x32`` fp32.  Exactly one JSON line is printed on stdout.
+in HBM.  The default workload is the headline configuration ``T=8, B=64, C=128, 32x32`` fp32.
+Exactly one JSON line is printed on stdout.
+
+The timed region, and with it ``value``, ``ms_per_step`` and the top level of ``roofline``, is the path
+a user of the reference's interface gets: the step loop calls ``snnlib.fire_s_fp(x, alpha, thresh)`` and
+``snnlib.fire_bp(x, g, alpha, thresh, beta, interval)`` of the pybind module (the two calls of
+``snnlib_func.FireFunc``), outputs come from PyTorch's caching allocator inside the calls, and no cache
+hint is passed (the reference's interface has no way to express one), so tensors of more than 32 MiB run
+the *streamed* kernels.  The loop rotates over several independent (x, g) sets, all forwards of a round
+first, then all backwards, so that several times the capacity of the 256 MB memory-side cache passes
+between a batch's forward and its backward, as the other layers of a network would put there: every
+byte comes from HBM.
 
 * ``value``      neuron-steps per second over the K timed steps (wall clock between two device
                  synchronisations).
-* ``roofline``   the backward kernel (the dominant one): algorithmic bytes per launch
+* ``roofline``   the streamed backward kernel (the dominant one): algorithmic bytes per launch
                  (12 B x neuron-steps in fp32: read x, read grad_spike, write grad_x) divided by its
                  mean duration, measured inside the timed region with HIP events attached to the
                  dispatches (kernel begin / kernel end) of about 25 steps spread evenly over it,
-                 against the 8 TB/s HBM peak.  ``fwd`` and ``fwd_bwd`` give the same figure for the forward kernel (8 B) and for the pair (20 B).
-* ``roofline.cold`` the same kernels with nothing of ``x`` left in the 256 MB memory-side cache when
-                 the backward starts: several independent (x, g, spike, grad_x) sets of the workload's
-                 shape, all forwards first, then all backwards, so that at least three other tensors'
-                 worth of traffic lies between a tensor's forward and its backward (a deep network
-                 puts whole layers there).  Kernel durations from the same attached events.  The
-                 figures outside ``cold`` come from the step loop on one set, where the backward runs
-                 right after the forward and finds part of ``x`` still cached.
+                 against the 8 TB/s HBM peak.  ``fwd`` and ``fwd_bwd`` give the same figure for the
+                 forward kernel (8 B) and for the pair (20 B); ``module`` repeats the leg's wall-clock
+                 figures and compares them with ``cabi_streamed``.
+* ``roofline.cabi_streamed`` the same rotation through the C ABI (ctypes, pre-allocated outputs,
+                 SNNLIF_STREAM_SPATIAL): what the module adds on top of the kernels shows as the difference.
+* ``roofline.same_tensors`` the module again, one tensor set, backward straight after the forward step
+                 after step (the pattern of the reference's test_fire.py): still the streamed kernels.
+* ``roofline.kept`` the C ABI with the SNNLIF_KEEP_SPATIAL hint on one tensor set: the caller declares that
+                 the backward follows the forward on the same input current, ``x`` is loaded with the
+                 default cache policy and stays in the memory-side cache, and the launch shape is the
+                 one that serves cache hits best.  Only a caller of the C ABI can ask for this.
 * ``cpu_baseline`` the pure-PyTorch restatement of the reference's gold path
                  (``oracle/gold_fire.py``) on the host cores, forward + autograd backward on the same
                  inputs, best of 3 after a warm-up; its outputs also serve as the parity check of
@@ -40,6 +53,9 @@ fire kernels, measured with events around the ``snnlib.fire_s_fp`` / ``snnlib.fi
 ``snnlif_bn_fire_s_fp``, ``snnlif_bn_fire_bp``) at the headline shape through the C ABI: 4 B per
 neuron-step for the batch statistics, 8 B forward, 20 B backward (two sweeps over x and the spike
 gradient, one write of the input gradient), checked against the CPU oracle on a sample of channels.
+
+``--workload bn`` does the same for the plain batch norm (``snnlif_bn_stats``, ``snnlif_bn_fp``,
+``snnlif_bn_bp``): 4 + 8 + 20 B per element.
 """
 import argparse
 import json
@@ -70,20 +86,43 @@ WORKLOADS = {
 }
 # HBM bytes per launch of the backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
 # of this file (each counter scaled by its reading for a plain device copy of the same tensor:
-# --copy-calibration).  Counters cannot be read from inside this process, so the figures are kept here
-# with the profile summary they come from; a workload without a profiled figure reports null.
-# "hot": the kernel of the step loop (SNNLIF_KEEP_SPATIAL), "cold": the streamed kernel of the cold leg.
-# bn_fire: the three backward kernels together.
-MEASURED_TRAFFIC = {
-    "cfg2": {"hot": 805282380, "cold": 805272791, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt"},
-    "cfg3": {"hot": 805382795, "cold": 805351821, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg3_f32.txt"},
-    "cfg5": {"hot": 3221239206, "cold": 3221248806, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_f32.txt"},
-    "cfg5_bf16": {"hot": 1610648811, "cold": 1610648468,
-                  "source": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_bf16.txt"},
-    "t96": {"hot": 807131851, "cold": 807130946, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_t96_f32.txt"},
-    "t100": {"hot": 1046477051, "cold": 1046477051, "source": "profiles/pmc_fetch_write_fire_fwd_bwd_t100_f32.txt"},
-    "bn_fire": {"hot": 1346499576, "cold": None, "source": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt"},
+# --copy-calibration).  Counters cannot be read from inside this process, so the figures are read from the
+# tracked profile summary they were written to; a workload without one reports null.
+TRAFFIC_PROFILES = {
+    "cfg2": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg2_f32.txt",
+    "cfg3": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg3_f32.txt",
+    "cfg5": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_f32.txt",
+    "cfg5_bf16": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_bf16.txt",
+    "t96": "profiles/pmc_fetch_write_fire_fwd_bwd_t96_f32.txt",
+    "t100": "profiles/pmc_fetch_write_fire_fwd_bwd_t100_f32.txt",
+    "bn_fire": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt",
+    "bn": "profiles/pmc_fetch_write_bn_fwd_bwd_cfg2_f32.txt",
 }
+
+
+def measured_traffic(workload):
+    """{"source": path, "<pass>, <policy>": bytes, ...} from the "Scaled HBM traffic" table of the
+    workload's PMC summary (lines `  <name> : <bytes> B = ...`), or {} when there is none."""
+    import re
+    rel = TRAFFIC_PROFILES.get(workload)
+    path = os.path.join(REPO, rel) if rel else None
+    if not path or not os.path.exists(path):
+        return {}
+    out = {"source": rel}
+    in_table = False
+    for line in open(path):
+        if line.startswith("Scaled HBM traffic"):
+            in_table = True
+            continue
+        if in_table:
+            m = re.match(r"\s+([^:]+?)\s*:\s*(\d+) B\b", line)
+            if m:
+                out[" ".join(m.group(1).split())] = int(m.group(2))
+            elif line.strip() and not line.startswith(" "):
+                in_table = False
+    return out
+
+
 HEADLINE = "cfg2"
 METRIC = "LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T=8,B=64,C=128,32x32"
 
@@ -127,64 +166,67 @@ def cpu_baseline(torch, x, g, repeats=3):
     return best, threads, outs
 
 
-def cold_cache_leg(torch, lif_cabi, x, g, spike_expected, bytes_fwd, bytes_bwd, rounds=6):
-    """Forward and backward kernel durations when the backward cannot find ``x`` in the memory-side
-    cache: K independent tensor sets, all K forwards, then all K backwards, `rounds` times (after
-    one untimed round).  Between the forward and the backward of one set lie the other sets'
-    forwards and backwards, several times the cache's capacity.  Every dispatch carries its own
-    start/stop events; the wall clock over the timed rounds is reported too."""
-    tensor_bytes = x.numel() * x.element_size()
+def tensor_sets(tensor_bytes):
+    """How many independent tensor sets the rotating legs cycle through: four (two for tensors beyond
+    512 MiB), more for small tensors so that a cycle moves at least 2 GiB of inputs."""
     sets = 4 if tensor_bytes <= (512 << 20) else 2
-    while sets * 2 * tensor_bytes < (2 << 30):      # small tensors: enough sets to cycle 2 GiB
+    while sets * 2 * tensor_bytes < (2 << 30):
         sets *= 2
-    sets = min(sets, 64)
-    xs = [x] + [x.clone() for _ in range(sets - 1)]
-    gs = [g] + [g.clone() for _ in range(sets - 1)]
-    spikes = [torch.empty_like(x) for _ in range(sets)]
-    gxs = [torch.empty_like(x) for _ in range(sets)]
+    return min(sets, 64)
 
-    def one_round(events):
-        for k in range(sets):
-            if events is not None:
-                lif_cabi.time_next_kernel(events[0][k][0], events[0][k][1])
-            lif_cabi.fire_s_fp_into(xs[k], spikes[k], ALPHA, THRESH, keep_spatial=False)
-        for k in range(sets):
-            if events is not None:
-                lif_cabi.time_next_kernel(events[1][k][0], events[1][k][1])
-            lif_cabi.fire_bp_into(xs[k], gs[k], gxs[k], ALPHA, THRESH, BETA, INTERVAL, keep_spatial=False)
 
-    ev = [[[[torch.cuda.Event(enable_timing=True) for _ in range(2)] for _ in range(sets)]
-           for _ in range(2)] for _ in range(rounds)]
-    for per_round in ev:
-        for per_kind in per_round:
-            for pair in per_kind:
-                for e in pair:
-                    e.record()
-    one_round(None)
+def rotation_leg(torch, lif_cabi, sets, steps, warmup, forward, backward, bytes_fwd, bytes_bwd,
+                 neuron_steps, instrumented=25):
+    """K steps over `sets` independent tensor sets in rounds: forward(j) for every set j of the round,
+    then backward(j) for every set, so that between a set's forward and its backward lie the other
+    sets' forwards and backwards, several times the capacity of the memory-side cache.  A round holds
+    `sets` steps (the last one what is left of K).  About `instrumented` steps spread evenly over the
+    timed region carry HIP events on their two dispatches (snnlif_time_next_kernel: kernel begin /
+    kernel end on the launch stream); the other steps are launched as any caller would."""
+    def run(n, events):
+        k = 0
+        while k < n:
+            r = min(sets, n - k)
+            for j in range(r):
+                ev = events.get(k + j) if events else None
+                if ev is not None:
+                    lif_cabi.time_next_kernel(ev[0], ev[1])
+                forward(j)
+            for j in range(r):
+                ev = events.get(k + j) if events else None
+                if ev is not None:
+                    lif_cabi.time_next_kernel(ev[2], ev[3])
+                backward(j)
+            k += r
+        return time.perf_counter()
+
+    run(max(warmup, sets), None)
+    stride = max(1, steps // instrumented)
+    events = {k: [torch.cuda.Event(enable_timing=True) for _ in range(4)] for k in range(0, steps, stride)}
+    for row in events.values():   # create them on the device side before handing out their handles
+        for e in row:
+            e.record()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for r in range(rounds):
-        one_round(ev[r])
+    t_enqueued = run(steps, events)
     torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    fwd = [p[0].elapsed_time(p[1]) for per_round in ev for p in per_round[0]]
-    bwd = [p[0].elapsed_time(p[1]) for per_round in ev for p in per_round[1]]
-    fwd_ms, bwd_ms = sum(fwd) / len(fwd), sum(bwd) / len(bwd)
-    same = all(torch.equal(sp, spike_expected) for sp in spikes) and all(torch.equal(q, gxs[0]) for q in gxs[1:])
+    t1 = time.perf_counter()
+    wall = t1 - t0
+    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events.values()) / len(events)
+    bwd_ms = sum(e[2].elapsed_time(e[3]) for e in events.values()) / len(events)
     rate = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
     return {
-        "what": f"{sets} independent tensor sets, all forwards then all backwards, {rounds} timed rounds after "
-                f"one untimed: {sets * 2 - 1} or more other tensors' traffic between a set's forward and its backward",
-        "sets": sets, "launches_timed": len(fwd),
-        "fwd": {"avg_launch_ms": fwd_ms, "achieved": rate(bytes_fwd, fwd_ms),
-                "frac": rate(bytes_fwd, fwd_ms) / HBM_PEAK_GBPS},
-        "bwd": {"avg_launch_ms": bwd_ms, "achieved": rate(bytes_bwd, bwd_ms),
-                "frac": rate(bytes_bwd, bwd_ms) / HBM_PEAK_GBPS},
-        "fwd_bwd": {"kernel_ms": fwd_ms + bwd_ms, "achieved": rate(bytes_fwd + bytes_bwd, fwd_ms + bwd_ms),
+        "sets": sets, "steps": steps, "launches_timed": len(events),
+        "ms_per_step": wall / steps * 1e3,
+        "host_enqueue_ms_per_step": (t_enqueued - t0) / steps * 1e3,
+        "neuron_steps_per_s": neuron_steps * steps / wall,
+        "fwd": {"kernel": "lif_forward_kernel", "algorithmic_bytes_per_launch": bytes_fwd, "avg_launch_ms": fwd_ms,
+                "achieved": rate(bytes_fwd, fwd_ms), "frac": rate(bytes_fwd, fwd_ms) / HBM_PEAK_GBPS},
+        "bwd": {"algorithmic_bytes_per_launch": bytes_bwd, "avg_launch_ms": bwd_ms,
+                "achieved": rate(bytes_bwd, bwd_ms), "frac": rate(bytes_bwd, bwd_ms) / HBM_PEAK_GBPS},
+        "fwd_bwd": {"algorithmic_bytes": bytes_fwd + bytes_bwd, "kernel_ms": fwd_ms + bwd_ms,
+                    "achieved": rate(bytes_fwd + bytes_bwd, fwd_ms + bwd_ms),
                     "frac": rate(bytes_fwd + bytes_bwd, fwd_ms + bwd_ms) / HBM_PEAK_GBPS},
-        "wall_ms_per_pair": wall / (rounds * sets) * 1e3,
-        "neuron_steps_per_s": x.numel() * rounds * sets / wall,
-        "outputs_equal_across_sets": bool(same),
     }
 
 
@@ -305,7 +347,10 @@ def run_train_step(args):
     }), flush=True)
 
 
-def run_bn_fire(args):
+def run_bn(args, plain):
+    """The training step of a batch-norm layer at the headline shape through the C ABI: batch statistics,
+    forward, backward.  plain = False: batch norm folded into the fire recurrence (snnlif_bn_fire_*);
+    plain = True: the batch norm on its own (snnlif_bn_fp / snnlif_bn_bp)."""
     import numpy as np
     import torch
     from snn_gpu_training_bptt_amd import lif_cabi
@@ -318,6 +363,7 @@ def run_bn_fire(args):
     T, B, C, HW = shape[0], shape[1], shape[2], shape[3] * shape[4]
     ns = T * B * C * HW
     eps = 1e-5
+    name = "bn" if plain else "bn_fire"
     gen = torch.Generator(device=dev).manual_seed(SEED)
     x = 0.5 + torch.randn(shape, generator=gen, device=dev)
     g = torch.randn(shape, generator=gen, device=dev)
@@ -327,22 +373,30 @@ def run_bn_fire(args):
     stats_ws = torch.empty(lif_cabi.bn_stats_workspace_bytes(lif_cabi.DTYPE_F32, T, B, C, HW),
                            dtype=torch.uint8, device=dev)
     lif_cabi.bn_stats_into(x, mean, var, stats_ws)
-    ivar, spike = torch.empty_like(var), torch.empty_like(x)
+    ivar, out = torch.empty_like(var), torch.empty_like(x)
     gx, gw, gb = torch.empty_like(x), torch.empty_like(weight), torch.empty_like(weight)
-    ws = torch.empty(lif_cabi.bn_fire_bp_workspace_bytes(lif_cabi.DTYPE_F32, T, B, C, HW),
-                     dtype=torch.uint8, device=dev)
+    ws_bytes = (lif_cabi.bn_bp_workspace_bytes if plain else lif_cabi.bn_fire_bp_workspace_bytes)(
+        lif_cabi.DTYPE_F32, T, B, C, HW)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
 
-    def stats():
-        lif_cabi.bn_stats_into(x, mean, var, stats_ws)
+    def stats(xk=x):
+        lif_cabi.bn_stats_into(xk, mean, var, stats_ws)
 
-    def fwd():
-        # the backward follows straight on the same tensors: x is worth keeping in the cache
-        lif_cabi.bn_fire_s_fp_into(x, weight, bias, var, mean, ivar, spike, eps, ALPHA, THRESH,
-                                   keep_spatial=True)
+    def fwd(xk=x, outk=out, keep=True):
+        if plain:
+            lif_cabi.bn_fp_into(xk, weight, bias, var, mean, ivar, outk, eps)
+        else:
+            # step loop: the backward follows straight on the same tensors, x is worth keeping in the
+            # cache; cold leg: no hint, as the layer calls it
+            lif_cabi.bn_fire_s_fp_into(xk, weight, bias, var, mean, ivar, outk, eps, ALPHA, THRESH,
+                                       keep_spatial=True if keep else None)
 
-    def bwd():
-        lif_cabi.bn_fire_bp_into(x, weight, bias, ivar, mean, g, gx, gw, gb, ALPHA, THRESH, BETA,
-                                 INTERVAL, ws)
+    def bwd(xk=x, gk=g, gxk=gx):
+        if plain:
+            lif_cabi.bn_bp_into(xk, weight, ivar, mean, gk, gxk, gw, gb, ws)
+        else:
+            lif_cabi.bn_fire_bp_into(xk, weight, bias, ivar, mean, gk, gxk, gw, gb, ALPHA, THRESH, BETA,
+                                     INTERVAL, ws)
 
     for _ in range(args.warmup):
         stats()
@@ -374,35 +428,47 @@ def run_bn_fire(args):
     fwd_ms = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
     bwd_ms = sum(e[2].elapsed_time(e[3]) for e in ev) / args.steps
 
+    traffic = measured_traffic(name)
+    bwd_traffic = [v for k, v in traffic.items() if k.startswith("backward")]
+    rate = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
+    if plain:
+        title = "Bn statistics+fwd+bwd elements/s (next-row op, not the headline metric)"
+        what = f"bn: plain batch norm fwd+bwd, [T,B,C,H,W]={list(shape)} float32, batch statistics, eps={eps}"
+        kernels = "bn_plain_sums_wave_kernel + bn_channel_reduce_finalize_kernel + bn_plain_input_kernel"
+        fwd_kernel = "bn_plain_forward_kernel"
+    else:
+        title = "BnFire statistics+fwd+bwd neuron-steps/s (next-row op, not the headline metric)"
+        what = (f"bn_fire: batch-norm + LIF fire fwd+bwd, [T,B,C,H,W]={list(shape)} float32, batch statistics, "
+                f"eps={eps}, alpha={ALPHA} thresh={THRESH} beta={BETA} interval={INTERVAL}")
+        kernels = "lif_bn_backward_partial_kernel + bn_channel_reduce/finalize + lif_bn_backward_input_kernel"
+        fwd_kernel = "lif_bn_forward_kernel"
     result = {
-        "metric": "BnFire statistics+fwd+bwd neuron-steps/s (next-row op, not the headline metric)",
-        "value": ns * args.steps / wall, "unit": "neuron-steps/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3, "higher_is_better": True,
-        "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"bn_fire: batch-norm + LIF fire fwd+bwd, [T,B,C,H,W]={list(shape)} float32, "
-                               f"batch statistics, eps={eps}, alpha={ALPHA} thresh={THRESH} beta={BETA} interval={INTERVAL}"},
-        "roofline": {"kernel": "lif_bn_backward_partial_kernel + bn_channel_reduce/finalize + lif_bn_backward_input_kernel",
+        "metric": title,
+        "value": ns * args.steps / wall, "unit": "elements/s" if plain else "neuron-steps/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall / args.steps * 1e3,
+        "higher_is_better": True, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": what},
+        "roofline": {"kernel": kernels,
+                     "policy": "step loop on one tensor set (statistics, forward, backward back to back)",
                      "bound": "hbm", "algorithmic_bytes_per_launch": 20 * ns, "avg_launch_ms": bwd_ms,
-                     "achieved": 20 * ns / (bwd_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": 20 * ns / (bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS,
-                     "traffic": MEASURED_TRAFFIC["bn_fire"]["hot"],
-                     "traffic_source": MEASURED_TRAFFIC["bn_fire"]["source"],
-                     "fwd": {"algorithmic_bytes_per_launch": 8 * ns, "avg_launch_ms": fwd_ms,
-                             "achieved": 8 * ns / (fwd_ms * 1e-3) / 1e9,
-                             "frac": 8 * ns / (fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS},
+                     "achieved": rate(20 * ns, bwd_ms), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": rate(20 * ns, bwd_ms) / HBM_PEAK_GBPS,
+                     "traffic": sum(bwd_traffic) if bwd_traffic else None,
+                     "traffic_source": traffic.get("source"),
+                     "fwd": {"kernel": fwd_kernel, "algorithmic_bytes_per_launch": 8 * ns, "avg_launch_ms": fwd_ms,
+                             "achieved": rate(8 * ns, fwd_ms), "frac": rate(8 * ns, fwd_ms) / HBM_PEAK_GBPS},
                      "stats": {"kernel": "bn_stats_wave_kernel + bn_stats_finalize_kernel",
                                "algorithmic_bytes_per_launch": 4 * ns, "avg_launch_ms": stats_ms,
-                               "achieved": 4 * ns / (stats_ms * 1e-3) / 1e9,
-                               "frac": 4 * ns / (stats_ms * 1e-3) / 1e9 / HBM_PEAK_GBPS}},
+                               "achieved": rate(4 * ns, stats_ms), "frac": rate(4 * ns, stats_ms) / HBM_PEAK_GBPS}},
     }
-    if not args.no_cold_leg:
+    if not args.no_extra_legs:
         # the layer with nothing cached between its forward and its backward: four tensor sets, all
         # (statistics + forward), then all backwards; events bracket each operation (for the
         # statistics and the backward: all of their kernels, dispatch gaps included)
         sets, rounds = 4, 5
         xs = [x] + [x.clone() for _ in range(sets - 1)]
         gs = [g] + [g.clone() for _ in range(sets - 1)]
-        spikes = [torch.empty_like(x) for _ in range(sets)]
+        outs = [torch.empty_like(x) for _ in range(sets)]
         gxs = [torch.empty_like(x) for _ in range(sets)]
         cev = [[[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(sets)] for _ in range(rounds + 1)]
         for per_round in cev:
@@ -414,29 +480,30 @@ def run_bn_fire(args):
             for k in range(sets):
                 e = cev[r][k]
                 lif_cabi.time_next_kernel(e[0], e[1])
-                lif_cabi.bn_stats_into(xs[k], mean, var, stats_ws)
+                stats(xs[k])
                 lif_cabi.time_next_kernel(e[2], e[3])
-                lif_cabi.bn_fire_s_fp_into(xs[k], weight, bias, var, mean, ivar, spikes[k], eps, ALPHA, THRESH)
+                fwd(xs[k], outs[k], keep=False)
             for k in range(sets):
                 e = cev[r][k]
                 lif_cabi.time_next_kernel(e[4], e[5])
-                lif_cabi.bn_fire_bp_into(xs[k], weight, bias, ivar, mean, gs[k], gxs[k], gw, gb, ALPHA, THRESH, BETA,
-                                         INTERVAL, ws)
+                bwd(xs[k], gs[k], gxs[k])
         torch.cuda.synchronize()
         timed = [e for per_round in cev[1:] for e in per_round]
         avg = lambda a, b: sum(e[a].elapsed_time(e[b]) for e in timed) / len(timed)
         cs, cf, cb = avg(0, 1), avg(2, 3), avg(4, 5)
-        rate = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
         result["roofline"]["cold"] = {
             "what": f"{sets} independent tensor sets, all (statistics + forward) then all backwards, {rounds} timed "
                     "rounds after one untimed; events bracket each operation",
+            "policy": "no hint, as the layer calls the ops; every byte of the backward from HBM",
             "stats": {"avg_ms": cs, "achieved": rate(4 * ns, cs), "frac": rate(4 * ns, cs) / HBM_PEAK_GBPS},
             "fwd": {"avg_ms": cf, "achieved": rate(8 * ns, cf), "frac": rate(8 * ns, cf) / HBM_PEAK_GBPS},
+            "stats_fwd": {"avg_ms": cs + cf, "achieved": rate(12 * ns, cs + cf),
+                          "frac": rate(12 * ns, cs + cf) / HBM_PEAK_GBPS},
             "bwd": {"avg_ms": cb, "achieved": rate(20 * ns, cb), "frac": rate(20 * ns, cb) / HBM_PEAK_GBPS},
-            "outputs_equal_across_sets": bool(all(torch.equal(sp, spikes[0]) for sp in spikes[1:])
+            "outputs_equal_across_sets": bool(all(torch.equal(o, outs[0]) for o in outs[1:])
                                               and all(torch.equal(q, gxs[0]) for q in gxs[1:])),
         }
-        del xs, gs, spikes, gxs
+        del xs, gs, outs, gxs
 
     if not args.no_cpu_baseline:
         # CPU leg: the scalar C loops of the oracle on a bounded sample (channels are independent given
@@ -448,16 +515,22 @@ def run_bn_fire(args):
         p = lambda t: t[pick].cpu().numpy()
         xs, gs = take(x), take(g)
         t0 = time.perf_counter()
-        ivar_o, _, spike_o = c_oracle.bn_fire_forward(xs, p(weight), p(bias), p(var), p(mean), eps, ALPHA, THRESH)
-        t1 = time.perf_counter()
-        c_oracle.bn_fire_backward(xs, p(weight), p(bias), ivar_o, p(mean), gs, ALPHA, THRESH, BETA, INTERVAL)
+        if plain:
+            ivar_o, out_o = c_oracle.bn_forward(xs, p(weight), p(bias), p(var), p(mean), eps)
+            t1 = time.perf_counter()
+            c_oracle.bn_backward(xs, p(weight), ivar_o, p(mean), gs)
+        else:
+            ivar_o, _, out_o = c_oracle.bn_fire_forward(xs, p(weight), p(bias), p(var), p(mean), eps, ALPHA, THRESH)
+            t1 = time.perf_counter()
+            c_oracle.bn_fire_backward(xs, p(weight), p(bias), ivar_o, p(mean), gs, ALPHA, THRESH, BETA, INTERVAL)
         t2 = time.perf_counter()
         result["cpu_baseline"] = {
-            "value": xs.size / (t2 - t0), "unit": "neuron-steps/s", "cores": 1, "kind": "port",
-            "sample": f"channels {pick} of batch entries [0, 8) ({xs.size} neuron-steps), forward + backward of "
+            "value": xs.size / (t2 - t0), "unit": result["unit"], "cores": 1, "kind": "port",
+            "sample": f"channels {pick} of batch entries [0, 8) ({xs.size} elements), forward + backward of "
                       "oracle/lif_oracle.c (scalar C loops), single run",
             "fwd_s": t1 - t0, "bwd_s": t2 - t1}
-        result["parity"] = {"sampled_spikes_bit_exact": bool(np.array_equal(take(spike), spike_o)),
+        result["parity"] = {("sampled_output_bit_exact" if plain else "sampled_spikes_bit_exact"):
+                            bool(np.array_equal(take(out), out_o)),
                             "sampled_ivar_bit_exact": bool(np.array_equal(p(ivar), ivar_o))}
     print(json.dumps(result), flush=True)
 
@@ -467,10 +540,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step", "bn_fire"])
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step", "bn_fire", "bn"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-cold-leg", action="store_true",
-                    help="skip the cold-cache leg (roofline.cold)")
+    ap.add_argument("--no-extra-legs", "--no-cold-leg", dest="no_extra_legs", action="store_true",
+                    help="run the timed region only (fire workloads: no cabi_streamed / same_tensors / kept "
+                         "blocks; bn_fire, bn: no cold-cache leg)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain device copies of the input tensor (known size: one "
                          "read + one write of it) so that rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE "
@@ -488,15 +562,17 @@ def main():
             args.warmup = 3
         return run_train_step(args)
 
-    if args.workload == "bn_fire":
-        return run_bn_fire(args)
+    if args.workload in ("bn_fire", "bn"):
+        return run_bn(args, plain=args.workload == "bn")
 
     import torch
     from snn_gpu_training_bptt_amd import lif_cabi
+    from snn_gpu_training_bptt_amd._loader import load_snnlib
 
     if not torch.cuda.is_available():
         sys.exit("bench.py: no ROCm GPU visible")
-    lif_cabi.load()  # raises if the HIP library has not been built
+    lif_cabi.load()          # raises if the HIP library has not been built
+    snnlib = load_snnlib()   # the pybind module the reference's autograd functions call; raises likewise
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
@@ -509,25 +585,14 @@ def main():
     esize = torch.empty((), dtype=dtype).element_size()
     bytes_fwd = 2 * esize * n_steps_total
     bytes_bwd = 3 * esize * n_steps_total
+    traffic = measured_traffic(args.workload)
 
     x_cpu, g_cpu = make_inputs(torch, shape, mean, std, dtype)
     x = x_cpu.to(dev)
     g = g_cpu.to(dev)
-    spike = torch.empty_like(x)
-    gx = torch.empty_like(x)
-    code = {torch.float32: lif_cabi.DTYPE_F32, torch.bfloat16: lif_cabi.DTYPE_BF16}[dtype]
-    ws_bytes = lif_cabi.fire_bp_workspace_bytes(code, T, n_steps_total // T)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
-
-    # The step loop runs the backward straight after the forward on the same input current, step after
-    # step, and says so (SNNLIF_KEEP_SPATIAL); the cold leg below makes no such promise.
-    def step():
-        lif_cabi.fire_s_fp_into(x, spike, ALPHA, THRESH, keep_spatial=True)
-        lif_cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws, keep_spatial=True)
-
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
+    sets = tensor_sets(x.numel() * esize)
+    xs = [x] + [x.clone() for _ in range(sets - 1)]
+    gs = [g] + [g.clone() for _ in range(sets - 1)]
 
     if args.copy_calibration:
         scratch_copy = torch.empty_like(x)
@@ -536,56 +601,37 @@ def main():
         torch.cuda.synchronize()
         del scratch_copy
 
-    # Timed region: K steps.  HIP events attached to the dispatches themselves
-    # (snnlif_time_next_kernel) give each kernel's own duration on the launch stream -- start when the
-    # kernel begins, stop when it has finished -- which is what rocprofv3 --kernel-trace reports.
-    # (Markers recorded between the launches would add ~10 us of dispatch gap to every interval and
-    # ~13 us of stream work to every step.)  A dispatch that carries events costs ~5 us of stream time
-    # itself, so only every `stride`-th step of the timed region is instrumented (about 25 steps in all,
-    # spread evenly); the other steps are launched exactly as a caller would launch them.
-    stride = max(1, args.steps // 25)
-    timed_steps = list(range(0, args.steps, stride))
-    kev = {k: [torch.cuda.Event(enable_timing=True) for _ in range(4)] for k in timed_steps}
-    for row in kev.values():   # create them on the device side before handing out their handles
-        for e in row:
-            e.record()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for k in range(args.steps):
-        ev = kev.get(k)
-        if ev is not None:
-            lif_cabi.time_next_kernel(ev[0], ev[1])
-        lif_cabi.fire_s_fp_into(x, spike, ALPHA, THRESH, keep_spatial=True)
-        if ev is not None:
-            lif_cabi.time_next_kernel(ev[2], ev[3])
-        lif_cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws, keep_spatial=True)
-    t_enqueued = time.perf_counter()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
+    # ---- the timed region: the module's two calls, rotating over the tensor sets ----
+    # The outputs of a round stay referenced until the next round replaces them (a network keeps a
+    # layer's spikes for the next layer), so the allocator hands out distinct blocks within a round.
+    spikes, gxs = [None] * sets, [None] * sets
 
-    wall = t1 - t0
-    ms_per_step = wall / args.steps * 1e3
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in kev.values()) / len(kev)
-    bwd_ms = sum(e[2].elapsed_time(e[3]) for e in kev.values()) / len(kev)
-    value = n_steps_total * args.steps / wall
+    def module_forward(j):
+        spikes[j] = snnlib.fire_s_fp(xs[j], ALPHA, THRESH)
 
-    def gbps(nbytes, ms):
-        return nbytes / (ms * 1e-3) / 1e9
+    def module_backward(j):
+        gxs[j] = snnlib.fire_bp(xs[j], gs[j], ALPHA, THRESH, BETA, INTERVAL)
 
-    bwd_gbps = gbps(bytes_bwd, bwd_ms)
-    fwd_gbps = gbps(bytes_fwd, fwd_ms)
-    pair_gbps = gbps(bytes_fwd + bytes_bwd, fwd_ms + bwd_ms)
+    head = rotation_leg(torch, lif_cabi, sets, args.steps, args.warmup, module_forward, module_backward,
+                        bytes_fwd, bytes_bwd, n_steps_total)
+    spike, gx = spikes[0], gxs[0]
+    same_across_sets = all(torch.equal(sp, spike) for sp in spikes[1:] if sp is not None) and \
+        all(torch.equal(q, gx) for q in gxs[1:] if q is not None)
+    spikes, gxs = [spike], [gx]   # release the other sets' outputs
     spike_rate = float(spike.float().mean().item())
+    segmented = T > lif_cabi.BP_FUSED_MAX_T and not (T % 8 == 0 and T <= 104)
+    bwd_kernel = ("lif_backward_stream_kernel" if T > lif_cabi.BP_NO_WORKSPACE_MAX_T
+                  else "lif_backward_segmented_kernel" if segmented else "lif_backward_fused_kernel")
 
     result = {
         "metric": metric_name(args.workload, shape, dtype_name),
-        "value": value,
+        "value": head["neuron_steps_per_s"],
         "unit": "neuron-steps/s",
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": ms_per_step,
-        "host_enqueue_ms_per_step": (t_enqueued - t0) / args.steps * 1e3,
+        "ms_per_step": head["ms_per_step"],
+        "host_enqueue_ms_per_step": head["host_enqueue_ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -597,32 +643,91 @@ def main():
                         f"beta={BETA} interval={INTERVAL}",
             "neuron_steps_per_step": n_steps_total,
             "spike_rate": round(spike_rate, 4),
+            "path": "snnlib.fire_s_fp + snnlib.fire_bp (pybind module, outputs from the caching allocator, "
+                    f"no cache hint), {sets} tensor sets in rotation: all forwards of a round, then all backwards",
         },
         "roofline": {
-            "kernel": "lif_backward_fused_kernel" if ws is None else "lif_backward_stream_kernel",
+            "kernel": bwd_kernel,
+            "policy": "streamed (no hint: what the module launches for tensors beyond 32 MiB; every byte from HBM)"
+                      if x.numel() * esize > (32 << 20) else "kept (no hint: tensors of at most 32 MiB)",
             "bound": "hbm",
-            "achieved": bwd_gbps,
+            "achieved": head["bwd"]["achieved"],
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
-            "frac": bwd_gbps / HBM_PEAK_GBPS,
-            "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("hot"),
-            "traffic_source": MEASURED_TRAFFIC.get(args.workload, {}).get("source"),
+            "frac": head["bwd"]["frac"],
+            "traffic": traffic.get("backward, streamed"),
+            "traffic_source": traffic.get("source"),
             "algorithmic_bytes_per_launch": bytes_bwd,
-            "avg_launch_ms": bwd_ms,
-            "timing": f"HIP events attached to the dispatches (kernel begin / kernel end) of {len(kev)} of the "
-                      f"{args.steps} steps inside the timed region (one step in {stride})",
-            "fwd": {"kernel": "lif_forward_kernel", "algorithmic_bytes_per_launch": bytes_fwd,
-                    "avg_launch_ms": fwd_ms,
-                    "achieved": fwd_gbps, "frac": fwd_gbps / HBM_PEAK_GBPS},
-            "fwd_bwd": {"algorithmic_bytes": bytes_fwd + bytes_bwd, "kernel_ms": fwd_ms + bwd_ms,
-                        "achieved": pair_gbps, "frac": pair_gbps / HBM_PEAK_GBPS},
+            "avg_launch_ms": head["bwd"]["avg_launch_ms"],
+            "timing": f"HIP events attached to the dispatches (kernel begin / kernel end) of {head['launches_timed']} "
+                      f"of the {args.steps} steps inside the timed region",
+            "fwd": head["fwd"],
+            "fwd_bwd": head["fwd_bwd"],
+            "module": {"policy": "streamed", "ms_per_step": head["ms_per_step"],
+                       "host_enqueue_ms_per_step": head["host_enqueue_ms_per_step"],
+                       "kernel_ms_per_step": head["fwd_bwd"]["kernel_ms"],
+                       "neuron_steps_per_s": head["neuron_steps_per_s"],
+                       "outputs_equal_across_sets": bool(same_across_sets)},
         },
     }
 
-    if not args.no_cold_leg:
-        cold = cold_cache_leg(torch, lif_cabi, x, g, spike, bytes_fwd, bytes_bwd)
-        cold["bwd"]["traffic"] = MEASURED_TRAFFIC.get(args.workload, {}).get("cold")
-        result["roofline"]["cold"] = cold
+    if not args.no_extra_legs:
+        code = {torch.float32: lif_cabi.DTYPE_F32, torch.bfloat16: lif_cabi.DTYPE_BF16}[dtype]
+        ws_bytes = lif_cabi.fire_bp_workspace_bytes(code, T, n_steps_total // T)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+        extra_steps = min(args.steps, 100)
+
+        # the same rotation through the C ABI: pre-allocated outputs, the streamed kernels asked for by name
+        c_spikes = [torch.empty_like(x) for _ in range(sets)]
+        c_gxs = [torch.empty_like(x) for _ in range(sets)]
+        cabi = rotation_leg(
+            torch, lif_cabi, sets, extra_steps, sets,
+            lambda j: lif_cabi.fire_s_fp_into(xs[j], c_spikes[j], ALPHA, THRESH, keep_spatial=False),
+            lambda j: lif_cabi.fire_bp_into(xs[j], gs[j], c_gxs[j], ALPHA, THRESH, BETA, INTERVAL, workspace=ws,
+                                            keep_spatial=False),
+            bytes_fwd, bytes_bwd, n_steps_total)
+        cabi["policy"] = "streamed (SNNLIF_STREAM_SPATIAL), C ABI through ctypes, pre-allocated outputs"
+        cabi["outputs_equal_to_module"] = bool(torch.equal(c_spikes[0], spike) and torch.equal(c_gxs[0], gx))
+        cabi["bwd"]["traffic"] = traffic.get("backward, streamed")
+        del c_spikes, c_gxs
+        result["roofline"]["cabi_streamed"] = cabi
+        result["roofline"]["module"]["wall_vs_cabi_streamed"] = head["ms_per_step"] / cabi["ms_per_step"]
+        result["roofline"]["module"]["kernels_vs_cabi_streamed"] = \
+            head["fwd_bwd"]["kernel_ms"] / cabi["fwd_bwd"]["kernel_ms"]
+
+        # the module on one tensor set, backward straight after the forward, step after step
+        one = {}
+
+        def same_forward(j):
+            one["spike"] = snnlib.fire_s_fp(x, ALPHA, THRESH)
+
+        def same_backward(j):
+            one["gx"] = snnlib.fire_bp(x, g, ALPHA, THRESH, BETA, INTERVAL)
+
+        same = rotation_leg(torch, lif_cabi, 1, extra_steps, 5, same_forward, same_backward, bytes_fwd,
+                            bytes_bwd, n_steps_total)
+        same["policy"] = ("streamed kernels (no hint), one tensor set: the backward runs straight after the "
+                          "forward on the same input current, step after step")
+        one.clear()
+        result["roofline"]["same_tensors"] = same
+
+        # the C ABI with the caller's promise that x is read again soon
+        k_spike, k_gx = torch.empty_like(x), torch.empty_like(x)
+        kept = rotation_leg(
+            torch, lif_cabi, 1, extra_steps, 5,
+            lambda j: lif_cabi.fire_s_fp_into(x, k_spike, ALPHA, THRESH, keep_spatial=True),
+            lambda j: lif_cabi.fire_bp_into(x, g, k_gx, ALPHA, THRESH, BETA, INTERVAL, workspace=ws,
+                                            keep_spatial=True),
+            bytes_fwd, bytes_bwd, n_steps_total)
+        kept["policy"] = ("kept (SNNLIF_KEEP_SPATIAL), C ABI through ctypes, one tensor set, backward straight after "
+                          "the forward: x stays in the 256 MB memory-side cache, so part of the bytes never "
+                          "come from HBM; not reachable through the reference's interface")
+        kept["outputs_equal_to_module"] = bool(torch.equal(k_spike, spike) and torch.equal(k_gx, gx))
+        kept["bwd"]["traffic"] = traffic.get("backward, kept")
+        del k_spike, k_gx
+        result["roofline"]["kept"] = kept
+
+    del xs, gs
 
     if not args.no_cpu_baseline:
         best, threads, (s_ref, gx_ref) = cpu_baseline(torch, x_cpu, g_cpu)
@@ -654,6 +759,7 @@ def main():
                            "sample": f"batch entries [0, {b8}) of the same tensor, best of 2"},
         }
         result["parity"] = {
+            "what": "outputs of the timed region (module path, set 0) against the CPU gold path",
             "spikes_bit_exact": bool(torch.equal(s_gpu, s_ref)),
             "spike_mismatches": int((s_gpu != s_ref).sum().item()),
             "grad_bit_exact": bool(torch.equal(gx_gpu, gx_ref_cmp)),
