@@ -93,9 +93,12 @@ inline size_t bn_stats_workspace_elems(int64_t T, int64_t B, int64_t C, int64_t 
 }
 
 // Plain batch norm (lif_bn_plain.h).  Rows of the [T*B, C*HW] matrix a lane of the element-wise passes
-// takes at a time, and a lane of the sums pass (x and g: twice as many requests in flight).
+// takes at a time, and a lane of the sums pass (x and g: twice as many requests in flight).  Measured
+// at [8,64,128,32,32] fp32 with 16-byte lanes, input-gradient kernel: 2 rows 111 us, 4 rows 110, 6 rows
+// 117, 8 rows 117-125, 16 rows 129; forward: 85 / 76 / 75 / 77 / 78; sums pass: 4 rows 107 us, 8 rows
+// 84-87, 16 rows 88.
 #ifndef SNNLIF_BN_PLAIN_ROWS
-#define SNNLIF_BN_PLAIN_ROWS 8
+#define SNNLIF_BN_PLAIN_ROWS 4
 #endif
 #ifndef SNNLIF_BN_PLAIN_SUM_ROWS
 #define SNNLIF_BN_PLAIN_SUM_ROWS 8

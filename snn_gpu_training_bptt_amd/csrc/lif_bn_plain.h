@@ -49,7 +49,27 @@ namespace snnlif {
 #ifndef SNNLIF_BN_PLAIN_LANE_BYTES
 #define SNNLIF_BN_PLAIN_LANE_BYTES 16
 #endif
+// Cache policy of the sums pass (1 = non-temporal loads): x with the default policy, the gradient
+// streamed.  The input-gradient pass reads both again straight away; what the 256 MB memory-side cache
+// can keep for it is one tensor's worth, and with only x competing for it the second pass finds more.
+// Measured at [8,64,128,32,32] fp32 (sums + input-gradient kernel, us): both default 87 + 125, gradient
+// streamed 84 + 117, both streamed 81 + 134.
+#ifndef SNNLIF_BN_PLAIN_SUM_STREAM_X
+#define SNNLIF_BN_PLAIN_SUM_STREAM_X 0
+#endif
+#ifndef SNNLIF_BN_PLAIN_SUM_STREAM_G
+#define SNNLIF_BN_PLAIN_SUM_STREAM_G 1
+#endif
+// The input-gradient pass takes its tiles from the last to the first (1) or in storage order (0).
+#ifndef SNNLIF_BN_PLAIN_INPUT_DESCENDING
+#define SNNLIF_BN_PLAIN_INPUT_DESCENDING 1
+#endif
+// Threads per workgroup of the sums pass.
+#ifndef SNNLIF_BN_PLAIN_SUM_BLOCK
+#define SNNLIF_BN_PLAIN_SUM_BLOCK 256
+#endif
 constexpr int kBnPlainBlock = SNNLIF_BN_PLAIN_BLOCK;
+constexpr int kBnPlainSumBlock = SNNLIF_BN_PLAIN_SUM_BLOCK;
 
 // Channel constants of the V positions a lane owns.
 template <typename F, int V>
@@ -127,7 +147,7 @@ bn_plain_input_kernel(const F* __restrict__ x, const F* __restrict__ g,
                       const F* __restrict__ mean_gxhatx, F* __restrict__ gx, int64_t R,
                       int64_t CHW, int64_t HW, int64_t across, int64_t tiles) {
   for (int64_t turn = blockIdx.x; turn < tiles; turn += gridDim.x) {
-    const int64_t tile = tiles - 1 - turn;
+    const int64_t tile = SNNLIF_BN_PLAIN_INPUT_DESCENDING ? tiles - 1 - turn : turn;
     const int64_t slice = tile / across;
     const int64_t first = ((tile - slice * across) * blockDim.x + threadIdx.x) * V;
     if (first >= CHW) continue;
@@ -182,8 +202,8 @@ __device__ __forceinline__ void bn_plain_add_rows(const F* __restrict__ x, const
         xin[k] = F(0);
         gin[k] = F(0);
         if (r + k < end) {
-            xin[k] = load_pack<F, 1, false>(x + (r + k) * CHW + at).e[0];
-            gin[k] = load_pack<F, 1, false>(g + (r + k) * CHW + at).e[0];
+            xin[k] = load_pack<F, 1, SNNLIF_BN_PLAIN_SUM_STREAM_X != 0>(x + (r + k) * CHW + at).e[0];
+            gin[k] = load_pack<F, 1, SNNLIF_BN_PLAIN_SUM_STREAM_G != 0>(g + (r + k) * CHW + at).e[0];
         }
     }
 #pragma unroll
@@ -200,7 +220,7 @@ __device__ __forceinline__ void bn_plain_add_rows(const F* __restrict__ x, const
 // leaves part_*[(s * C + c) * G + i].
 // ---------------------------------------------------------------------------------------------
 template <typename F>
-__global__ void __launch_bounds__(kBnPlainBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_BN_PLAIN_WAVES)
+__global__ void __launch_bounds__(kBnPlainSumBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_BN_PLAIN_WAVES)
 bn_plain_sums_wave_kernel(const F* __restrict__ x, const F* __restrict__ g,
                           const F* __restrict__ ivar, const F* __restrict__ mean,
                           F* __restrict__ part_g, F* __restrict__ part_gx, int64_t R, int64_t rps,
@@ -236,7 +256,7 @@ bn_plain_sums_wave_kernel(const F* __restrict__ x, const F* __restrict__ g,
 // Sums, smaller planes: workgroup (blockIdx.x, blockIdx.y = s) sums the rows of slice s in its columns;
 // split = {g[S][CHW], g*xhat[S][CHW]}, the layout bn_channel_finalize_kernel folds.
 template <typename F>
-__global__ void __launch_bounds__(kBnPlainBlock)
+__global__ void __launch_bounds__(kBnPlainSumBlock)
 bn_plain_sums_column_kernel(const F* __restrict__ x, const F* __restrict__ g,
                             const F* __restrict__ ivar, const F* __restrict__ mean,
                             F* __restrict__ split, int64_t R, int64_t rps, int S, int64_t CHW,
@@ -338,8 +358,8 @@ int bn_plain_backward_stats(const F* x, const F* weight, const F* ivar, const F*
         const int64_t G = (HW + 63) / 64;
         F* part_g = workspace;
         F* part_gx = workspace + S * C * G;
-        launch_kernel(bn_plain_sums_wave_kernel<F>, dim3(grid_for(S * C * G * 64, kBnPlainBlock)),
-                      dim3(kBnPlainBlock), 0, stream, x, g, ivar, mean, part_g, part_gx, R, rps, S, C,
+        launch_kernel(bn_plain_sums_wave_kernel<F>, dim3(grid_for(S * C * G * 64, kBnPlainSumBlock)),
+                      dim3(kBnPlainSumBlock), 0, stream, x, g, ivar, mean, part_g, part_gx, R, rps, S, C,
                       HW, G);
         int rc = launch_status();
         if (rc != SNNLIF_OK) return rc;
@@ -350,9 +370,9 @@ int bn_plain_backward_stats(const F* x, const F* weight, const F* ivar, const F*
     }
     F* split = workspace;
     launch_kernel(bn_plain_sums_column_kernel<F>,
-                  dim3(static_cast<unsigned>((CHW + kBnPlainBlock - 1) / kBnPlainBlock),
+                  dim3(static_cast<unsigned>((CHW + kBnPlainSumBlock - 1) / kBnPlainSumBlock),
                        static_cast<unsigned>(S)),
-                  dim3(kBnPlainBlock), 0, stream, x, g, ivar, mean, split, R, rps, static_cast<int>(S),
+                  dim3(kBnPlainSumBlock), 0, stream, x, g, ivar, mean, split, R, rps, static_cast<int>(S),
                   CHW, HW);
     int rc = launch_status();
     if (rc != SNNLIF_OK) return rc;
