@@ -439,6 +439,80 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------
+// Forward with a rolling window of W rows in flight, for windows of a multiple of W steps: once a row
+// has been consumed and its spike stored, the row W steps later is requested into the register it
+// left.  A wavefront then keeps W loads outstanding from its first instruction to its last group and
+// issues loads and stores alternately, instead of a burst of requests followed by a burst of stores.
+// ---------------------------------------------------------------------------------------------
+// Used for streamed windows of a multiple of SNNLIF_FWD_ROLLING_W steps from SNNLIF_FWD_ROLLING_MIN_T on.
+// Measured cold on MI355X against the burst form (32 rows at once at 3 wavefronts per SIMD, groups of 16
+// beyond), fp32, % of the HBM peak: 32 steps 71.9 -> 73.1 (256 MiB tensors), 63.4 -> 65.7 (128 MiB),
+// 76.8 -> 77.8 (512 MiB); 64 steps 59.7 -> 67.0; 96 steps 66.2 -> 70.7.  16 rows at 2 wavefronts per SIMD
+// is the best of 4 / 8 / 16 / 32 rows at 1-8 wavefronts (8 rows at 4: 66 % at 32 steps; 16 rows at 1: 64 %).
+#ifndef SNNLIF_FWD_ROLLING_W
+#define SNNLIF_FWD_ROLLING_W 16
+#endif
+#ifndef SNNLIF_FWD_ROLLING_MIN_T
+#define SNNLIF_FWD_ROLLING_MIN_T 32
+#endif
+#ifndef SNNLIF_FWD_ROLLING_WAVES
+#define SNNLIF_FWD_ROLLING_WAVES 2
+#endif
+template <typename S, typename M, int V, int W, bool WRITE_U, bool WRITE_S, bool KEEP>
+__global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_FWD_ROLLING_WAVES)
+lif_forward_rolling_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__ spike, int T,
+                           int64_t N, int64_t nvec, typename Arith<S>::type alpha,
+                           typename Arith<S>::type thresh) {
+    using C = typename Arith<S>::type;
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+    for (int64_t v = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; v < nvec;
+         v += stride) {
+        const int64_t col = v * V;
+        C u[V], s[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            u[j] = C(0);
+            s[j] = C(0);
+        }
+        Pack<S, V> buf[W];
+#pragma unroll
+        for (int k = 0; k < W; ++k) buf[k] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(k) * N + col);
+        int t0 = 0;
+        for (; t0 + W < T; t0 += W) {
+#pragma unroll
+            for (int k = 0; k < W; ++k) {
+                Pack<M, V> mo;
+                Pack<S, V> so;
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    lif_step<C>(u[j], s[j], Arith<S>::load(buf[k].e[j]), alpha, thresh);
+                    if (WRITE_U) mo.e[j] = Arith<M>::store(u[j]);
+                    if (WRITE_S) so.e[j] = Arith<S>::store(s[j]);
+                }
+                const int64_t off = static_cast<int64_t>(t0 + k) * N + col;
+                if (WRITE_U) store_pack<M, V>(mem + off, mo);
+                if (WRITE_S) store_pack<S, V>(spike + off, so);
+                buf[k] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(t0 + W + k) * N + col);
+            }
+        }
+#pragma unroll
+        for (int k = 0; k < W; ++k) {
+            Pack<M, V> mo;
+            Pack<S, V> so;
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                lif_step<C>(u[j], s[j], Arith<S>::load(buf[k].e[j]), alpha, thresh);
+                if (WRITE_U) mo.e[j] = Arith<M>::store(u[j]);
+                if (WRITE_S) so.e[j] = Arith<S>::store(s[j]);
+            }
+            const int64_t off = static_cast<int64_t>(t0 + k) * N + col;
+            if (WRITE_U) store_pack<M, V>(mem + off, mo);
+            if (WRITE_S) store_pack<S, V>(spike + off, so);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
 // One register-resident backward window of at most TW rows, for the neuron(s) at column `col`.
 // Row pointers x, g, gx are those of the window's first row; rows of x and gx are N elements apart,
 // rows of g GN elements (GN == N: a dense gradient; GN == 0: one row that stands for every step).  On entry uc / sc hold the membrane
@@ -823,7 +897,8 @@ int launch_forward_rows(const S* x, M* mem, S* spike, int64_t T, int64_t N, floa
 // window of 9-16 rows as one group measures +5-8 points over two groups of 8), and so are windows
 // of 24-32 rows, in a 32-row instantiation at 3 wavefronts per SIMD (+3-5 points over two groups of
 // 16; a 20-row window zero-filled to 32 loses 4-8, so 17-23 rows stay in groups).  Everything else
-// goes in groups of 16 (groups of 32 gain 3-4 points at 48 and 64 rows and lose 1-7 from 96 on).
+// goes in groups of 16 (groups of 32 gain 3-4 points at 48 and 64 rows and lose 1-7 from 96 on), except
+// windows of a multiple of 16 rows from 32 on, which run the rolling-window kernel.
 template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S, bool KEEP>
 int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
                      hipStream_t stream) {
@@ -843,6 +918,16 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
                 x, mem, spike, T, N, alpha, thresh, threads, stream);
     }
     if (T <= TC) return SNNLIF_FWD_LAUNCH(TC, false);
+    if constexpr (!KEEP && SNNLIF_FWD_ROLLING_W > 0) {
+        if (T >= SNNLIF_FWD_ROLLING_MIN_T && T > SNNLIF_FWD_ROLLING_W && T % (SNNLIF_FWD_ROLLING_W > 0 ? SNNLIF_FWD_ROLLING_W : 1) == 0) {
+            using C = typename Arith<S>::type;
+            const int64_t nvec = N / V;
+            launch_kernel(lif_forward_rolling_kernel<S, M, V, (SNNLIF_FWD_ROLLING_W > 0 ? SNNLIF_FWD_ROLLING_W : 1), WRITE_U, WRITE_S, KEEP>,
+                          dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
+                          static_cast<int>(T), N, nvec, C(alpha), C(thresh));
+            return launch_status();
+        }
+    }
     if constexpr (!KEEP) {
         if (T <= TM) return SNNLIF_FWD_LAUNCH(TM, false);
         if (T <= TL && T >= TL - TL / 4) return SNNLIF_FWD_LAUNCH(TL, false);

@@ -151,6 +151,25 @@ def test_windows_between_64_and_128(cabi, oracle, T, dtype, keep):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("T", [32, 48, 64, 160, 1040])
+def test_streamed_windows_of_a_multiple_of_16_steps(cabi, oracle, T, dtype):
+    """The streamed forward of these windows is the rolling-window kernel (16 rows in flight, refilled
+    row by row): spikes, the membrane output and, for the 1040-step window, the potential it stages in
+    the backward's workspace (fp32 behind bf16 storage) must be the oracle's bits.  Even and odd N."""
+    wide = torch.float64 if dtype == torch.float64 else torch.float32
+    for n_inner in (256, 77):
+        x32, g32 = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=9000 + T)
+        x, g = x32.to(dtype), g32.to(dtype)
+        mem, spike_a, spike_b, gx = run_gpu(cabi, x, g, alpha=0.3, keep=False)
+        mem_o, spike_o = oracle.fire_forward(x.to(wide).numpy(), 0.3, THRESH)
+        gx_o = oracle.fire_backward(x.to(wide).numpy(), g.to(wide).numpy(), 0.3, THRESH, BETA, INTERVAL)
+        as_stored = lambda a: torch.from_numpy(a).to(dtype)
+        assert torch.equal(spike_a, as_stored(spike_o)) and torch.equal(spike_b, as_stored(spike_o))
+        assert torch.equal(mem, as_stored(mem_o))
+        assert torch.equal(gx, as_stored(gx_o))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
 @pytest.mark.parametrize("T", [33, 34, 39, 57, 63, 65, 66, 71, 95, 97, 105, 127, 129, 159, 160, 161, 191, 193, 250, 1023])
 def test_segmented_windows(cabi, oracle, T, dtype):
     """Windows cut into 32-step segments, the last one partial: one step into a new segment (33, 65, 97,
