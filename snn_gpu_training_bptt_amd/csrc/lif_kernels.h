@@ -525,8 +525,10 @@ lif_forward_rolling_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __re
 // Gradient rows are fetched in groups of at most GC, the newest time steps first; the fetch of the
 // next (earlier) group is issued before the current group is consumed.
 // KEEP: x is loaded with the default cache policy, otherwise with the non-temporal hint.
+// GSHARED: the gradient is one row that stands for every step of the window (GN == 0): it is loaded
+// once instead of once per step.
 // ---------------------------------------------------------------------------------------------
-template <typename S, int V, int TW, bool EXACT, bool KEEP = true>
+template <typename S, int V, int TW, bool EXACT, bool KEEP = true, bool GSHARED = false>
 __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S* __restrict__ g,
                                                 S* __restrict__ gx, int rows, int64_t N,
                                                 int64_t GN, int64_t col,
@@ -553,10 +555,12 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
                 xin[t] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(t) * N + col);
         }
     }
-    Pack<S, V> gbuf[2][GC];
+    Pack<S, V> gbuf[2][GSHARED ? 1 : GC];
+    if constexpr (GSHARED) gbuf[0][0] = load_pack<S, V, true>(g + col);
 #pragma unroll
     for (int t = TW - 1; t >= ((TW - GC) > 0 ? (TW - GC) : 0); --t) {
-        const int k = t - ((TW - GC) > 0 ? (TW - GC) : 0);
+        if constexpr (GSHARED) break;
+        const int k = GSHARED ? 0 : t - ((TW - GC) > 0 ? (TW - GC) : 0);
         if (EXACT) {
             gbuf[0][k] = load_pack<S, V, true>(g + static_cast<int64_t>(t) * GN + col);
         } else {
@@ -579,18 +583,18 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
     for (int q = 0; q < NG; ++q) {
         const int hi = TW - q * GC;
         const int lo = (hi - GC) > 0 ? (hi - GC) : 0;
-        if (q + 1 < NG) {
+        if (!GSHARED && q + 1 < NG) {
             const int nhi = lo;
             const int nlo = (nhi - GC) > 0 ? (nhi - GC) : 0;
 #pragma unroll
             for (int t = nhi - 1; t >= nlo; --t) {
                 if (EXACT) {
-                    gbuf[(q + 1) & 1][t - nlo] =
+                    gbuf[(q + 1) & 1][GSHARED ? 0 : t - nlo] =
                         load_pack<S, V, true>(g + static_cast<int64_t>(t) * GN + col);
                 } else {
-                    gbuf[(q + 1) & 1][t - nlo] = zero_pack<S, V>();
+                    gbuf[(q + 1) & 1][GSHARED ? 0 : t - nlo] = zero_pack<S, V>();
                     if (t < rows)
-                        gbuf[(q + 1) & 1][t - nlo] =
+                        gbuf[(q + 1) & 1][GSHARED ? 0 : t - nlo] =
                             load_pack<S, V, true>(g + static_cast<int64_t>(t) * GN + col);
                 }
             }
@@ -601,7 +605,8 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
                 Pack<S, V> out;
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
-                    lif_reverse_step<C>(gu[j], u[t][j], Arith<S>::load(gbuf[q & 1][t - lo].e[j]),
+                    lif_reverse_step<C>(gu[j], u[t][j],
+                                        Arith<S>::load(gbuf[GSHARED ? 0 : (q & 1)][GSHARED ? 0 : t - lo].e[j]),
                                         alpha, thresh, beta, interval);
                     out.e[j] = Arith<S>::store(gu[j]);
                 }
@@ -623,7 +628,7 @@ __device__ __forceinline__ int64_t backward_column(int64_t v, int64_t nvec, int 
 // ---------------------------------------------------------------------------------------------
 // Fused backward for T <= TW: the whole time axis is one register window.
 // ---------------------------------------------------------------------------------------------
-template <typename S, int V, int TW, bool EXACT, bool KEEP>
+template <typename S, int V, int TW, bool EXACT, bool KEEP, bool GSHARED = false>
 __global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW, KEEP))
 lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
                           int T, int64_t N, int64_t GN, int64_t nvec,
@@ -641,8 +646,8 @@ lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* _
             sc[j] = C(0);
             gu[j] = C(0);
         }
-        backward_window<S, V, TW, EXACT, KEEP>(x, g, gx, T, N, GN, col, uc, sc, gu, alpha, thresh,
-                                               beta, interval);
+        backward_window<S, V, TW, EXACT, KEEP, GSHARED>(x, g, gx, T, N, GN, col, uc, sc, gu, alpha,
+                                                        thresh, beta, interval);
     }
 }
 
@@ -1034,7 +1039,15 @@ int launch_backward_fused_policy(const S* x, const S* g, S* gx, int64_t T, int64
             backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S), 64, KEEP);
         const dim3 grid(grid_for(nvec, threads)), block(threads);
         const int Ti = static_cast<int>(T);
-        if (exact) {
+        // one gradient row for all steps, window with a straight-line instantiation of its own: the
+        // form that loads the row once (other lengths read it in place once per step)
+        constexpr bool has_shared = TW >= 2 && TW <= SNNLIF_BP_FUSED_MAX_T;
+        if (exact && GN == 0 && has_shared) {
+            if constexpr (has_shared)
+                launch_kernel(lif_backward_fused_kernel<S, V, TW, true, KEEP, true>, grid, block, 0,
+                              stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta),
+                              C(interval));
+        } else if (exact) {
             launch_kernel(lif_backward_fused_kernel<S, V, TW, true, KEEP>, grid, block, 0, stream,
                                x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
         } else if constexpr (can_be_inexact) {
