@@ -178,8 +178,8 @@ int snnlif_fire_bp_strided(const void* spatial, const void* grad_spike, void* gr
                            float beta, float interval, void* workspace, size_t workspace_bytes,
                            void* stream);
 
-/* Bytes of device workspace snnlif_bn_stats needs (partial sums: two of the storage type per wavefront
- * when HW >= 32, two per (row slice, channel position) otherwise).  0 for invalid arguments. */
+/* Bytes of device workspace snnlif_bn_stats needs (partial sums: two doubles per wavefront when
+ * HW >= 32, two per (row slice, channel position) otherwise).  0 for invalid arguments. */
 size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t C, int64_t HW);
 
 /*
@@ -190,8 +190,8 @@ size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t 
  * Replaces the framework reductions the reference's layers run before every batch-norm op:
  * torch.var_mean(x, dim_bn, unbiased=False) (snnlib/example/snnlib_op.py:36-37, 76-78, 113-115,
  * 175-177) and torch.mean(x), torch.mean(x**2) of the sharded layers (snnlib/example/snnlib_op.py:263-264,
- * 326-327, 386-387).  One pass over the tensor; sums are taken of x minus the channel's first element and
- * added up per channel in double precision, in a fixed order (reproducible results).  `spatial` is
+ * 326-327, 386-387).  One pass over the tensor; sums are taken of x minus the channel's first element, in
+ * double precision throughout, and added up per channel in a fixed order (reproducible results).  `spatial` is
  * loaded with the default cache policy, so a tensor that fits the memory-side cache is still there
  * for the batch-norm op that follows.  T, B or HW of zero with C > 0 is SNNLIF_ERR_ARG (a channel
  * without elements has no statistics).  `workspace`: snnlif_bn_stats_workspace_bytes() bytes, 16-byte

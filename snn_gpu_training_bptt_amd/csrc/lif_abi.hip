@@ -285,7 +285,7 @@ size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t 
     const size_t es = bn_element_size(dtype, &rc);
     if (es == 0 || bn_shape_error(T, B, C, HW) != SNNLIF_OK) return 0;
     if (T == 0 || B * C * HW == 0) return 0;
-    return snnlif::bn_stats_workspace_elems(T, B, C, HW) * es;
+    return snnlif::bn_stats_workspace_elems(T, B, C, HW) * sizeof(double);
 }
 
 int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64_t T, int64_t B,
@@ -303,7 +303,7 @@ int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64
     if (!spatial || !mean || !var) return SNNLIF_ERR_ARG;
     const void* ptrs[3] = {spatial, mean, var};
     if (!all_aligned(ptrs, 3, es)) return SNNLIF_ERR_ALIGN;
-    const size_t need = snnlif::bn_stats_workspace_elems(T, B, C, HW) * es;
+    const size_t need = snnlif::bn_stats_workspace_elems(T, B, C, HW) * sizeof(double);
     if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
     if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -311,7 +311,7 @@ int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64
     return SNNLIF_BN_DISPATCH(
         es,
         snnlif::bn_stats_f32(CF(spatial), MF(mean), MF(var), raw_moments != 0, T, B, C, HW,
-                             MF(workspace), st),
+                             MD(workspace), st),
         snnlif::bn_stats_f64(CD(spatial), MD(mean), MD(var), raw_moments != 0, T, B, C, HW,
                              MD(workspace), st));
 }

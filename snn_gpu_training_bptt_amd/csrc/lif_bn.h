@@ -56,7 +56,7 @@ inline size_t bn_backward_workspace_elems(int64_t T, int64_t B, int64_t C, int64
 
 // Batch statistics (lif_bn_stats.h): threads per workgroup of the partial-sum kernels, the number of
 // slices the rows of a small-plane tensor are dealt to (enough workgroups to fill the chip), partial
-// sums per quantity (one per wavefront, or one per (slice, column)), and the workspace in elements.
+// sums per quantity (one per wavefront, or one per (slice, column)), and the workspace in doubles.
 #ifndef SNNLIF_STATS_BLOCK
 #define SNNLIF_STATS_BLOCK 256
 #endif
@@ -144,7 +144,7 @@ enum class SpatialHint;  // lif_kernels.h
                             int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,\
                             SpatialHint keep_x, hipStream_t stream);                               \
     int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,      \
-                          int64_t C, int64_t HW, F* workspace, hipStream_t stream);                \
+                          int64_t C, int64_t HW, double* workspace, hipStream_t stream);           \
     int bn_backward_stats_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,      \
                                    const F* mean, const F* g, F* grad_weight, F* grad_bias,        \
                                    F* mean_gxhat, F* mean_gxhatx, int64_t T, int64_t B, int64_t C, \

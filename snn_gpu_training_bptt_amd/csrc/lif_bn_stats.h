@@ -12,10 +12,10 @@
 // One pass over x (4 bytes per neuron-step in fp32), HBM-bound, two kernels:
 //   1. partial sums.  Planes of at least 32 positions: wavefronts are laid over the (batch entry,
 //      channel) planes as in sweep 1 of the batch-norm backward (ceil(HW/64) wavefronts per plane,
-//      all lanes of a wavefront share a channel); a lane adds up its neuron's T values (sixteen at
-//      a time in the storage type, the groups in double; windows of fewer than sixteen steps: the
-//      values of several batch entries, so that sixteen requests are in flight all the same), the wavefront
-//      folds the 64 lanes by shuffles and leaves one pair of sums.  Smaller planes (fully
+//      all lanes of a wavefront share a channel); a lane adds up its neuron's T values (requested
+//      sixteen at a time, summed in double; windows of fewer than sixteen steps: the values of several
+//      batch entries, so that sixteen requests are in flight all the same), the wavefront
+//      folds the 64 lanes by shuffles and leaves one pair of sums (doubles, whatever the storage type).  Smaller planes (fully
 //      connected shapes): one lane per (channel, position) column of the [T*B, C*HW] matrix, the rows
 //      dealt round-robin to S slices of workgroups; consecutive lanes read consecutive addresses.
 //   2. one workgroup per channel adds the partial sums in double precision, in an order fixed by the
@@ -23,7 +23,10 @@
 // Sums are taken of d = x - K[c] with K[c] the channel's first element (t = 0, b = 0, position 0):
 // a shift by any sample of the channel keeps sum(d)^2/n and sum(d^2) of comparable size, so that
 // var = (sum(d^2) - sum(d)^2/n)/n does not cancel even when |mean| >> sqrt(var) (the textbook shifted
-// two-sum formula); mean = K + sum(d)/n.
+// two-sum formula); mean = K + sum(d)/n.  d, d^2 and every sum are formed in double precision (the
+// subtraction is then exact for fp32 storage), so a shift that happens to be an outlier -- D standard
+// deviations from the mean -- costs about 1e-16 * D^2 of relative accuracy in the variance, not
+// 6e-8 * D^2 as squares taken in fp32 would.
 #ifndef SNNLIF_LIF_BN_STATS_H
 #define SNNLIF_LIF_BN_STATS_H
 
@@ -46,23 +49,19 @@ constexpr int kStatsRows = SNNLIF_STATS_ROWS;
 #define SNNLIF_STATS_LANE_BYTES 4
 #endif
 
-// Adds the group sums of kStatsRows x V values (sum of d and of d*d, d = value - shift, in the storage
-// type) to the running sums in double.
+// Adds kStatsRows x V values to the running sums of d and d*d, d = value - shift, all in double.
 template <typename F, int V>
-__device__ __forceinline__ void stats_add_group(const Pack<F, V> (&v)[kStatsRows], F shift,
+__device__ __forceinline__ void stats_add_group(const Pack<F, V> (&v)[kStatsRows], double shift,
                                                 double& acc_d, double& acc_dd) {
-    F group_d = F(0), group_dd = F(0);
 #pragma unroll
     for (int r = 0; r < kStatsRows; ++r) {
 #pragma unroll
         for (int j = 0; j < V; ++j) {
-            const F d = v[r].e[j] - shift;
-            group_d += d;
-            group_dd += d * d;
+            const double d = static_cast<double>(v[r].e[j]) - shift;
+            acc_d += d;
+            acc_dd += d * d;
         }
     }
-    acc_d += static_cast<double>(group_d);
-    acc_dd += static_cast<double>(group_dd);
 }
 
 template <typename F, int V>
@@ -78,13 +77,14 @@ __device__ __forceinline__ Pack<F, V> stats_fill(F value) {
 // [rows = T*B, C*HW] matrix (row t*B + b) there; part_* indexed [slice][channel][chunk].
 //   SLICED = false (windows of at least kStatsRows steps): S = B slices, slice b = the T rows of
 //       batch entry b, `step` = B*C*HW elements apart, kStatsRows at a time;
-//   SLICED = true (shorter windows): the rows are dealt round-robin to S = rows / kStatsRows slices
-//       (rows s, s+S, s+2S, ... belong to slice s), so that a lane still has kStatsRows requests in
+//   SLICED = true (shorter windows): S = rows / kStatsRows slices of consecutive rows (slice s = rows
+//       [s * rps, (s + 1) * rps), rps = ceil(rows / S)), so that a lane still has kStatsRows requests in
 //       flight: it sums the values of several batch entries.  `step` = C*HW.
 template <typename F, int V, bool SLICED>
 __global__ void __launch_bounds__(kStatsBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_STATS_WAVES)
-bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restrict__ part_dd,
-                     int rows, int64_t step, int64_t C, int64_t HW, int64_t G, int64_t S) {
+bn_stats_wave_kernel(const F* __restrict__ x, double* __restrict__ part_d,
+                     double* __restrict__ part_dd, int rows, int64_t step, int64_t C, int64_t HW,
+                     int64_t G, int64_t S) {
     const int64_t lanes = S * C * G * 64;
     const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
     for (int64_t pc = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; pc < lanes;
@@ -95,11 +95,15 @@ bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restr
         const int c = static_cast<int>(plane % C);
         double acc_d = 0.0, acc_dd = 0.0;
         if (k < HW) {
-            const F shift = x[static_cast<int64_t>(c) * HW];
-            // first row of the slice; its further rows are `hop` elements apart
-            const F* col = x + plane * HW + k;
-            const int64_t hop = SLICED ? S * step : step;
-            const int count = SLICED ? static_cast<int>((rows - plane / C + S - 1) / S) : rows;
+            const double shift = static_cast<double>(x[static_cast<int64_t>(c) * HW]);
+            // first row of the slice; its further rows are `step` elements apart
+            const int64_t slice = plane / C;
+            const int rps = SLICED ? static_cast<int>((rows + S - 1) / S) : rows;
+            const int64_t first = SLICED ? slice * rps : 0;
+            const F* col = SLICED ? x + first * step + static_cast<int64_t>(c) * HW + k : x + plane * HW + k;
+            const int64_t hop = step;
+            const int left = rows - static_cast<int>(first);
+            const int count = SLICED ? (left < rps ? (left < 0 ? 0 : left) : rps) : rows;
             int t0 = 0;
             for (; t0 + kStatsRows <= count; t0 += kStatsRows) {  // whole groups: straight-line loads
                 Pack<F, V> v[kStatsRows];
@@ -112,7 +116,7 @@ bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restr
                 Pack<F, V> v[kStatsRows];
 #pragma unroll
                 for (int r = 0; r < kStatsRows; ++r) {
-                    v[r] = stats_fill<F, V>(shift);  // rows past the end contribute d = 0
+                    v[r] = stats_fill<F, V>(x[static_cast<int64_t>(c) * HW]);  // rows past the end: d = 0
                     if (t0 + r < count)
                         v[r] = load_pack<F, V, false>(col + static_cast<int64_t>(t0 + r) * hop);
                 }
@@ -122,8 +126,8 @@ bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restr
         acc_d = wave_sum(acc_d);
         acc_dd = wave_sum(acc_dd);
         if ((pc & 63) == 0) {
-            part_d[wave] = static_cast<F>(acc_d);
-            part_dd[wave] = static_cast<F>(acc_dd);
+            part_d[wave] = acc_d;
+            part_dd[wave] = acc_dd;
         }
     }
 }
@@ -133,25 +137,26 @@ bn_stats_wave_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restr
 // part_* indexed [slice][column].
 template <typename F>
 __global__ void __launch_bounds__(kStatsBlock)
-bn_stats_column_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __restrict__ part_dd,
-                       int64_t rows, int64_t CHW, int64_t HW, int S) {
+bn_stats_column_kernel(const F* __restrict__ x, double* __restrict__ part_d,
+                       double* __restrict__ part_dd, int64_t rows, int64_t CHW, int64_t HW, int S) {
     const int64_t j = static_cast<int64_t>(blockIdx.x) * kStatsBlock + threadIdx.x;
     if (j >= CHW) return;
     const int s = blockIdx.y;
-    const F shift = x[(j / HW) * HW];
+    const F first_of_channel = x[(j / HW) * HW];
+    const double shift = static_cast<double>(first_of_channel);
     double acc_d = 0.0, acc_dd = 0.0;
     for (int64_t r0 = s; r0 < rows; r0 += static_cast<int64_t>(S) * kStatsRows) {
         Pack<F, 1> v[kStatsRows];
 #pragma unroll
         for (int q = 0; q < kStatsRows; ++q) {
             const int64_t r = r0 + static_cast<int64_t>(q) * S;
-            v[q] = stats_fill<F, 1>(shift);
+            v[q] = stats_fill<F, 1>(first_of_channel);
             if (r < rows) v[q] = load_pack<F, 1, false>(x + r * CHW + j);
         }
         stats_add_group<F, 1>(v, shift, acc_d, acc_dd);
     }
-    part_d[static_cast<int64_t>(s) * CHW + j] = static_cast<F>(acc_d);
-    part_dd[static_cast<int64_t>(s) * CHW + j] = static_cast<F>(acc_dd);
+    part_d[static_cast<int64_t>(s) * CHW + j] = acc_d;
+    part_dd[static_cast<int64_t>(s) * CHW + j] = acc_dd;
 }
 
 // One workgroup per channel: adds the channel's partial sums in double and writes
@@ -161,8 +166,8 @@ bn_stats_column_kernel(const F* __restrict__ x, F* __restrict__ part_d, F* __res
 // s < S, i < HW.  Both are "outer" groups of "inner" consecutive entries, outer_stride apart.
 template <typename F>
 __global__ void __launch_bounds__(kReduceBlock)
-bn_stats_finalize_kernel(const F* __restrict__ x, const F* __restrict__ part_d,
-                         const F* __restrict__ part_dd, F* __restrict__ out_a,
+bn_stats_finalize_kernel(const F* __restrict__ x, const double* __restrict__ part_d,
+                         const double* __restrict__ part_dd, F* __restrict__ out_a,
                          F* __restrict__ out_b, int64_t HW, int64_t outer, int64_t inner,
                          int64_t outer_stride, double count, bool moments) {
     const int c = blockIdx.x;
@@ -171,8 +176,8 @@ bn_stats_finalize_kernel(const F* __restrict__ x, const F* __restrict__ part_d,
     double a = 0.0, aa = 0.0;
     for (int64_t e = threadIdx.x; e < n; e += kReduceBlock) {
         const int64_t at = (e / inner) * outer_stride + base + (e % inner);
-        a += static_cast<double>(part_d[at]);
-        aa += static_cast<double>(part_dd[at]);
+        a += part_d[at];
+        aa += part_dd[at];
     }
     __shared__ double lds[2][kReduceBlock / 64];
     a = wave_sum(a);
@@ -202,11 +207,11 @@ bn_stats_finalize_kernel(const F* __restrict__ x, const F* __restrict__ part_d,
 
 template <typename F>
 int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B, int64_t C,
-             int64_t HW, F* workspace, hipStream_t stream) {
+             int64_t HW, double* workspace, hipStream_t stream) {
     const int64_t N = B * C * HW;
     const size_t P = bn_stats_partial_count(T, B, C, HW);
-    F* part_d = workspace;
-    F* part_dd = workspace + P;
+    double* part_d = workspace;
+    double* part_dd = workspace + P;
     const double count = static_cast<double>(T) * static_cast<double>(B) * static_cast<double>(HW);
     if (bn_wave_partials(HW)) {
         // widest lanes for which rows, planes and the base address stay aligned and a wavefront
@@ -253,7 +258,7 @@ int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,
 #define SNNLIF_DEFINE_BN_STATS_DTYPE(SUFFIX, F)                                                    \
     namespace snnlif {                                                                             \
     int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,      \
-                          int64_t C, int64_t HW, F* workspace, hipStream_t stream) {               \
+                          int64_t C, int64_t HW, double* workspace, hipStream_t stream) {          \
         return bn_stats<F>(x, out_a, out_b, moments, T, B, C, HW, workspace, stream);              \
     }                                                                                              \
     }

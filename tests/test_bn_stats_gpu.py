@@ -126,6 +126,27 @@ def test_variance_survives_a_mean_far_from_zero(cabi, shape):
     assert_close(var, var_ref, var_ref, 1e-6, "biased variance")
 
 
+@pytest.mark.parametrize("shape", [(8, 16, 8, 16, 16), (8, 64, 32), (5, 2, 9, 31)])
+@pytest.mark.parametrize("distance", [100.0, 1000.0])
+def test_variance_survives_an_outlier_as_the_shift(cabi, shape, distance):
+    """The sums are shifted by each channel's first element (t = 0, b = 0, position 0).  Make that element
+    an outlier, `distance` standard deviations from the channel's mean: the shift is then a poor guess of
+    the mean, the shifted squares are `distance`^2 times the variance, and sums of squares taken in
+    float32 would lose 6e-8 * distance^2 of it (6e-4 and 6e-2 here).  Formed in double they must still
+    meet the 1e-6 bar."""
+    x = make(shape, seed=54)
+    C = shape[2]
+    flat = x.reshape(shape[0], shape[1], C, -1)
+    sigma = flat.double().std(dim=(0, 1, 3))
+    flat[0, 0, :, 0] += (distance * sigma).float()
+    mean_ref, var_ref, second_ref = reference(x)
+    mean, var = run_stats(cabi, x.cuda())
+    assert_close(mean, mean_ref, var_ref.sqrt() + mean_ref.abs(), 1e-6, "mean")
+    assert_close(var, var_ref, var_ref, 1e-6, "biased variance")
+    _, second = run_stats(cabi, x.cuda(), raw_moments=True)
+    assert_close(second, second_ref, second_ref, 1e-6, "second raw moment")
+
+
 def test_constant_channels_have_zero_variance(cabi):
     x = torch.full((4, 3, 5, 6, 6), 0.75)
     x[:, :, 2] = -3.0
