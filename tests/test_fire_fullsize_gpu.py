@@ -3,7 +3,9 @@ not need a full-size CPU run:
 
 * neuron independence -- a random sample of neuron columns, gathered from the full-size device
   tensors, must equal the oracle run on just those columns (exact for fp32; spikes exact and
-  gradients equal to the fp32 result rounded once for bf16 storage);
+  gradients equal to the fp32 result rounded once for bf16 storage), for the spikes, the membrane
+  potential of snnlif_fire_us_fp and the input gradient, in both the streamed instantiations of the
+  kernels (what tensors of this size get without a hint) and the kept ones;
 * prefix property     -- the first T' steps of the full window equal a run over a T'-step window;
 * linearity           -- scaling the spike gradient by 4 scales the input gradient by 4, bit for bit;
 * the stored golden vectors (tests/golden/fire_vectors.json) are reproduced exactly.
@@ -46,8 +48,9 @@ def oracle():
     return c_oracle
 
 
+@pytest.mark.parametrize("keep", [None, True], ids=["by-size", "kept"])
 @pytest.mark.parametrize("name", list(FULL))
-def test_full_size_configuration(cabi, oracle, name):
+def test_full_size_configuration(cabi, oracle, name, keep):
     shape, mean, std, dtype = FULL[name]
     T = shape[0]
     N = int(np.prod(shape[1:]))
@@ -56,8 +59,8 @@ def test_full_size_configuration(cabi, oracle, name):
     g = torch.randn(shape, generator=gen, device="cuda").to(dtype)
     spike = torch.empty_like(x)
     gx = torch.empty_like(x)
-    cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
-    cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+    cabi.fire_s_fp_into(x, spike, ALPHA, THRESH, keep_spatial=keep)
+    cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL, keep_spatial=keep)
     torch.cuda.synchronize()
 
     # -- sampled neurons against the oracle
@@ -65,9 +68,16 @@ def test_full_size_configuration(cabi, oracle, name):
     idx[:4] = torch.tensor([0, 1, N - 2, N - 1])        # both ends of the tensor
     take = lambda t: t.view(T, N)[:, idx].float().cpu().numpy().reshape(T, 1, -1)
     xs, gs = take(x), take(g)
-    _, spike_o = oracle.fire_forward(xs, ALPHA, THRESH)
+    mem_o, spike_o = oracle.fire_forward(xs, ALPHA, THRESH)
     gx_o = oracle.fire_backward(xs, gs, ALPHA, THRESH, BETA, INTERVAL)
     assert np.array_equal(take(spike), spike_o), "sampled spikes differ from the oracle"
+    # the membrane potential of the (u, spike) forward, and its spikes, on the same sample
+    mem, spike_b = torch.empty_like(x), torch.empty_like(x)
+    cabi.fire_us_fp_into(x, mem, spike_b, ALPHA, THRESH, keep_spatial=keep)
+    assert torch.equal(spike_b, spike)
+    mem_expect = mem_o if dtype == torch.float32 else torch.from_numpy(mem_o).to(dtype).float().numpy()
+    assert np.array_equal(take(mem), mem_expect), "sampled membrane potentials differ from the oracle"
+    del mem, spike_b
     if dtype == torch.float32:
         assert np.array_equal(take(gx), gx_o), "sampled gradients differ from the oracle"
     else:
@@ -81,14 +91,14 @@ def test_full_size_configuration(cabi, oracle, name):
     # -- prefix property on the device
     Tp = T // 2
     spike_p = torch.empty_like(x[:Tp])
-    cabi.fire_s_fp_into(x[:Tp], spike_p, ALPHA, THRESH)
+    cabi.fire_s_fp_into(x[:Tp], spike_p, ALPHA, THRESH, keep_spatial=keep)
     assert torch.equal(spike_p, spike[:Tp])
     del spike_p
 
     # -- linearity in the spike gradient (power-of-two scale commutes with rounding)
     g4 = g * 4
     gx4 = torch.empty_like(x)
-    cabi.fire_bp_into(x, g4, gx4, ALPHA, THRESH, BETA, INTERVAL)
+    cabi.fire_bp_into(x, g4, gx4, ALPHA, THRESH, BETA, INTERVAL, keep_spatial=keep)
     assert torch.equal(gx4, gx * 4)
 
 
