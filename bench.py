@@ -6,6 +6,7 @@
     python bench.py --workload train_step [--steps K] [--warmup W]     (context figure, see below)
     python bench.py --workload bn_fire    [--steps K] [--warmup W]     (next-row op, see below)
     python bench.py --workload bn         [--steps K] [--warmup W]     (next-row op, see below)
+    python bench.py --workload policy_sweep                            (kernel rates over shapes, see below)
 
 One "step" is one forward (spikes from the input current) plus one backward (input gradient from
 the saved input current and the spike gradient) over one synthetic batch that is already resident
@@ -53,6 +54,9 @@ fire kernels, measured with events around the ``snnlib.fire_s_fp`` / ``snnlib.fi
 ``snnlif_bn_fire_s_fp``, ``snnlif_bn_fire_bp``) at the headline shape through the C ABI: 4 B per
 neuron-step for the batch statistics, 8 B forward, 20 B backward (two sweeps over x and the spike
 gradient, one write of the input gradient), checked against the CPU oracle on a sample of channels.
+
+``--workload policy_sweep`` lists forward / backward kernel rates in both cache policies over some twenty
+shapes (the reference's callers, window lengths, tensor sizes, odd row pitches, odd neuron counts).
 
 ``--workload bn`` does the same for the plain batch norm (``snnlif_bn_stats``, ``snnlif_bn_fp``,
 ``snnlif_bn_bp``): 4 + 8 + 20 B per element.
@@ -535,12 +539,100 @@ def run_bn(args, plain):
     print(json.dumps(result), flush=True)
 
 
+# Shapes of the policy sweep: the reference's own callers of Fire, window lengths 4-32 at about 256 MiB,
+# tensor sizes 8 MiB - 1 GiB at 8 steps, row pitches that are an odd multiple of 4 KiB, neuron counts
+# that are not a multiple of the workgroup size.
+SWEEP_SHAPES = [
+    ((6, 64, 4096), "Alexnet_BN_DIST.fire (models.py:78,100)"),
+    ((6, 64, 512, 7, 7), "Resnet_DIST.fire (models.py:145,183)"),
+    ((4, 64, 256, 32, 32), "T=4, 256 MiB"),
+    ((6, 64, 128, 32, 32), "T=6, 192 MiB"),
+    ((8, 64, 128, 32, 32), "T=8, 256 MiB (configuration 2)"),
+    ((12, 64, 64, 32, 32), "T=12, 192 MiB"),
+    ((16, 64, 64, 32, 32), "T=16, 256 MiB"),
+    ((24, 32, 64, 32, 32), "T=24, 192 MiB"),
+    ((32, 32, 256, 16, 16), "T=32, 256 MiB (configuration 3)"),
+    ((8, 64, 4, 32, 32), "T=8, 8 MiB"),
+    ((8, 64, 16, 32, 32), "T=8, 32 MiB"),
+    ((8, 64, 32, 32, 32), "T=8, 64 MiB"),
+    ((8, 64, 64, 32, 32), "T=8, 128 MiB"),
+    ((8, 64, 256, 32, 32), "T=8, 512 MiB"),
+    ((8, 64, 512, 32, 32), "T=8, 1 GiB"),
+    ((16, 128, 512, 16, 16), "T=16, 1 GiB (configuration 5)"),
+    ((8, 63, 127, 32, 32), "T=8, row pitch 8001 x 4 KiB"),
+    ((16, 65, 63, 32, 32), "T=16, row pitch 4095 x 4 KiB"),
+    ((32, 33, 61, 32, 32), "T=32, row pitch 2013 x 4 KiB"),
+    ((8, 63, 127, 31, 33), "T=8, N = 8185023 (odd)"),
+    ((6, 50, 100, 17, 19), "T=6, N = 1615000, 37 MiB"),
+    ((20, 32, 64, 32, 32), "T=20 (no instantiation of its own), 160 MiB"),
+]
+
+
+def run_policy_sweep(args):
+    """Forward and backward kernel rates in both cache policies over shapes the launch policy was not
+    tuned on.  Streamed: rotation over independent tensor sets (cold cache), SNNLIF_STREAM_SPATIAL; kept:
+    one tensor set, backward straight after the forward, SNNLIF_KEEP_SPATIAL.  Kernel durations from
+    events attached to the dispatches.  `no_hint` names the policy the library picks by itself."""
+    import torch
+    from snn_gpu_training_bptt_amd import lif_cabi
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no ROCm GPU visible")
+    lif_cabi.load()
+    dev = torch.device("cuda:0")
+    rows = []
+    for shape, what in SWEEP_SHAPES:
+        T = shape[0]
+        ns = 1
+        for d in shape:
+            ns *= d
+        gen = torch.Generator(device=dev).manual_seed(SEED)
+        x = 0.5 + torch.randn(shape, generator=gen, device=dev)
+        g = torch.randn(shape, generator=gen, device=dev)
+        tensor_bytes = ns * 4
+        sets = tensor_sets(tensor_bytes)
+        xs = [x] + [x.clone() for _ in range(sets - 1)]
+        gs = [g] + [g.clone() for _ in range(sets - 1)]
+        spikes = [torch.empty_like(x) for _ in range(sets)]
+        gxs = [torch.empty_like(x) for _ in range(sets)]
+        steps = max(sets * 3, 12)
+        streamed = rotation_leg(
+            torch, lif_cabi, sets, steps, sets,
+            lambda j: lif_cabi.fire_s_fp_into(xs[j], spikes[j], ALPHA, THRESH, keep_spatial=False),
+            lambda j: lif_cabi.fire_bp_into(xs[j], gs[j], gxs[j], ALPHA, THRESH, BETA, INTERVAL, keep_spatial=False),
+            8 * ns, 12 * ns, ns, instrumented=steps)
+        s_ref, gx_ref = spikes[0].clone(), gxs[0].clone()
+        kept = rotation_leg(
+            torch, lif_cabi, 1, 24, 4,
+            lambda j: lif_cabi.fire_s_fp_into(x, spikes[0], ALPHA, THRESH, keep_spatial=True),
+            lambda j: lif_cabi.fire_bp_into(x, g, gxs[0], ALPHA, THRESH, BETA, INTERVAL, keep_spatial=True),
+            8 * ns, 12 * ns, ns, instrumented=24)
+        same = bool(torch.equal(spikes[0], s_ref) and torch.equal(gxs[0], gx_ref))
+        rows.append({"shape": list(shape), "what": what, "tensor_MiB": round(tensor_bytes / 2**20, 1),
+                     "row_pitch_bytes": ns // T * 4, "no_hint": "kept" if tensor_bytes <= (32 << 20) else "streamed",
+                     "streamed": {"fwd_us": streamed["fwd"]["avg_launch_ms"] * 1e3, "fwd_frac": streamed["fwd"]["frac"],
+                                  "bwd_us": streamed["bwd"]["avg_launch_ms"] * 1e3, "bwd_frac": streamed["bwd"]["frac"],
+                                  "pair_frac": streamed["fwd_bwd"]["frac"]},
+                     "kept": {"fwd_us": kept["fwd"]["avg_launch_ms"] * 1e3, "fwd_frac": kept["fwd"]["frac"],
+                              "bwd_us": kept["bwd"]["avg_launch_ms"] * 1e3, "bwd_frac": kept["bwd"]["frac"],
+                              "pair_frac": kept["fwd_bwd"]["frac"]},
+                     "policies_agree_bit_for_bit": same})
+        print(f"{str(list(shape)):24s} {rows[-1]['tensor_MiB']:7.1f} MiB | streamed fwd {rows[-1]['streamed']['fwd_frac']:.3f} "
+              f"bwd {rows[-1]['streamed']['bwd_frac']:.3f} | kept fwd {rows[-1]['kept']['fwd_frac']:.3f} "
+              f"bwd {rows[-1]['kept']['bwd_frac']:.3f} | {what}", file=sys.stderr, flush=True)
+        del xs, gs, spikes, gxs, x, g, s_ref, gx_ref
+        torch.cuda.empty_cache()
+    print(json.dumps({"metric": "LIF fire kernel rates over shapes (fraction of the 8 TB/s HBM peak of algorithmic bytes; "
+                                "not the headline metric)", "unit": "fraction of peak", "n_gpus": 1, "dtype": "f32",
+                      "data": "synthetic", "config": {"workload": "policy_sweep"}, "rows": rows}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step", "bn_fire", "bn"])
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step", "bn_fire", "bn", "policy_sweep"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-legs", "--no-cold-leg", dest="no_extra_legs", action="store_true",
                     help="run the timed region only (fire workloads: no cabi_streamed / same_tensors / kept "
@@ -561,6 +653,9 @@ def main():
         if args.warmup == 20:
             args.warmup = 3
         return run_train_step(args)
+
+    if args.workload == "policy_sweep":
+        return run_policy_sweep(args)
 
     if args.workload in ("bn_fire", "bn"):
         return run_bn(args, plain=args.workload == "bn")

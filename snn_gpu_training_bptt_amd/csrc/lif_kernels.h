@@ -29,9 +29,10 @@
 //     membrane tensor to HBM and reading it back: 12 bytes per neuron-step instead of 20.
 //     Gradient rows are streamed in reverse time order through a double-buffered register window.
 //     The register-resident window needs compile-time row indices, so the kernel is instantiated
-//     per window length; lengths without an instantiation of their own run the next larger one
-//     with the missing rows replaced by zeros (no per-row control flow around live registers,
-//     which costs the compiler hundreds of VGPRs).
+//     per window length (1-8, then multiples of 2, 4 and 8); every other length runs the multiple
+//     of 8 below it as a straight-line body preceded by a head of up to 7 steps, the only rows
+//     behind run-time tests (per-row control flow around the whole window costs the compiler
+//     hundreds of VGPRs).
 //   * The op is element-wise and HBM-bound: no LDS, no cross-lane traffic, no MFMA.
 //   * Cache policy and launch shape follow what the caller says about the input current x
 //     (template parameter KEEP of the kernels, SNNLIF_KEEP_SPATIAL of the C ABI):
@@ -53,8 +54,8 @@
 //     element-wise CPU/GPU ops do, which makes spikes, potentials and gradients bit-identical to
 //     the per-op rounded reference arithmetic.
 //
-// Windows of a multiple of 8 steps up to 104 (64 with fp64 arithmetic) still run as one register window.  Other longer windows
-// (32 < T <= 1024) are cut into 32-step segments: one forward pass leaves the
+// Windows of up to 111 steps (71 with fp64 arithmetic; bf16 with a head up to 63) still run as one
+// register window.  Other longer windows (up to 1024 steps) are cut into 32-step segments: one forward pass leaves the
 // membrane potential at the segment boundaries in LDS, then each segment is recomputed into registers
 // and swept in reverse, last segment first (x is read twice, nothing else changes).  Beyond that the
 // forward kernel writes u to a caller-provided workspace and a streaming reverse kernel reads it back.
@@ -164,6 +165,10 @@
 // streamed with the next group of rows in flight).
 #ifndef SNNLIF_FWD_ROWS
 #define SNNLIF_FWD_ROWS 8
+#endif
+// Backward windows longer than this fix their instruction schedule (see backward_window).
+#ifndef SNNLIF_BWD_PIN_MIN_TW
+#define SNNLIF_BWD_PIN_MIN_TW 32
 #endif
 // Rows of the gradient held in flight per buffer of the backward's reverse sweep.
 #ifndef SNNLIF_BWD_GCHUNK
@@ -444,11 +449,15 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 // left.  A wavefront then keeps W loads outstanding from its first instruction to its last group and
 // issues loads and stores alternately, instead of a burst of requests followed by a burst of stores.
 // ---------------------------------------------------------------------------------------------
-// Used for streamed windows of a multiple of SNNLIF_FWD_ROLLING_W steps from SNNLIF_FWD_ROLLING_MIN_T on.
+// RAGGED: the window is not a multiple of W steps; refills past its end are skipped and the last
+// group is partial (tests that do not depend on the lane).
+// Used for streamed windows from SNNLIF_FWD_ROLLING_MIN_T steps on.
 // Measured cold on MI355X against the burst form (32 rows at once at 3 wavefronts per SIMD, groups of 16
 // beyond), fp32, % of the HBM peak: 32 steps 71.9 -> 73.1 (256 MiB tensors), 63.4 -> 65.7 (128 MiB),
 // 76.8 -> 77.8 (512 MiB); 64 steps 59.7 -> 67.0; 96 steps 66.2 -> 70.7.  16 rows at 2 wavefronts per SIMD
 // is the best of 4 / 8 / 16 / 32 rows at 1-8 wavefronts (8 rows at 4: 66 % at 32 steps; 16 rows at 1: 64 %).
+// Ragged windows against bursts of 16 rows: 40 steps 71.5 -> 75, 50 steps 67.5 -> 71, 100 steps 66 -> 70.5;
+// below 32 steps the ragged form is no better than the bursts (20 steps 73 -> 71, 24 steps +1, 28 steps -1).
 #ifndef SNNLIF_FWD_ROLLING_W
 #define SNNLIF_FWD_ROLLING_W 16
 #endif
@@ -458,7 +467,7 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 #ifndef SNNLIF_FWD_ROLLING_WAVES
 #define SNNLIF_FWD_ROLLING_WAVES 2
 #endif
-template <typename S, typename M, int V, int W, bool WRITE_U, bool WRITE_S, bool KEEP>
+template <typename S, typename M, int V, int W, bool WRITE_U, bool WRITE_S, bool KEEP, bool RAGGED = false>
 __global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(SNNLIF_FWD_ROLLING_WAVES)
 lif_forward_rolling_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__ spike, int T,
                            int64_t N, int64_t nvec, typename Arith<S>::type alpha,
@@ -492,11 +501,13 @@ lif_forward_rolling_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __re
                 const int64_t off = static_cast<int64_t>(t0 + k) * N + col;
                 if (WRITE_U) store_pack<M, V>(mem + off, mo);
                 if (WRITE_S) store_pack<S, V>(spike + off, so);
-                buf[k] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(t0 + W + k) * N + col);
+                if (!RAGGED || t0 + W + k < T)
+                    buf[k] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(t0 + W + k) * N + col);
             }
         }
 #pragma unroll
         for (int k = 0; k < W; ++k) {
+            if (RAGGED && t0 + k >= T) break;
             Pack<M, V> mo;
             Pack<S, V> so;
 #pragma unroll
@@ -527,8 +538,16 @@ lif_forward_rolling_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __re
 // KEEP: x is loaded with the default cache policy, otherwise with the non-temporal hint.
 // GSHARED: the gradient is one row that stands for every step of the window (GN == 0): it is loaded
 // once instead of once per step.
+// HEAD > 0: the window is preceded by `head` (0 <= head <= HEAD, the same for all lanes) further rows,
+// at rows -head .. -1 relative to the row pointers, which are part of the same register window: their
+// loads are issued with the window's (behind run-time tests that do not depend on the lane, around a
+// handful of registers only), their potentials are recomputed first and swept last.  A window of any
+// length then runs as a straight-line body of a multiple of 8 steps plus a head of up to 7, and still
+// reads every operand once.
 // ---------------------------------------------------------------------------------------------
-template <typename S, int V, int TW, bool EXACT, bool KEEP = true, bool GSHARED = false>
+constexpr int kHeadMax = 7;
+
+template <typename S, int V, int TW, bool EXACT, bool KEEP = true, bool GSHARED = false, int HEAD = 0>
 __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S* __restrict__ g,
                                                 S* __restrict__ gx, int rows, int64_t N,
                                                 int64_t GN, int64_t col,
@@ -538,12 +557,37 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
                                                 typename Arith<S>::type alpha,
                                                 typename Arith<S>::type thresh,
                                                 typename Arith<S>::type beta,
-                                                typename Arith<S>::type interval) {
+                                                typename Arith<S>::type interval, int head = 0) {
     using C = typename Arith<S>::type;
     constexpr int GC = (TW < SNNLIF_BWD_GCHUNK) ? TW : SNNLIF_BWD_GCHUNK;
     constexpr int NG = (TW + GC - 1) / GC;  // groups; group 0 holds the newest rows
     // group q covers rows [lo(q), hi(q)) with hi(q) = TW - q*GC and lo(q) = max(0, hi(q) - GC)
+    constexpr int HS = HEAD > 0 ? HEAD : 1;
+    // Windows with a head and all windows beyond SNNLIF_BWD_PIN_MIN_TW steps pin the order "requests of
+    // the window, recomputation, then per group: requests of the next group, sweep and stores of this
+    // one" with scheduling barriers.  Left to itself the compiler keeps that order for most window
+    // lengths but falls back to one request at a time, each followed by a full wait, for some (fp32 40
+    // steps; fp64 48 and 64; bf16 40 and 72-104 with one neuron per lane; every window with a head):
+    // 33 % of the HBM peak instead of 75 % for the 40-step window.  Up to 32 steps no instantiation is
+    // affected and the free schedule (all requests up front) measures 1-2 points better.
+    constexpr bool kPinned = HEAD > 0 || (EXACT && TW > SNNLIF_BWD_PIN_MIN_TW);
+    static_assert(HEAD == 0 || (EXACT && !GSHARED), "a head goes with a straight-line body");
 
+    // slot k: row k - head, present when k < head.  Both operands of the head are requested here, ahead
+    // of the body's rows, and its potentials are formed with selects: no branch lies between the body's
+    // first load and its last store, so the body keeps the instruction order of the window without a head.
+    Pack<S, V> xhead[HS], ghead[HS];
+    if constexpr (HEAD > 0) {
+#pragma unroll
+        for (int k = 0; k < HEAD; ++k) {
+            xhead[k] = zero_pack<S, V>();
+            ghead[k] = zero_pack<S, V>();
+            if (k < head) {
+                xhead[k] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(k - head) * N + col);
+                ghead[k] = load_pack<S, V, true>(g + static_cast<int64_t>(k - head) * GN + col);
+            }
+        }
+    }
     Pack<S, V> xin[TW];
 #pragma unroll
     for (int t = 0; t < TW; ++t) {
@@ -569,6 +613,24 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
         }
     }
 
+    if constexpr (HEAD == 0 && kPinned) __builtin_amdgcn_sched_barrier(0);
+    C uhead[HS][V];
+    if constexpr (HEAD > 0) {
+        // everything requested so far stays ahead of the arithmetic (with the head's registers live
+        // across the body the compiler otherwise falls back to one load at a time)
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int k = 0; k < HEAD; ++k) {
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                C un = uc[j], sn = sc[j];
+                lif_step<C>(un, sn, Arith<S>::load(xhead[k].e[j]), alpha, thresh);
+                uc[j] = k < head ? un : uc[j];
+                sc[j] = k < head ? sn : sc[j];
+                uhead[k][j] = uc[j];
+            }
+        }
+    }
     C u[TW][V];
 #pragma unroll
     for (int t = 0; t < TW; ++t) {
@@ -599,6 +661,8 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
                 }
             }
         }
+        // with a head: each group's requests stay ahead of the group before it being consumed
+        if constexpr (kPinned) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int t = hi - 1; t >= lo; --t) {
             if (EXACT || t < rows) {
@@ -611,6 +675,22 @@ __device__ __forceinline__ void backward_window(const S* __restrict__ x, const S
                     out.e[j] = Arith<S>::store(gu[j]);
                 }
                 store_pack<S, V>(gx + static_cast<int64_t>(t) * N + col, out);
+            }
+        }
+        if constexpr (kPinned) __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (HEAD > 0) {
+#pragma unroll
+        for (int k = HEAD - 1; k >= 0; --k) {
+            if (k < head) {
+                Pack<S, V> out;
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    lif_reverse_step<C>(gu[j], uhead[k][j], Arith<S>::load(ghead[k].e[j]), alpha, thresh,
+                                        beta, interval);
+                    out.e[j] = Arith<S>::store(gu[j]);
+                }
+                store_pack<S, V>(gx + static_cast<int64_t>(k - head) * N + col, out);
             }
         }
     }
@@ -626,10 +706,11 @@ __device__ __forceinline__ int64_t backward_column(int64_t v, int64_t nvec, int 
 }
 
 // ---------------------------------------------------------------------------------------------
-// Fused backward for T <= TW: the whole time axis is one register window.
+// Fused backward for T <= TW: the whole time axis is one register window.  HEAD > 0: for
+// TW < T <= TW + HEAD, the first T - TW steps being the window's head (see backward_window).
 // ---------------------------------------------------------------------------------------------
-template <typename S, int V, int TW, bool EXACT, bool KEEP, bool GSHARED = false>
-__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW, KEEP))
+template <typename S, int V, int TW, bool EXACT, bool KEEP, bool GSHARED = false, int HEAD = 0>
+__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW + HEAD, KEEP))
 lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
                           int T, int64_t N, int64_t GN, int64_t nvec,
                           typename Arith<S>::type alpha, typename Arith<S>::type thresh,
@@ -646,8 +727,11 @@ lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* _
             sc[j] = C(0);
             gu[j] = C(0);
         }
-        backward_window<S, V, TW, EXACT, KEEP, GSHARED>(x, g, gx, T, N, GN, col, uc, sc, gu, alpha,
-                                                        thresh, beta, interval);
+        const int head = HEAD > 0 ? T - TW : 0;
+        backward_window<S, V, TW, EXACT, KEEP, GSHARED, HEAD>(
+            x + static_cast<int64_t>(head) * N, g + static_cast<int64_t>(head) * GN,
+            gx + static_cast<int64_t>(head) * N, T - head, N, GN, col, uc, sc, gu, alpha, thresh, beta,
+            interval, head);
     }
 }
 
@@ -902,8 +986,8 @@ int launch_forward_rows(const S* x, M* mem, S* spike, int64_t T, int64_t N, floa
 // window of 9-16 rows as one group measures +5-8 points over two groups of 8), and so are windows
 // of 24-32 rows, in a 32-row instantiation at 3 wavefronts per SIMD (+3-5 points over two groups of
 // 16; a 20-row window zero-filled to 32 loses 4-8, so 17-23 rows stay in groups).  Everything else
-// goes in groups of 16 (groups of 32 gain 3-4 points at 48 and 64 rows and lose 1-7 from 96 on), except
-// windows of a multiple of 16 rows from 32 on, which run the rolling-window kernel.
+// goes in groups of 16, i.e. the windows of 17-23 rows: from 32 rows on every window runs the
+// rolling-window kernel.
 template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S, bool KEEP>
 int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
                      hipStream_t stream) {
@@ -924,12 +1008,19 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
     }
     if (T <= TC) return SNNLIF_FWD_LAUNCH(TC, false);
     if constexpr (!KEEP && SNNLIF_FWD_ROLLING_W > 0) {
-        if (T >= SNNLIF_FWD_ROLLING_MIN_T && T > SNNLIF_FWD_ROLLING_W && T % (SNNLIF_FWD_ROLLING_W > 0 ? SNNLIF_FWD_ROLLING_W : 1) == 0) {
+        constexpr int W = SNNLIF_FWD_ROLLING_W > 0 ? SNNLIF_FWD_ROLLING_W : 1;
+        if (T >= SNNLIF_FWD_ROLLING_MIN_T && T > W) {
             using C = typename Arith<S>::type;
             const int64_t nvec = N / V;
-            launch_kernel(lif_forward_rolling_kernel<S, M, V, (SNNLIF_FWD_ROLLING_W > 0 ? SNNLIF_FWD_ROLLING_W : 1), WRITE_U, WRITE_S, KEEP>,
-                          dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
-                          static_cast<int>(T), N, nvec, C(alpha), C(thresh));
+            const dim3 grid(grid_for(nvec, threads)), block(threads);
+            if (T % W == 0)
+                launch_kernel(lif_forward_rolling_kernel<S, M, V, W, WRITE_U, WRITE_S, KEEP, false>, grid,
+                              block, 0, stream, x, mem, spike, static_cast<int>(T), N, nvec, C(alpha),
+                              C(thresh));
+            else
+                launch_kernel(lif_forward_rolling_kernel<S, M, V, W, WRITE_U, WRITE_S, KEEP, true>, grid,
+                              block, 0, stream, x, mem, spike, static_cast<int>(T), N, nvec, C(alpha),
+                              C(thresh));
             return launch_status();
         }
     }
@@ -1028,10 +1119,7 @@ int launch_backward_fused_policy(const S* x, const S* g, S* gx, int64_t T, int64
     const void* ptrs[3] = {x, g, gx};
     const size_t elem[3] = {sizeof(S), sizeof(S), sizeof(S)};
     const int v = pick_vec(maxv, N, ptrs, elem, 3, GN);
-    // Every window of at most 8 rows has an instantiation of its own, so only the longer ones
-    // are ever entered with T < TW; windows beyond the fused range are entered with T == TW only.
-    constexpr bool can_be_inexact = TW > 8 && TW <= SNNLIF_BP_FUSED_MAX_T;
-    const bool exact = !can_be_inexact || (T == TW);
+    // always entered with T == TW: every other length takes the form with a head
     return with_vec<maxv>(v, [&](auto vc) {
         constexpr int V = decltype(vc)::value;
         const int64_t nvec = N / V;
@@ -1039,19 +1127,16 @@ int launch_backward_fused_policy(const S* x, const S* g, S* gx, int64_t T, int64
             backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S), 64, KEEP);
         const dim3 grid(grid_for(nvec, threads)), block(threads);
         const int Ti = static_cast<int>(T);
-        // one gradient row for all steps, window with a straight-line instantiation of its own: the
-        // form that loads the row once (other lengths read it in place once per step)
+        // one gradient row for all steps: the form that loads the row once (windows with a head and
+        // the long ones read it in place once per step)
         constexpr bool has_shared = TW >= 2 && TW <= SNNLIF_BP_FUSED_MAX_T;
-        if (exact && GN == 0 && has_shared) {
+        if (GN == 0 && has_shared) {
             if constexpr (has_shared)
                 launch_kernel(lif_backward_fused_kernel<S, V, TW, true, KEEP, true>, grid, block, 0,
                               stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta),
                               C(interval));
-        } else if (exact) {
+        } else {
             launch_kernel(lif_backward_fused_kernel<S, V, TW, true, KEEP>, grid, block, 0, stream,
-                               x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
-        } else if constexpr (can_be_inexact) {
-            launch_kernel(lif_backward_fused_kernel<S, V, TW, false, KEEP>, grid, block, 0, stream,
                                x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
         }
         return launch_status();
@@ -1067,6 +1152,34 @@ int launch_backward_fused(const S* x, const S* g, S* gx, int64_t T, int64_t N, i
                                                          interval, stream);
     return launch_backward_fused_policy<S, TW, false>(x, g, gx, T, N, GN, alpha, thresh, beta,
                                                       interval, stream);
+}
+
+// Windows of TB + 1 .. TB + kHeadMax steps, TB a multiple of 8: straight-line body with a head.
+template <typename S, int TB>
+int launch_backward_headed(const S* x, const S* g, S* gx, int64_t T, int64_t N, int64_t GN,
+                           float alpha, float thresh, float beta, float interval, SpatialHint keep_x,
+                           hipStream_t stream) {
+    using C = typename Arith<S>::type;
+    constexpr int maxv = fused_max_vec<S, TB + kHeadMax>();
+    const void* ptrs[3] = {x, g, gx};
+    const size_t elem[3] = {sizeof(S), sizeof(S), sizeof(S)};
+    const int v = pick_vec(maxv, N, ptrs, elem, 3, GN);
+    const size_t bytes = static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S);
+    const bool keep = keep_policy(keep_x, bytes);
+    return with_vec<maxv>(v, [&](auto vc) {
+        constexpr int V = decltype(vc)::value;
+        const int64_t nvec = N / V;
+        const int threads = backward_block(bytes, 64, keep);
+        const dim3 grid(grid_for(nvec, threads)), block(threads);
+        const int Ti = static_cast<int>(T);
+        if (keep)
+            launch_kernel(lif_backward_fused_kernel<S, V, TB, true, true, false, kHeadMax>, grid, block,
+                          0, stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
+        else
+            launch_kernel(lif_backward_fused_kernel<S, V, TB, true, false, false, kHeadMax>, grid, block,
+                          0, stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
+        return launch_status();
+    });
 }
 
 template <typename S, int V>
@@ -1092,12 +1205,24 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
     if (!aligned_to(x, sizeof(S)) || !aligned_to(g, sizeof(S)) || !aligned_to(gx, sizeof(S)))
         return SNNLIF_ERR_ALIGN;
 
-    // Window lengths with an instantiation of their own; any other T <= 32 runs the next larger
-    // one in its zero-filled form.
+    // Window lengths with a straight-line instantiation of their own (T == TW) ...
 #define SNNLIF_BWD_WINDOW(TW)                                                                    \
-    if (T <= TW)                                                                                 \
+    if (T == TW)                                                                                 \
         return launch_backward_fused<S, TW>(x, g, gx, T, N, GN, alpha, thresh, beta, interval,     \
                                             keep_x, stream);
+    // ... and every length between them: the multiple of 8 below it as a straight-line body, the
+    // first T % 8 steps as its head (see backward_window).  Against the next larger window with the
+    // absent rows replaced by zeros, which this form replaced, cold at 64 Mi elements, % of the HBM
+    // peak: fp32 18 steps 71 -> 76, 22 steps 69 -> 73.5, 26 steps 57 -> 73, 30 steps 66 -> 72 (9-15
+    // steps unchanged within a point); bf16 13 steps 61 -> 70, 26 steps 30 -> 70.
+#define SNNLIF_BWD_HEADED_WINDOW(TB)                                                             \
+    if constexpr (fused_max_vec<S, TB + kHeadMax>() >= Arith<S>::kMaxVec) {                       \
+        if (TB <= wide_max && T > TB && T <= TB + kHeadMax)                                      \
+            return launch_backward_headed<S, TB>(x, g, gx, T, N, GN, alpha, thresh, beta,         \
+                                                 interval, keep_x, stream);                      \
+    }
+    constexpr int64_t wide_max =
+        sizeof(C) == 4 ? SNNLIF_BWD_WIDE_MAX_T : SNNLIF_BWD_WIDE_MAX_T_F64;
     SNNLIF_BWD_WINDOW(1)
     SNNLIF_BWD_WINDOW(2)
     SNNLIF_BWD_WINDOW(3)
@@ -1114,6 +1239,9 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
     SNNLIF_BWD_WINDOW(28)
     SNNLIF_BWD_WINDOW(32)
 #undef SNNLIF_BWD_WINDOW
+    SNNLIF_BWD_HEADED_WINDOW(8)
+    SNNLIF_BWD_HEADED_WINDOW(16)
+    SNNLIF_BWD_HEADED_WINDOW(24)
     static_assert(SNNLIF_BP_FUSED_MAX_T == 32, "windows above must cover the fused range");
 
     // Windows of a multiple of 8 steps still fit the register file whole a good way further (u alone
@@ -1123,8 +1251,6 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
     // re-reads x; cold-cache backward at 64 Mi elements, fp32: 67-72 % of the HBM peak against
     // 54-65 %.  Only the exact length qualifies: the zero-filled form of these wide windows runs at
     // 40-58 %, below the segmented kernel.
-    constexpr int64_t wide_max =
-        sizeof(C) == 4 ? SNNLIF_BWD_WIDE_MAX_T : SNNLIF_BWD_WIDE_MAX_T_F64;
 #define SNNLIF_BWD_WIDE_WINDOW(TW)                                                               \
     if (TW <= wide_max && T == TW)                                                               \
         return launch_backward_fused<S, TW>(x, g, gx, T, N, GN, alpha, thresh, beta, interval,     \
@@ -1141,6 +1267,28 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
         SNNLIF_BWD_WIDE_WINDOW(104)
     }
 #undef SNNLIF_BWD_WIDE_WINDOW
+
+    // Every other length up to 7 steps past the longest of these, again as body + head.  Still 12
+    // bytes per neuron-step, where the segmented kernel below reads x twice.  Cold-cache backward at
+    // 64 Mi elements, % of the HBM peak of 12 bytes per neuron-step, segmented -> with a head: fp32
+    // 33 steps 66 -> 74, 39 steps 62 -> 68, 50 steps 62 -> 70, 60 steps 65 -> 71, 84 steps 62 -> 70,
+    // 100 steps 62 -> 68.5, 111 steps 56 -> 59; bf16 39 steps 54 -> 66, 47 steps 53 -> 64, 60 steps
+    // 57 -> 67.  Only while the register budget still allows full dword lanes: bf16 bodies from 64
+    // steps on would be down to one neuron per lane and lose to the segmented kernel (71 steps
+    // 50 -> 46, 100 steps 53 -> 50).
+    SNNLIF_BWD_HEADED_WINDOW(32)
+    SNNLIF_BWD_HEADED_WINDOW(40)
+    SNNLIF_BWD_HEADED_WINDOW(48)
+    SNNLIF_BWD_HEADED_WINDOW(56)
+    SNNLIF_BWD_HEADED_WINDOW(64)
+    if constexpr (sizeof(C) == 4) {
+        SNNLIF_BWD_HEADED_WINDOW(72)
+        SNNLIF_BWD_HEADED_WINDOW(80)
+        SNNLIF_BWD_HEADED_WINDOW(88)
+        SNNLIF_BWD_HEADED_WINDOW(96)
+        SNNLIF_BWD_HEADED_WINDOW(104)
+    }
+#undef SNNLIF_BWD_HEADED_WINDOW
 
     // Longer windows, up to what the boundary values of a workgroup fit into 64 KiB of LDS for
     // every storage type: segmented kernel, still no scratch memory in HBM.

@@ -82,9 +82,10 @@ CASES = [
     ((16, 2, 32, 8, 8), 0.5, 1.0),      # T=16
     ((32, 2, 16, 16, 16), 0.3, 0.8),    # T=32 (configuration 3's window)
     ((29, 2, 300), 0.3, 0.8),           # T=29 inside the T<=32 window
-    ((33, 2, 16, 8, 8), 0.3, 0.8),      # first T beyond one register window: two segments
-    ((70, 3, 129), 0.3, 0.8),           # three segments, the last partial, odd N
-    ((64, 2, 500), 0.3, 0.8),           # exactly two full segments
+    ((33, 2, 16, 8, 8), 0.3, 0.8),      # 32-step body with a one-step head
+    ((70, 3, 129), 0.3, 0.8),           # 64-step body with a 6-step head, odd N
+    ((64, 2, 500), 0.3, 0.8),           # a 64-step register window
+    ((120, 2, 100), 0.3, 0.8),          # four segments, the last partial
     ((257, 2, 130), 0.2, 0.7),          # nine segments
     ((1024, 1, 192), 0.2, 0.7),         # the longest window kept on chip
     ((1030, 1, 64), 0.2, 0.7),          # beyond it: membrane potential staged in the workspace
@@ -107,9 +108,10 @@ def test_fp32_parity(cabi, oracle, shape, mean, std, keep):
 @HINTS
 @pytest.mark.parametrize("T", list(range(1, 35)))
 def test_fp32_every_window_length(cabi, oracle, T, keep):
-    """Each window length up to 32 maps to its own or the next larger register window; 33 and 34
-    are cut into two segments.  Even and odd N.  The streamed forward requests windows of 9 to 16
-    steps whole and longer ones in groups of 16."""
+    """Each window length up to 34 has a straight-line register window of its own or runs as the
+    multiple of 8 below it preceded by a head of 1 to 7 steps.  Even and odd N.  The streamed forward
+    requests windows of 9 to 16 and 24 to 31 steps whole, 17 to 23 in groups of 16, longer ones through
+    a rolling window."""
     for n_inner in (256, 77):
         x, g = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=1000 + T)
         assert_parity(oracle, x, g, run_gpu(cabi, x, g, alpha=0.3, keep=keep), alpha=0.3)
@@ -151,11 +153,13 @@ def test_windows_between_64_and_128(cabi, oracle, T, dtype, keep):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
-@pytest.mark.parametrize("T", [32, 48, 64, 160, 1040])
-def test_streamed_windows_of_a_multiple_of_16_steps(cabi, oracle, T, dtype):
+@pytest.mark.parametrize("T", [32, 33, 40, 47, 48, 49, 63, 64, 65, 100, 160, 161, 175, 1040, 1047])
+def test_streamed_windows_from_32_steps_on(cabi, oracle, T, dtype):
     """The streamed forward of these windows is the rolling-window kernel (16 rows in flight, refilled
-    row by row): spikes, the membrane output and, for the 1040-step window, the potential it stages in
-    the backward's workspace (fp32 behind bf16 storage) must be the oracle's bits.  Even and odd N."""
+    row by row; lengths that are not a multiple of 16 skip the refills past the end and finish on a
+    partial group of 1 to 15 rows): spikes, the membrane output and, beyond 1024 steps, the potential it
+    stages in the backward's workspace (fp32 behind bf16 storage) must be the oracle's bits.  Even and
+    odd N."""
     wide = torch.float64 if dtype == torch.float64 else torch.float32
     for n_inner in (256, 77):
         x32, g32 = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=9000 + T)
@@ -167,6 +171,48 @@ def test_streamed_windows_of_a_multiple_of_16_steps(cabi, oracle, T, dtype):
         assert torch.equal(spike_a, as_stored(spike_o)) and torch.equal(spike_b, as_stored(spike_o))
         assert torch.equal(mem, as_stored(mem_o))
         assert torch.equal(gx, as_stored(gx_o))
+
+
+@HINTS
+@pytest.mark.parametrize("T", list(range(33, 114)))
+def test_fp32_windows_with_a_head(cabi, oracle, T, keep):
+    """Backward windows of 33 to 111 steps that are not a multiple of 8 run as a straight-line body of a
+    multiple of 8 steps preceded by a head of 1-7 steps (every operand read once); multiples of 8 up to
+    104 run without a head, 112 and 113 steps are the first lengths cut into segments again.  Every
+    length, both instantiations, a negative threshold (a wrong spike flag or potential at the seam between
+    head and body would show), odd N."""
+    x, g = make_inputs((T, 3, 77), 0.1, 0.9, seed=11000 + T)
+    xd, gd = x.cuda(), g.cuda()
+    gx = torch.empty_like(xd)
+    cabi.fire_bp_into(xd, gd, gx, 0.3, -0.25, BETA, INTERVAL, keep_spatial=keep)
+    torch.cuda.synchronize()
+    gx_o = oracle.fire_backward(x.numpy(), g.numpy(), 0.3, -0.25, BETA, INTERVAL)
+    assert np.array_equal(gx.cpu().numpy(), gx_o)
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("T", [33, 36, 39, 41, 47, 63, 65, 71, 73, 79, 100, 103, 105, 111])
+def test_windows_with_a_head_other_storage_types(cabi, oracle, T, dtype):
+    """The same in fp64 (heads up to a 64-step body, i.e. 71 steps; longer windows are segmented) and
+    bf16 (two neurons per lane when N is even; bodies from 64 steps on stay segmented), with a dense gradient and with one row of gradient that
+    stands for every step (row stride 0)."""
+    wide = torch.float64 if dtype == torch.float64 else torch.float32
+    for n_inner in (128, 77):
+        x32, g32 = make_inputs((T, 2, n_inner), 0.1, 0.9, seed=12000 + T)
+        x, g = x32.to(dtype), g32.to(dtype)
+        for keep in (True, False):
+            xd, gd = x.cuda(), g.cuda()
+            gx = torch.empty_like(xd)
+            cabi.fire_bp_into(xd, gd, gx, 0.3, THRESH, BETA, INTERVAL, keep_spatial=keep)
+            gx1 = torch.empty_like(xd)
+            cabi.fire_bp_into(xd, gd[:1].expand_as(xd), gx1, 0.3, THRESH, BETA, INTERVAL, keep_spatial=keep)
+            torch.cuda.synchronize()
+            xw, gw = x.to(wide).numpy(), g.to(wide).numpy()
+            gx_o = oracle.fire_backward(xw, gw, 0.3, THRESH, BETA, INTERVAL)
+            gx1_o = oracle.fire_backward(xw, np.ascontiguousarray(np.broadcast_to(gw[:1], gw.shape)), 0.3,
+                                         THRESH, BETA, INTERVAL)
+            assert torch.equal(gx.cpu(), torch.from_numpy(gx_o).to(dtype))
+            assert torch.equal(gx1.cpu(), torch.from_numpy(gx1_o).to(dtype))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
@@ -352,7 +398,7 @@ def test_gradient_expanded_over_time_is_read_in_place(cabi, oracle, T, dtype, ke
     """A gradient that is one [N] row for every time step (stride 0 on the time axis, what autograd
     hands over after ``spike.sum(dim=0)``) goes to ``snnlif_fire_bp_strided`` as it is.  The result
     must be the oracle's on the gradient made dense, and the bits of the dense call: every kernel
-    form of the backward (register windows exact and zero-filled, wide windows, segments, workspace
+    form of the backward (register windows with and without a head, wide windows, segments, workspace
     stream) takes the row stride.  Even N (pairs of bf16 per lane) and odd N."""
     for n_inner in (256, 77):
         x32, g32 = make_inputs((T, 2, n_inner), 0.4, 0.9, seed=5000 + T)
