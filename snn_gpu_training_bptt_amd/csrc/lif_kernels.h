@@ -381,10 +381,10 @@ __device__ __forceinline__ void lif_reverse_step(C& gu, C u, C g, C alpha, C thr
 // TC: rows requested before the first is consumed.  MULTI = false: the whole window fits in TC
 // rows.  MULTI = true: the window is streamed TC rows at a time with the next TC rows already in
 // flight while the current ones are processed.  KEEP: x is loaded with the default cache policy
-// (see the file header); otherwise with the non-temporal hint.
+// (see the file header); otherwise with the non-temporal hint.  FULL: T == TC, no test around any row.
 // ---------------------------------------------------------------------------------------------
 template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP,
-          bool CAPPED = false>
+          bool CAPPED = false, bool FULL = false>
 __global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(forward_waves(TC, KEEP, CAPPED))
 lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__ spike, int T,
                    int64_t N, int64_t nvec, typename Arith<S>::type alpha,
@@ -404,7 +404,7 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
         Pack<S, V> nxt[MULTI ? TC : 1];
 #pragma unroll
         for (int k = 0; k < TC; ++k) {
-            if (k < T)
+            if (FULL || k < T)
                 cur[k] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(k) * N + col);
         }
         for (int t0 = 0; t0 < T; t0 += TC) {
@@ -420,7 +420,7 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
 #pragma unroll
             for (int k = 0; k < TC; ++k) {
                 const int t = t0 + k;
-                if (t < T) {
+                if (FULL || t < T) {
                     Pack<M, V> mo;
                     Pack<S, V> so;
 #pragma unroll
@@ -975,6 +975,19 @@ int launch_forward_rows(const S* x, M* mem, S* spike, int64_t T, int64_t N, floa
                         int threads, hipStream_t stream) {
     using C = typename Arith<S>::type;
     const int64_t nvec = N / V;
+    // A window that fills the instantiation can run without the tests around each row.  Measured
+    // cold: fp64 windows of 8 / 16 steps 62 -> 71 % / 51 -> 65.5 % of the HBM peak (behind the tests the
+    // compiler waits for each 8-byte load before it issues the next); fp32 +1 point for the capped
+    // 8-step window and for 4 steps, -0.5 to -1.5 for 16 steps and for tensors beyond 256 MiB; bf16 -0.5.
+    constexpr bool can_fill = !MULTI && (sizeof(S) == 8 || (sizeof(S) == 4 && (CAPPED || TC == 4)));
+    if constexpr (can_fill) {
+        if (T == TC) {
+            launch_kernel(lif_forward_kernel<S, M, V, TC, false, WRITE_U, WRITE_S, KEEP, CAPPED, true>,
+                          dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
+                          static_cast<int>(T), N, nvec, C(alpha), C(thresh));
+            return launch_status();
+        }
+    }
     launch_kernel(lif_forward_kernel<S, M, V, TC, MULTI, WRITE_U, WRITE_S, KEEP, CAPPED>,
                   dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
                   static_cast<int>(T), N, nvec, C(alpha), C(thresh));
