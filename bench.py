@@ -85,8 +85,11 @@ WORKLOADS = {
     # no configuration of the reference: a 96-step window, the longest range of the backward that
     # still recomputes the whole window in registers (67 239 936 neuron-steps, 257 MiB per tensor)
     "t96": ((96, 4, 171, 32, 32), 0.5, 1.0, "float32"),
-    # ... and a 100-step one, which the backward cuts into 32-step segments (67 174 400 neuron-steps)
+    # ... a 100-step one, which the backward runs as a 96-step body with a 4-step head (67 174 400
+    # neuron-steps) ...
     "t100": ((100, 4, 164, 32, 32), 0.5, 1.0, "float32"),
+    # ... and a 120-step one, which it cuts into 32-step segments (67 338 240 neuron-steps)
+    "t120": ((120, 4, 137, 32, 32), 0.5, 1.0, "float32"),
 }
 # HBM bytes per launch of the backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs
 # of this file (each counter scaled by its reading for a plain device copy of the same tensor:
@@ -99,6 +102,7 @@ TRAFFIC_PROFILES = {
     "cfg5_bf16": "profiles/pmc_fetch_write_fire_fwd_bwd_cfg5_bf16.txt",
     "t96": "profiles/pmc_fetch_write_fire_fwd_bwd_t96_f32.txt",
     "t100": "profiles/pmc_fetch_write_fire_fwd_bwd_t100_f32.txt",
+    "t120": "profiles/pmc_fetch_write_fire_fwd_bwd_t120_f32.txt",
     "bn_fire": "profiles/pmc_fetch_write_bn_fire_fwd_bwd_cfg2_f32.txt",
     "bn": "profiles/pmc_fetch_write_bn_fwd_bwd_cfg2_f32.txt",
 }
@@ -138,6 +142,18 @@ def metric_name(workload, shape, dtype_name):
         return METRIC
     T, B, C, H, W = shape
     return f"LIF fwd+bwd neuron-steps/s + HBM GB/s (% of peak), T={T},B={B},C={C},{H}x{W} {dtype_name} ({workload})"
+
+
+def backward_kernel_name(T, esize, lif_cabi):
+    """Which kernel the library launches for a backward window of T steps (fp32 arithmetic: fp32 or bf16
+    storage).  One register window (a multiple of 8 steps, or that plus a head of up to 7 steps) up to
+    111 steps (bf16 with a head: up to 63), 32-step segments up to 1024, the workspace stream beyond."""
+    if T > lif_cabi.BP_NO_WORKSPACE_MAX_T:
+        return "lif_backward_stream_kernel"
+    body = T // 8 * 8
+    whole = T <= lif_cabi.BP_FUSED_MAX_T or (T == body and T <= 104)
+    headed = body <= 104 and (esize == 4 or body + 7 <= 64)
+    return "lif_backward_fused_kernel" if whole or headed else "lif_backward_segmented_kernel"
 
 
 def make_inputs(torch, shape, mean, std, dtype):
@@ -564,7 +580,11 @@ SWEEP_SHAPES = [
     ((32, 33, 61, 32, 32), "T=32, row pitch 2013 x 4 KiB"),
     ((8, 63, 127, 31, 33), "T=8, N = 8185023 (odd)"),
     ((6, 50, 100, 17, 19), "T=6, N = 1615000, 37 MiB"),
-    ((20, 32, 64, 32, 32), "T=20 (no instantiation of its own), 160 MiB"),
+    ((20, 32, 64, 32, 32), "T=20, 160 MiB"),
+    ((26, 40, 64, 32, 32), "T=26 (24-step body + 2-step head), 260 MiB"),
+    ((40, 16, 100, 32, 32), "T=40, 250 MiB"),
+    ((100, 4, 164, 32, 32), "T=100 (96-step body + 4-step head), 256 MiB"),
+    ((120, 4, 137, 32, 32), "T=120 (segmented backward), 257 MiB"),
 ]
 
 
@@ -714,9 +734,7 @@ def main():
         all(torch.equal(q, gx) for q in gxs[1:] if q is not None)
     spikes, gxs = [spike], [gx]   # release the other sets' outputs
     spike_rate = float(spike.float().mean().item())
-    segmented = T > lif_cabi.BP_FUSED_MAX_T and not (T % 8 == 0 and T <= 104)
-    bwd_kernel = ("lif_backward_stream_kernel" if T > lif_cabi.BP_NO_WORKSPACE_MAX_T
-                  else "lif_backward_segmented_kernel" if segmented else "lif_backward_fused_kernel")
+    bwd_kernel = backward_kernel_name(T, esize, lif_cabi)
 
     result = {
         "metric": metric_name(args.workload, shape, dtype_name),

@@ -67,6 +67,9 @@
 
 #include <cstddef>
 #include <cstdint>
+#ifdef SNNLIF_LAB
+#include <cstdlib>
+#endif
 #include <tuple>
 #include <type_traits>
 
@@ -146,20 +149,13 @@
 #define SNNLIF_STREAM_FWD_WAVES_LONG 3
 #endif
 // Rows the streamed forward requests at once: windows of 9 rows up to the first run whole in that
-// instantiation, windows of at least three quarters of the second and up to it whole in that one;
-// all others go in groups of the first.
+// instantiation, windows up to halfway between the two in an instantiation of that many rows, longer
+// ones up to the second in that one.
 #ifndef SNNLIF_STREAM_FWD_ROWS_MID
 #define SNNLIF_STREAM_FWD_ROWS_MID 16
 #endif
 #ifndef SNNLIF_STREAM_FWD_ROWS_LONG
 #define SNNLIF_STREAM_FWD_ROWS_LONG 32
-#endif
-// ... and of the forward for a window of exactly 8 rows on a tensor of at most so many bytes.
-#ifndef SNNLIF_STREAM_FWD_WAVES_8
-#define SNNLIF_STREAM_FWD_WAVES_8 5
-#endif
-#ifndef SNNLIF_STREAM_FWD_CAPPED_BYTES
-#define SNNLIF_STREAM_FWD_CAPPED_BYTES (size_t(256) << 20)
 #endif
 // Rows of x the forward requests before consuming the first (windows longer than this are
 // streamed with the next group of rows in flight).
@@ -204,22 +200,42 @@ constexpr int backward_waves(int rows, bool keep = true) {
 #endif
 }
 
+// Streamed backward on tensors of at most SNNLIF_STREAM_SMALL_BYTES: windows of 4 to 16 steps run with
+// fewer wavefronts still (0: no instantiation of its own).  Measured cold over 2-8 wavefronts, fp32, %
+// of the HBM peak at this figure / at the one above: 4 steps on 128 MiB tensors 78.6 / 75.8, on 64 MiB
+// 70.5 / 69.2; 6 steps on 96 MiB 73.7 / 71.2; 7 steps on 112 MiB 73.8 / 70.3; 8 steps on 128 MiB
+// 72.8 / 68.8, on 64 MiB 73.4 / 70.1; 12 steps on 96 MiB 73.3 / 71.9; 16 steps on 128 MiB 73.4 / 71.5;
+// bf16 8 steps on 128 MiB 72.8 / 68.5.  Larger tensors are best at the figures above (8 steps on
+// 256 MiB: 84.6 % at 4 wavefronts, 83.1 at 5; on 512 MiB 82.6 / 83.3).
+constexpr int stream_backward_small_waves(int rows) {
+    return rows == 4 ? 5 : (rows >= 5 && rows <= 16) ? 3 : 0;
+}
+
 // The forward keeps `rows` (twice that when the window is streamed in groups) requests per wavefront
-// in flight; long streamed windows gain from a cap, and so does (`capped`) the streamed 8-step window
-// on tensors of up to SNNLIF_STREAM_FWD_CAPPED_BYTES: there the 16 row streams of the kernel sit a
-// power of two apart in the usual shapes, and with all 8 wavefronts resident the rate depends on
-// where the output tensor lies relative to the input (66 % of the HBM peak with the output right
-// behind the input, 78 % one tensor further; capped: 77-79 % either way; plain copies of 8 rows in
-// that layout behave the same: 68 / 76 % uncapped, 79 / 80 % at 4 wavefronts).  Windows of 5-7 steps
-// share the kernel but lose 2-10 points under the cap, larger tensors 2-3, so neither is capped.
-constexpr int forward_waves(int rows, bool keep, bool capped = false) {
+// in flight; long streamed windows gain from a cap.  `cap` > 0: the instantiation's own figure
+// (streamed windows of up to 8 steps, see stream_forward_waves).
+constexpr int forward_waves(int rows, bool keep, int cap = 0) {
 #ifdef SNNLIF_FWD_MAX_WAVES
     return SNNLIF_FWD_MAX_WAVES;
 #else
-    if (capped) return SNNLIF_STREAM_FWD_WAVES_8;
+    if (cap > 0) return cap;
     if (!keep && rows > SNNLIF_STREAM_FWD_ROWS_MID) return SNNLIF_STREAM_FWD_WAVES_LONG;
     return (!keep && rows > 8) ? SNNLIF_STREAM_FWD_WAVES_MID : 8;  // groups of SNNLIF_STREAM_FWD_ROWS_MID too
 #endif
+}
+
+// Wavefronts per SIMD of the streamed forward of a window of up to 8 steps (one of the instantiations
+// launch_forward_v lists).  Measured cold over 2-8 wavefronts, fp32, % of the HBM peak at the best / at
+// 8 wavefronts: 8 steps 78 / 76 (256 MiB tensors, best at 5), 80 / 79 (512 MiB, 5), 69 / 62 (128 MiB, 3);
+// 7 steps 77 / 76.5 (224 MiB, 5), 69 / 63.5 (112 MiB, 3); 6 steps 76 / 75 (192 MiB, 5), 68 / 64 (96 MiB,
+// 4); 5 steps 75 / 72.5 (160 MiB, 5-7), 68 / 67 (80 MiB, 5); 4 and 3 steps are best at 7-8 at every size
+// (3 steps: 72 % at 8, 63 % at 5); bf16 8 steps on 256 MiB tensors 81 / 76.5 (5).
+inline int stream_forward_waves(int rows, size_t tensor_bytes) {
+    const bool small = tensor_bytes <= static_cast<size_t>(SNNLIF_STREAM_SMALL_BYTES);
+    if (rows >= 7) return small ? 3 : 5;
+    if (rows == 6) return small ? 4 : 5;
+    if (rows == 5) return 5;
+    return 8;
 }
 
 constexpr int kLaneBytes = SNNLIF_LANE_BYTES;
@@ -381,11 +397,13 @@ __device__ __forceinline__ void lif_reverse_step(C& gu, C u, C g, C alpha, C thr
 // TC: rows requested before the first is consumed.  MULTI = false: the whole window fits in TC
 // rows.  MULTI = true: the window is streamed TC rows at a time with the next TC rows already in
 // flight while the current ones are processed.  KEEP: x is loaded with the default cache policy
-// (see the file header); otherwise with the non-temporal hint.  FULL: T == TC, no test around any row.
+// (see the file header); otherwise with the non-temporal hint.  CAP > 0: wavefronts per SIMD of this
+// instantiation.  FULL: T == TC; no test around any row, requests go out in time order and each row is
+// consumed and its result stored as soon as it has arrived.
 // ---------------------------------------------------------------------------------------------
 template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP,
-          bool CAPPED = false, bool FULL = false>
-__global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(forward_waves(TC, KEEP, CAPPED))
+          int CAP = 0, bool FULL = false>
+__global__ void __launch_bounds__(kFwdBlock) SNNLIF_WAVES_PER_SIMD(forward_waves(TC, KEEP, CAP))
 lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__ spike, int T,
                    int64_t N, int64_t nvec, typename Arith<S>::type alpha,
                    typename Arith<S>::type thresh) {
@@ -406,6 +424,8 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
         for (int k = 0; k < TC; ++k) {
             if (FULL || k < T)
                 cur[k] = load_pack<S, V, !KEEP>(x + static_cast<int64_t>(k) * N + col);
+            // requests go out in time order (left alone, the compiler issues the first row last but one)
+            if (FULL) __builtin_amdgcn_sched_barrier(0);
         }
         for (int t0 = 0; t0 < T; t0 += TC) {
             if (MULTI && t0 + TC < T) {
@@ -433,6 +453,9 @@ lif_forward_kernel(const S* __restrict__ x, M* __restrict__ mem, S* __restrict__
                     if (WRITE_U) store_pack<M, V>(mem + off, mo);
                     if (WRITE_S) store_pack<S, V>(spike + off, so);
                 }
+                // a row is consumed and its result stored as soon as it has arrived, not after the
+                // whole group has (left alone, the compiler gathers the stores behind the last wait)
+                if (FULL) __builtin_amdgcn_sched_barrier(0);
             }
             if (!MULTI) break;
             if (t0 + TC < T) {
@@ -709,8 +732,9 @@ __device__ __forceinline__ int64_t backward_column(int64_t v, int64_t nvec, int 
 // Fused backward for T <= TW: the whole time axis is one register window.  HEAD > 0: for
 // TW < T <= TW + HEAD, the first T - TW steps being the window's head (see backward_window).
 // ---------------------------------------------------------------------------------------------
-template <typename S, int V, int TW, bool EXACT, bool KEEP, bool GSHARED = false, int HEAD = 0>
-__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(TW + HEAD, KEEP))
+template <typename S, int V, int TW, bool EXACT, bool KEEP, bool GSHARED = false, int HEAD = 0, int CAP = 0>
+__global__ void __launch_bounds__(kBwdBlock)
+    SNNLIF_WAVES_PER_SIMD(CAP > 0 ? CAP : backward_waves(TW + HEAD, KEEP))
 lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* __restrict__ gx,
                           int T, int64_t N, int64_t GN, int64_t nvec,
                           typename Arith<S>::type alpha, typename Arith<S>::type thresh,
@@ -970,36 +994,41 @@ inline int with_vec(int v, F&& f) {
 
 // One forward launch with TC rows per group.
 template <typename S, typename M, int V, int TC, bool MULTI, bool WRITE_U, bool WRITE_S, bool KEEP,
-          bool CAPPED = false>
+          int CAP = 0>
 int launch_forward_rows(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
                         int threads, hipStream_t stream) {
     using C = typename Arith<S>::type;
     const int64_t nvec = N / V;
-    // A window that fills the instantiation can run without the tests around each row.  Measured
-    // cold: fp64 windows of 8 / 16 steps 62 -> 71 % / 51 -> 65.5 % of the HBM peak (behind the tests the
-    // compiler waits for each 8-byte load before it issues the next); fp32 +1 point for the capped
-    // 8-step window and for 4 steps, -0.5 to -1.5 for 16 steps and for tensors beyond 256 MiB; bf16 -0.5.
-    constexpr bool can_fill = !MULTI && (sizeof(S) == 8 || (sizeof(S) == 4 && (CAPPED || TC == 4)));
+    // A window that fills the instantiation can run without the tests around each row.  fp64 windows
+    // of 8 / 16 steps: 62 -> 71 % / 51 -> 65.5 % of the HBM peak, cold (behind the tests the compiler waits
+    // for each 8-byte load before it issues the next); the streamed fp32 / bf16 windows of up to 8 steps
+    // have an instantiation per length (CAP > 0), and 4 steps gain a point in the kept form as well.
+    constexpr bool can_fill = !MULTI && (sizeof(S) == 8 || CAP > 0 || (sizeof(S) == 4 && TC == 4));
     if constexpr (can_fill) {
         if (T == TC) {
-            launch_kernel(lif_forward_kernel<S, M, V, TC, false, WRITE_U, WRITE_S, KEEP, CAPPED, true>,
+            launch_kernel(lif_forward_kernel<S, M, V, TC, false, WRITE_U, WRITE_S, KEEP, CAP, true>,
                           dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
                           static_cast<int>(T), N, nvec, C(alpha), C(thresh));
             return launch_status();
         }
     }
-    launch_kernel(lif_forward_kernel<S, M, V, TC, MULTI, WRITE_U, WRITE_S, KEEP, CAPPED>,
-                  dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
-                  static_cast<int>(T), N, nvec, C(alpha), C(thresh));
-    return launch_status();
+    if constexpr (CAP > 0) {
+        return SNNLIF_ERR_ARG;  // the capped instantiations exist for T == TC only
+    } else {
+        launch_kernel(lif_forward_kernel<S, M, V, TC, MULTI, WRITE_U, WRITE_S, KEEP, CAP>,
+                      dim3(grid_for(nvec, threads)), dim3(threads), 0, stream, x, mem, spike,
+                      static_cast<int>(T), N, nvec, C(alpha), C(thresh));
+        return launch_status();
+    }
 }
 
 // Rows per group by window length.  Kept x: the whole window up to SNNLIF_FWD_ROWS rows, longer ones
 // streamed in groups of that many.  Streamed x: windows of up to 16 rows are requested whole (a
-// window of 9-16 rows as one group measures +5-8 points over two groups of 8), and so are windows
-// of 24-32 rows, in a 32-row instantiation at 3 wavefronts per SIMD (+3-5 points over two groups of
-// 16; a 20-row window zero-filled to 32 loses 4-8, so 17-23 rows stay in groups).  Everything else
-// goes in groups of 16, i.e. the windows of 17-23 rows: from 32 rows on every window runs the
+// window of 9-16 rows as one group measures +5-8 points over two groups of 8), windows of 17-24 rows
+// whole in a 24-row instantiation and windows of 25-31 rows in a 32-row one, both at 3 wavefronts per
+// SIMD (against a group of 16 followed by the rest, cold, rows 8 MiB apart: 17 rows 48 -> 55 % of the HBM
+// peak, 20 rows 59 -> 64, 23 rows 63 -> 66; 24 rows in their own instantiation +2 over the 32-row one;
+// 32 rows at once +3-5 points over two groups of 16).  From 32 rows on every window runs the
 // rolling-window kernel.
 template <typename S, typename M, int V, bool WRITE_U, bool WRITE_S, bool KEEP>
 int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float alpha, float thresh,
@@ -1012,13 +1041,40 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
 #define SNNLIF_FWD_LAUNCH(ROWS, MULTI)                                                           \
     launch_forward_rows<S, M, V, ROWS, MULTI, WRITE_U, WRITE_S, KEEP>(x, mem, spike, T, N, alpha,  \
                                                                       thresh, threads, stream)
-    if (T <= 4 && TC > 4) return SNNLIF_FWD_LAUNCH(4, false);
-    if constexpr (!KEEP && TC == 8) {
-        if (T == TC && static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S) <=
-                           static_cast<size_t>(SNNLIF_STREAM_FWD_CAPPED_BYTES))
-            return launch_forward_rows<S, M, V, TC, false, WRITE_U, WRITE_S, KEEP, true>(
-                x, mem, spike, T, N, alpha, thresh, threads, stream);
+    if constexpr (!KEEP) {
+        // streamed windows of up to 8 steps: a straight-line instantiation per length and number of
+        // wavefronts per SIMD
+        const size_t tensor_bytes = static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S);
+        int waves = stream_forward_waves(static_cast<int>(T), tensor_bytes);
+#ifdef SNNLIF_LAB
+        if (const char* e = getenv("SNNLIF_LAB_FWD_WAVES")) waves = atoi(e);
+#endif
+#define SNNLIF_FWD_EXACT(ROWS, WAVES)                                                              \
+    if (T == ROWS && waves == WAVES)                                                               \
+        return launch_forward_rows<S, M, V, ROWS, false, WRITE_U, WRITE_S, KEEP, WAVES>(            \
+            x, mem, spike, T, N, alpha, thresh, threads, stream);
+#ifdef SNNLIF_LAB
+#define SNNLIF_FWD_EXACT_ALL(ROWS)                                                                 \
+    SNNLIF_FWD_EXACT(ROWS, 2) SNNLIF_FWD_EXACT(ROWS, 3) SNNLIF_FWD_EXACT(ROWS, 4)                   \
+    SNNLIF_FWD_EXACT(ROWS, 5) SNNLIF_FWD_EXACT(ROWS, 6) SNNLIF_FWD_EXACT(ROWS, 7) SNNLIF_FWD_EXACT(ROWS, 8)
+        SNNLIF_FWD_EXACT_ALL(3) SNNLIF_FWD_EXACT_ALL(4) SNNLIF_FWD_EXACT_ALL(5) SNNLIF_FWD_EXACT_ALL(6)
+        SNNLIF_FWD_EXACT_ALL(7) SNNLIF_FWD_EXACT_ALL(8)
+#undef SNNLIF_FWD_EXACT_ALL
+#endif
+        SNNLIF_FWD_EXACT(1, 8)
+        SNNLIF_FWD_EXACT(2, 8)
+        SNNLIF_FWD_EXACT(3, 8)
+        SNNLIF_FWD_EXACT(4, 8)
+        SNNLIF_FWD_EXACT(5, 5)
+        SNNLIF_FWD_EXACT(6, 5)
+        SNNLIF_FWD_EXACT(6, 4)
+        SNNLIF_FWD_EXACT(7, 5)
+        SNNLIF_FWD_EXACT(7, 3)
+        SNNLIF_FWD_EXACT(8, 5)
+        SNNLIF_FWD_EXACT(8, 3)
+#undef SNNLIF_FWD_EXACT
     }
+    if (T <= 4 && TC > 4) return SNNLIF_FWD_LAUNCH(4, false);
     if (T <= TC) return SNNLIF_FWD_LAUNCH(TC, false);
     if constexpr (!KEEP && SNNLIF_FWD_ROLLING_W > 0) {
         constexpr int W = SNNLIF_FWD_ROLLING_W > 0 ? SNNLIF_FWD_ROLLING_W : 1;
@@ -1039,9 +1095,10 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
     }
     if constexpr (!KEEP) {
         if (T <= TM) return SNNLIF_FWD_LAUNCH(TM, false);
-        if (T <= TL && T >= TL - TL / 4) return SNNLIF_FWD_LAUNCH(TL, false);
+        if (T <= (TM + TL) / 2) return SNNLIF_FWD_LAUNCH((TM + TL) / 2, false);
+        if (T <= TL) return SNNLIF_FWD_LAUNCH(TL, false);
     }
-    return SNNLIF_FWD_LAUNCH(TM, true);
+    return SNNLIF_FWD_LAUNCH(TM, true);  // kept x only: streamed windows of this length have returned above
 #undef SNNLIF_FWD_LAUNCH
 }
 
@@ -1149,6 +1206,16 @@ int launch_backward_fused_policy(const S* x, const S* g, S* gx, int64_t T, int64
                               stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta),
                               C(interval));
         } else {
+            if constexpr (!KEEP && stream_backward_small_waves(TW) > 0) {
+                if (static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S) <=
+                    static_cast<size_t>(SNNLIF_STREAM_SMALL_BYTES)) {
+                    launch_kernel(lif_backward_fused_kernel<S, V, TW, true, KEEP, false, 0,
+                                                            stream_backward_small_waves(TW)>,
+                                  grid, block, 0, stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh),
+                                  C(beta), C(interval));
+                    return launch_status();
+                }
+            }
             launch_kernel(lif_backward_fused_kernel<S, V, TW, true, KEEP>, grid, block, 0, stream,
                                x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
         }
@@ -1185,12 +1252,19 @@ int launch_backward_headed(const S* x, const S* g, S* gx, int64_t T, int64_t N, 
         const int threads = backward_block(bytes, 64, keep);
         const dim3 grid(grid_for(nvec, threads)), block(threads);
         const int Ti = static_cast<int>(T);
-        if (keep)
+        constexpr int small_waves = stream_backward_small_waves(TB + kHeadMax);
+        if (keep) {
             launch_kernel(lif_backward_fused_kernel<S, V, TB, true, true, false, kHeadMax>, grid, block,
                           0, stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
-        else
+        } else if (small_waves > 0 && bytes <= static_cast<size_t>(SNNLIF_STREAM_SMALL_BYTES)) {
+            if constexpr (small_waves > 0)
+                launch_kernel(lif_backward_fused_kernel<S, V, TB, true, false, false, kHeadMax, small_waves>,
+                              grid, block, 0, stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh),
+                              C(beta), C(interval));
+        } else {
             launch_kernel(lif_backward_fused_kernel<S, V, TB, true, false, false, kHeadMax>, grid, block,
                           0, stream, x, g, gx, Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
+        }
         return launch_status();
     });
 }
