@@ -76,7 +76,8 @@ extern "C" {
 #define SNNLIF_ERR_UNSUPPORTED -5 /* valid arguments this entry point does not implement (bf16 in the batch-norm ones) */
 
 /* Every T up to this keeps the whole recomputed membrane potential in registers in the backward
- * (one kernel, 12 bytes per neuron-step in fp32); so do multiples of 8 steps up to 104 (64 in fp64). */
+ * (one kernel, 12 bytes per neuron-step in fp32) whatever the storage type; so do longer windows up to
+ * 111 steps in fp32 (71 in fp64; bf16: up to 63, and multiples of 8 up to 104). */
 #define SNNLIF_BP_FUSED_MAX_T 32
 /* Largest T for which snnlif_fire_bp needs no workspace: up to here longer windows are processed
  * in register-sized segments whose boundary potentials live in LDS (16 bytes per neuron-step). */
