@@ -136,6 +136,15 @@
 #ifndef SNNLIF_STREAM_BWD_WAVES_LONG
 #define SNNLIF_STREAM_BWD_WAVES_LONG 4
 #endif
+#ifndef SNNLIF_STREAM_BWD_WAVES_LONGER  // windows of 13 to 24 rows / 25 to 64 / beyond
+#define SNNLIF_STREAM_BWD_WAVES_LONGER 3
+#endif
+#ifndef SNNLIF_STREAM_BWD_WAVES_LONGEST
+#define SNNLIF_STREAM_BWD_WAVES_LONGEST 2
+#endif
+#ifndef SNNLIF_STREAM_BWD_WAVES_WIDE
+#define SNNLIF_STREAM_BWD_WAVES_WIDE 2
+#endif
 #ifndef SNNLIF_STREAM_BWD_WAVES_3  // windows of exactly 3 / 4 rows
 #define SNNLIF_STREAM_BWD_WAVES_3 8
 #endif
@@ -185,17 +194,24 @@ namespace snnlif {
 // Streamed x (everything from HBM): fewer wavefronts already pay for windows of 5 to 8 rows (8 rows:
 // 84 % of peak at 5 wavefronts against 78 % at 8), while windows of 3 and 4 rows need 8 and 7 to keep
 // enough requests going (cold, 256 MiB tensors: 3 rows 71 -> 83 %, 4 rows 76 -> 84 % against 5
-// wavefronts; 5 rows and more lose 1-6 points beyond 5).  SNNLIF_BWD_MAX_WAVES overrides both.
+// wavefronts; 5 rows and more lose 1-6 points beyond 5); windows of 9-12 rows run 4, 13-24 rows 3 (16
+// rows 80.0 -> 81.4 %, 20 rows 77.6 -> 78.8, 24 rows 77.8 -> 79.2 against 4), 25-64 rows 2 (32 rows
+// 76.3 -> 77.5, 40 rows 75.4 -> 77.2, 64 rows 68.5 -> 70.7), and so do the windows beyond 64 rows (72
+// rows 67.7 -> 69.1, 80 rows 72.8 -> 74.5, 96 rows 70.4 -> 73.4 against 3).  SNNLIF_BWD_MAX_WAVES
+// overrides both.
 constexpr int backward_waves(int rows, bool keep = true) {
 #ifdef SNNLIF_BWD_MAX_WAVES
     return SNNLIF_BWD_MAX_WAVES;
 #else
-    if (rows > 64) return 3;  // u alone takes `rows` VGPRs per lane
     if (!keep) {
         if (rows == 3) return SNNLIF_STREAM_BWD_WAVES_3;
         if (rows == 4) return SNNLIF_STREAM_BWD_WAVES_4;
-        return rows <= 8 ? SNNLIF_STREAM_BWD_WAVES_SHORT : SNNLIF_STREAM_BWD_WAVES_LONG;
+        if (rows <= 8) return SNNLIF_STREAM_BWD_WAVES_SHORT;
+        if (rows <= 12) return SNNLIF_STREAM_BWD_WAVES_LONG;
+        if (rows <= 24) return SNNLIF_STREAM_BWD_WAVES_LONGER;
+        return rows > 64 ? SNNLIF_STREAM_BWD_WAVES_WIDE : SNNLIF_STREAM_BWD_WAVES_LONGEST;
     }
+    if (rows > 64) return 3;  // u alone takes `rows` VGPRs per lane
     return rows <= 8 ? 8 : (rows <= 12 ? 5 : 4);
 #endif
 }
@@ -333,7 +349,11 @@ __device__ __forceinline__ Pack<S, V> load_pack(const S* p) {
 template <typename S, int V>
 __device__ __forceinline__ void store_pack(S* p, const Pack<S, V>& v) {
     using raw_t = typename Pack<S, V>::raw_t;
+#ifdef SNNLIF_STORE_PLAIN
+    *reinterpret_cast<raw_t*>(p) = v.raw;
+#else
     __builtin_nontemporal_store(v.raw, reinterpret_cast<raw_t*>(p));
+#endif
 }
 
 // Storage type -> arithmetic type and conversions.
