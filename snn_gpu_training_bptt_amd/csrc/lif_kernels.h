@@ -67,9 +67,6 @@
 
 #include <cstddef>
 #include <cstdint>
-#ifdef SNNLIF_LAB
-#include <cstdlib>
-#endif
 #include <tuple>
 #include <type_traits>
 
@@ -1065,22 +1062,11 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
         // streamed windows of up to 8 steps: a straight-line instantiation per length and number of
         // wavefronts per SIMD
         const size_t tensor_bytes = static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S);
-        int waves = stream_forward_waves(static_cast<int>(T), tensor_bytes);
-#ifdef SNNLIF_LAB
-        if (const char* e = getenv("SNNLIF_LAB_FWD_WAVES")) waves = atoi(e);
-#endif
+        const int waves = stream_forward_waves(static_cast<int>(T), tensor_bytes);
 #define SNNLIF_FWD_EXACT(ROWS, WAVES)                                                              \
     if (T == ROWS && waves == WAVES)                                                               \
         return launch_forward_rows<S, M, V, ROWS, false, WRITE_U, WRITE_S, KEEP, WAVES>(            \
             x, mem, spike, T, N, alpha, thresh, threads, stream);
-#ifdef SNNLIF_LAB
-#define SNNLIF_FWD_EXACT_ALL(ROWS)                                                                 \
-    SNNLIF_FWD_EXACT(ROWS, 2) SNNLIF_FWD_EXACT(ROWS, 3) SNNLIF_FWD_EXACT(ROWS, 4)                   \
-    SNNLIF_FWD_EXACT(ROWS, 5) SNNLIF_FWD_EXACT(ROWS, 6) SNNLIF_FWD_EXACT(ROWS, 7) SNNLIF_FWD_EXACT(ROWS, 8)
-        SNNLIF_FWD_EXACT_ALL(3) SNNLIF_FWD_EXACT_ALL(4) SNNLIF_FWD_EXACT_ALL(5) SNNLIF_FWD_EXACT_ALL(6)
-        SNNLIF_FWD_EXACT_ALL(7) SNNLIF_FWD_EXACT_ALL(8)
-#undef SNNLIF_FWD_EXACT_ALL
-#endif
         SNNLIF_FWD_EXACT(1, 8)
         SNNLIF_FWD_EXACT(2, 8)
         SNNLIF_FWD_EXACT(3, 8)

@@ -183,9 +183,35 @@ std::vector<Tensor> linear_backward_folded(const Tensor& in, const Tensor& grad_
     return {grad_in, grad_weight, at::sum(grad_fc, dim_fc)};
 }
 
+// The reference hands `benchmark` and `deterministic` to cuDNN with every convolution call
+// (snnlib/cuda/snn_kernel_fp.cu:404-407, snnlib/cuda/snn_kernel_bp.cu:1107-1118).  PyTorch-ROCm takes
+// them from the process-wide settings (torch.backends.cudnn.benchmark / .deterministic) when it calls
+// MIOpen -- benchmark = true lets MIOpen search for the fastest algorithm of a shape the first time it
+// sees it, false takes its immediate choice -- so the caller's flags are put there for the duration
+// of the dense call and the previous settings restored afterwards.
+class ConvSearchGuard {
+public:
+    ConvSearchGuard(bool benchmark, bool deterministic)
+        : benchmark_(at::globalContext().benchmarkCuDNN()),
+          deterministic_(at::globalContext().deterministicCuDNN()) {
+        at::globalContext().setBenchmarkCuDNN(benchmark);
+        at::globalContext().setDeterministicCuDNN(deterministic);
+    }
+    ~ConvSearchGuard() {
+        at::globalContext().setBenchmarkCuDNN(benchmark_);
+        at::globalContext().setDeterministicCuDNN(deterministic_);
+    }
+    ConvSearchGuard(const ConvSearchGuard&) = delete;
+    ConvSearchGuard& operator=(const ConvSearchGuard&) = delete;
+
+private:
+    bool benchmark_, deterministic_;
+};
+
 Tensor conv_folded(const Tensor& in, const Tensor& weight, const Tensor& bias,
                    const IntList& stride, const IntList& padding, const IntList& dilation,
-                   int64_t groups) {
+                   int64_t groups, bool benchmark, bool deterministic) {
+    const ConvSearchGuard search(benchmark, deterministic);
     Tensor conv = at::convolution(fold_time(in), weight, bias, stride, padding, dilation,
                                   /*transposed=*/false, /*output_padding=*/{0, 0}, groups);
     return reshaped_result(conv, {in.size(0), in.size(1), conv.size(1), conv.size(2), conv.size(3)});
@@ -195,7 +221,9 @@ Tensor conv_folded(const Tensor& in, const Tensor& weight, const Tensor& bias,
 std::vector<Tensor> conv_backward_folded(const Tensor& in, const Tensor& grad_conv,
                                          const Tensor& weight, const IntList& stride,
                                          const IntList& padding, const IntList& dilation,
-                                         int64_t groups, const IntList& dim_conv, const char* op) {
+                                         int64_t groups, bool benchmark, bool deterministic,
+                                         const IntList& dim_conv, const char* op) {
+    const ConvSearchGuard search(benchmark, deterministic);
     TORCH_CHECK(grad_conv.dim() == 5 && grad_conv.size(0) == in.size(0) &&
                     grad_conv.size(1) == in.size(1) && grad_conv.size(2) == weight.size(0),
                 "snnlib.", op, ": grad_conv must be [T, B, cout, Hout, Wout], got ",
@@ -604,29 +632,30 @@ std::vector<Tensor> fc_bp(Tensor spatial, Tensor grad_fc, Tensor weight_fc, Tens
     return linear_backward_folded(spatial, grad_fc, weight_fc, dim_fc, "fc_bp");
 }
 
-// `benchmark` / `deterministic` / `allow_tf32` select cuDNN behaviour in the reference; on ROCm the
-// convolution algorithm is MIOpen's choice under torch.backends.cudnn.{benchmark,deterministic}.
+// `benchmark` / `deterministic` reach MIOpen through ConvSearchGuard; `allow_tf32` has no meaning on
+// this hardware and is ignored.
 Tensor conv_fp(Tensor spatial, Tensor weight_conv, Tensor bias_conv, IntList stride,
-               IntList padding, IntList dilation, int64_t groups, bool /*benchmark*/,
-               bool /*deterministic*/) {
+               IntList padding, IntList dilation, int64_t groups, bool benchmark,
+               bool deterministic) {
     check_input(spatial, "conv_fp", "spatial");
     check_image(spatial, "conv_fp");
     check_like(weight_conv, spatial, "conv_fp", "weight_conv");
     check_like(bias_conv, spatial, "conv_fp", "bias_conv");
     const DeviceGuard guard(spatial.device());
-    return conv_folded(spatial, weight_conv, bias_conv, stride, padding, dilation, groups);
+    return conv_folded(spatial, weight_conv, bias_conv, stride, padding, dilation, groups, benchmark,
+                       deterministic);
 }
 
 std::vector<Tensor> conv_bp(Tensor spatial, Tensor grad_conv, Tensor weight_conv, IntList stride,
-                            IntList padding, IntList dilation, int64_t groups, bool /*benchmark*/,
-                            bool /*deterministic*/, bool /*allow_tf32*/, IntList dim_conv) {
+                            IntList padding, IntList dilation, int64_t groups, bool benchmark,
+                            bool deterministic, bool /*allow_tf32*/, IntList dim_conv) {
     check_input(spatial, "conv_bp", "spatial");
     check_image(spatial, "conv_bp");
     check_like(weight_conv, spatial, "conv_bp", "weight_conv");
     check_like(grad_conv, spatial, "conv_bp", "grad_conv");
     const DeviceGuard guard(spatial.device());
     return conv_backward_folded(spatial, grad_conv, weight_conv, stride, padding, dilation, groups,
-                                dim_conv, "conv_bp");
+                                benchmark, deterministic, dim_conv, "conv_bp");
 }
 
 // ---- fire, then a fully connected layer / a convolution -------------------------------------------
@@ -656,20 +685,21 @@ std::vector<Tensor> fire_fc_bp(Tensor spatial, Tensor grad_fc, Tensor weight_fc,
 }
 
 Tensor fire_conv_fp(Tensor spatial, Tensor weight_conv, Tensor bias_conv, IntList stride,
-                    IntList padding, IntList dilation, int64_t groups, bool /*benchmark*/,
-                    bool /*deterministic*/, float alpha, float thresh) {
+                    IntList padding, IntList dilation, int64_t groups, bool benchmark,
+                    bool deterministic, float alpha, float thresh) {
     check_input(spatial, "fire_conv_fp", "spatial");
     check_image(spatial, "fire_conv_fp");
     check_like(weight_conv, spatial, "fire_conv_fp", "weight_conv");
     check_like(bias_conv, spatial, "fire_conv_fp", "bias_conv");
     Tensor spike = fire_s_fp(spatial, alpha, thresh);
     const DeviceGuard guard(spatial.device());
-    return conv_folded(spike, weight_conv, bias_conv, stride, padding, dilation, groups);
+    return conv_folded(spike, weight_conv, bias_conv, stride, padding, dilation, groups, benchmark,
+                       deterministic);
 }
 
 std::vector<Tensor> fire_conv_bp(Tensor spatial, Tensor grad_conv, Tensor weight_conv,
                                  IntList stride, IntList padding, IntList dilation, int64_t groups,
-                                 bool /*benchmark*/, bool /*deterministic*/, bool /*allow_tf32*/,
+                                 bool benchmark, bool deterministic, bool /*allow_tf32*/,
                                  IntList dim_conv, float alpha, float thresh, float beta,
                                  float interval) {
     check_input(spatial, "fire_conv_bp", "spatial");
@@ -679,7 +709,7 @@ std::vector<Tensor> fire_conv_bp(Tensor spatial, Tensor grad_conv, Tensor weight
     Tensor spike = fire_s_fp(spatial, alpha, thresh);
     const DeviceGuard guard(spatial.device());
     auto dense = conv_backward_folded(spike, grad_conv, weight_conv, stride, padding, dilation,
-                                      groups, dim_conv, "fire_conv_bp");
+                                      groups, benchmark, deterministic, dim_conv, "fire_conv_bp");
     return {fire_bp(spatial, dense[0], alpha, thresh, beta, interval), dense[1], dense[2]};
 }
 
@@ -718,8 +748,8 @@ std::vector<Tensor> bn_fire_fc_bp(Tensor spatial, Tensor weight_bn, Tensor bias_
 std::vector<Tensor> bn_fire_conv_fp(Tensor spatial, Tensor weight_bn, Tensor bias_bn, Tensor var,
                                     Tensor mean, float eps_bn, Tensor weight_conv,
                                     Tensor bias_conv, IntList stride, IntList padding,
-                                    IntList dilation, int64_t groups, bool /*benchmark*/,
-                                    bool /*deterministic*/, float alpha, float thresh) {
+                                    IntList dilation, int64_t groups, bool benchmark,
+                                    bool deterministic, float alpha, float thresh) {
     check_input(spatial, "bn_fire_conv_fp", "spatial");
     check_image(spatial, "bn_fire_conv_fp");
     check_like(weight_conv, spatial, "bn_fire_conv_fp", "weight_conv");
@@ -727,14 +757,15 @@ std::vector<Tensor> bn_fire_conv_fp(Tensor spatial, Tensor weight_bn, Tensor bia
     auto fired = bn_fire_s_fp(spatial, weight_bn, bias_bn, var, mean, eps_bn, alpha, thresh);
     const DeviceGuard guard(spatial.device());
     return {fired[0],
-            conv_folded(fired[1], weight_conv, bias_conv, stride, padding, dilation, groups)};
+            conv_folded(fired[1], weight_conv, bias_conv, stride, padding, dilation, groups, benchmark,
+                        deterministic)};
 }
 
 std::vector<Tensor> bn_fire_conv_bp(Tensor spatial, Tensor weight_bn, Tensor bias_bn, Tensor ivar,
                                     Tensor mean, IntList dim_bn, Tensor grad_conv,
                                     Tensor weight_conv, IntList stride, IntList padding,
-                                    IntList dilation, int64_t groups, bool /*benchmark*/,
-                                    bool /*deterministic*/, bool /*allow_tf32*/, IntList dim_conv,
+                                    IntList dilation, int64_t groups, bool benchmark,
+                                    bool deterministic, bool /*allow_tf32*/, IntList dim_conv,
                                     float alpha, float thresh, float beta, float interval) {
     check_input(spatial, "bn_fire_conv_bp", "spatial");
     check_image(spatial, "bn_fire_conv_bp");
@@ -744,7 +775,7 @@ std::vector<Tensor> bn_fire_conv_bp(Tensor spatial, Tensor weight_bn, Tensor bia
                                             "bn_fire_conv_bp");
     const DeviceGuard guard(spatial.device());
     auto dense = conv_backward_folded(spike, grad_conv, weight_conv, stride, padding, dilation,
-                                      groups, dim_conv, "bn_fire_conv_bp");
+                                      groups, benchmark, deterministic, dim_conv, "bn_fire_conv_bp");
     auto bn = bn_fire_bp(spatial, weight_bn, bias_bn, ivar, mean, dim_bn, dense[0], alpha, thresh,
                          beta, interval);
     return {bn[0], bn[1], bn[2], dense[1], dense[2]};
@@ -774,8 +805,8 @@ std::vector<Tensor> bn_fire_fc_bp_dist1(Tensor spatial, Tensor weight_bn, Tensor
 std::vector<Tensor> bn_fire_conv_bp_dist1(Tensor spatial, Tensor weight_bn, Tensor bias_bn,
                                           Tensor ivar, Tensor mean, IntList dim_bn, Tensor grad_conv,
                                           Tensor weight_conv, IntList stride, IntList padding,
-                                          IntList dilation, int64_t groups, bool /*benchmark*/,
-                                          bool /*deterministic*/, bool /*allow_tf32*/,
+                                          IntList dilation, int64_t groups, bool benchmark,
+                                          bool deterministic, bool /*allow_tf32*/,
                                           IntList dim_conv, float alpha, float thresh, float beta,
                                           float interval) {
     const char* op = "bn_fire_conv_bp_dist1";
@@ -786,7 +817,7 @@ std::vector<Tensor> bn_fire_conv_bp_dist1(Tensor spatial, Tensor weight_bn, Tens
     Tensor spike = bn_fire_spikes_from_ivar(spatial, weight_bn, bias_bn, ivar, mean, alpha, thresh, op);
     const DeviceGuard guard(spatial.device());
     auto dense = conv_backward_folded(spike, grad_conv, weight_conv, stride, padding, dilation,
-                                      groups, dim_conv, op);
+                                      groups, benchmark, deterministic, dim_conv, op);
     auto bn = bn_fire_bp_dist1(spatial, weight_bn, bias_bn, ivar, mean, dim_bn, dense[0], alpha,
                                thresh, beta, interval);
     return {dense[0], bn[0], bn[1], bn[2], bn[3], dense[1], dense[2]};

@@ -27,7 +27,10 @@ interval = 0.5
 thresh = 0.25
 time_step = 6
 
-conv_benchmark = False  # accepted for interface parity; MIOpen's search follows torch.backends.cudnn
+# True: MIOpen searches for the fastest algorithm of each convolution shape the first time it sees it
+# (slower first step, often a faster steady state); handed to the native convolution ops with every
+# call, as the reference does (snnlib_func.py:17), and applied there for the duration of the call.
+conv_benchmark = False
 
 _DIM_FC = (0, 1)            # axes a fully connected bias gradient sums over
 _DIM_CONV = (0, 1, 3, 4)    # axes a convolution bias gradient / conv-shaped batch norm sums over

@@ -102,3 +102,35 @@ def test_layer_surfaces(mods):
     assert conv.weight_conv.shape == (6, 4, 3, 3)
     assert (conv.stride, conv.padding, conv.if_bias_conv, conv.cin) == ((1, 1), (1, 1), True, 4)
     assert sf.fire_fc_func == sf.FireFcFunc.apply and sf.fire_conv_func == sf.FireConvFunc.apply
+
+
+@pytest.mark.parametrize("benchmark,deterministic", [(True, False), (False, True), (True, True)])
+def test_convolution_flags_reach_the_library_for_the_call_only(mods, benchmark, deterministic):
+    """The reference forwards `benchmark` / `deterministic` to the convolution with every call
+    (snn_kernel_fp.cu:404-407).  Here they become the process-wide settings PyTorch-ROCm hands to MIOpen
+    while the dense call runs and the previous settings come back afterwards, whichever way they were
+    set; the results agree with the default call to the dense library's accuracy."""
+    from snn_gpu_training_bptt_amd._loader import load_snnlib
+    snnlib = load_snnlib()
+    torch.manual_seed(5)
+    x = (0.5 + torch.randn(4, 2, 8, 8, 8)).cuda()
+    w = torch.randn(6, 8, 3, 3).cuda() * 0.2
+    b = torch.randn(6).cuda()
+    g = torch.randn(4, 2, 6, 8, 8).cuda()
+    saved = (torch.backends.cudnn.benchmark, torch.backends.cudnn.deterministic)
+    try:
+        for before in ((False, False), (True, True)):
+            torch.backends.cudnn.benchmark, torch.backends.cudnn.deterministic = before
+            ref = snnlib.fire_conv_fp(x, w, b, (1, 1), (1, 1), (1, 1), 1, False, False, ALPHA, THRESH)
+            out = snnlib.fire_conv_fp(x, w, b, (1, 1), (1, 1), (1, 1), 1, benchmark, deterministic, ALPHA, THRESH)
+            assert (torch.backends.cudnn.benchmark, torch.backends.cudnn.deterministic) == before
+            close(out, ref, "fire_conv_fp under the flags")
+            gref = snnlib.fire_conv_bp(x, g, w, (1, 1), (1, 1), (1, 1), 1, False, False, True, (0, 1, 3, 4),
+                                       ALPHA, THRESH, BETA, INTERVAL)
+            gout = snnlib.fire_conv_bp(x, g, w, (1, 1), (1, 1), (1, 1), 1, benchmark, deterministic, True,
+                                       (0, 1, 3, 4), ALPHA, THRESH, BETA, INTERVAL)
+            assert (torch.backends.cudnn.benchmark, torch.backends.cudnn.deterministic) == before
+            for a, r, what in zip(gout, gref, ("grad_spatial", "grad_weight", "grad_bias")):
+                close(a, r, what)
+    finally:
+        torch.backends.cudnn.benchmark, torch.backends.cudnn.deterministic = saved
