@@ -237,14 +237,25 @@ constexpr int forward_waves(int rows, bool keep, int cap = 0) {
 #endif
 }
 
-// Wavefronts per SIMD of the streamed forward of a window of up to 8 steps (one of the instantiations
-// launch_forward_v lists).  Measured cold over 2-8 wavefronts, fp32, % of the HBM peak at the best / at
+// Wavefronts per SIMD of the straight-line instantiation of the streamed forward for a window of `rows`
+// steps (one of those launch_forward_v lists).  Measured cold over 2-8 wavefronts, fp32, % of the HBM peak at the best / at
 // 8 wavefronts: 8 steps 78 / 76 (256 MiB tensors, best at 5), 80 / 79 (512 MiB, 5), 69 / 62 (128 MiB, 3);
 // 7 steps 77 / 76.5 (224 MiB, 5), 69 / 63.5 (112 MiB, 3); 6 steps 76 / 75 (192 MiB, 5), 68 / 64 (96 MiB,
 // 4); 5 steps 75 / 72.5 (160 MiB, 5-7), 68 / 67 (80 MiB, 5); 4 and 3 steps are best at 7-8 at every size
 // (3 steps: 72 % at 8, 63 % at 5); bf16 8 steps on 256 MiB tensors 81 / 76.5 (5).
+// Longer windows: 10 steps 71 -> 78 % at 4 wavefronts against the 16-row instantiation with a test
+// around each row; 12 steps at 3: 74 -> 77 % (256 MiB), 69.6 -> 71 (128 MiB); 16 steps gain only on
+// tensors of at most 128 MiB, at 2 wavefronts (67 -> 72.7 %; 64 MiB 63 -> 66.5), and lose 2-6 points on
+// larger ones; 20 / 24 / 28 steps at 2: 72 -> 77 % / 74 -> 79 / 73 -> 76 (256 MiB tensors) against the
+// 24- and 32-row instantiations with tests, 32 steps 72.5 -> 73.8 against the rolling window.
+// 0: no straight-line instantiation for this length and size.
 inline int stream_forward_waves(int rows, size_t tensor_bytes) {
     const bool small = tensor_bytes <= static_cast<size_t>(SNNLIF_STREAM_SMALL_BYTES);
+    if (rows == 20 || rows == 24 || rows == 28 || rows == 32) return 2;
+    if (rows == 16) return small ? 2 : 0;
+    if (rows == 12) return 3;
+    if (rows == 10) return 4;
+    if (rows > 8) return 0;
     if (rows >= 7) return small ? 3 : 5;
     if (rows == 6) return small ? 4 : 5;
     if (rows == 5) return 5;
@@ -1059,8 +1070,8 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
     launch_forward_rows<S, M, V, ROWS, MULTI, WRITE_U, WRITE_S, KEEP>(x, mem, spike, T, N, alpha,  \
                                                                       thresh, threads, stream)
     if constexpr (!KEEP) {
-        // streamed windows of up to 8 steps: a straight-line instantiation per length and number of
-        // wavefronts per SIMD
+        // streamed windows of up to 8 steps and of 10, 12, 16 (small tensors), 20, 24, 28, 32: a
+        // straight-line instantiation per length and number of wavefronts per SIMD
         const size_t tensor_bytes = static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S);
         const int waves = stream_forward_waves(static_cast<int>(T), tensor_bytes);
 #define SNNLIF_FWD_EXACT(ROWS, WAVES)                                                              \
@@ -1078,6 +1089,13 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
         SNNLIF_FWD_EXACT(7, 3)
         SNNLIF_FWD_EXACT(8, 5)
         SNNLIF_FWD_EXACT(8, 3)
+        SNNLIF_FWD_EXACT(10, 4)
+        SNNLIF_FWD_EXACT(12, 3)
+        SNNLIF_FWD_EXACT(16, 2)
+        SNNLIF_FWD_EXACT(20, 2)
+        SNNLIF_FWD_EXACT(24, 2)
+        SNNLIF_FWD_EXACT(28, 2)
+        SNNLIF_FWD_EXACT(32, 2)
 #undef SNNLIF_FWD_EXACT
     }
     if (T <= 4 && TC > 4) return SNNLIF_FWD_LAUNCH(4, false);
