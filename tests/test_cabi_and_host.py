@@ -330,3 +330,15 @@ def test_static_scratch_backward_refuses_oversized_shapes_without_a_gpu():
     assert lib.snnlif_bn_fire_bp_static(*[None] * 9, f32, 4, 2, 8, 1, *tail) == lif_cabi.ERR_ARG
     assert lib.snnlif_bn_fire_bp_static(*[None] * 9, f32, 0, 2, 8, 1, *tail) == lif_cabi.OK
     assert "SNNLIF_STATIC_SCRATCH_BYTES" in lif_cabi.strerror(lif_cabi.ERR_SCRATCH)
+
+
+def test_no_kernel_is_scheduled_one_request_at_a_time():
+    """hipcc keeps the order "all requests of a window, then the arithmetic" for most instantiations of
+    the kernels but has fallen back to one request at a time, each followed by a full wait, for some
+    (a third of the bandwidth; results stay correct, so no parity test can see it).  The check
+    compiles every kernel to gfx950 assembly -- no GPU involved -- and counts loads that are directly
+    followed by `s_waitcnt vmcnt(0)`, and scratch memory."""
+    proc = subprocess.run([sys.executable, "-m", "snn_gpu_training_bptt_amd.schedule_check"],
+                          capture_output=True, text=True, cwd=REPO)
+    assert proc.returncode == 0, proc.stdout[-4000:] + proc.stderr[-2000:]
+    assert "0 with an unexpected schedule or scratch memory" in proc.stdout
