@@ -88,7 +88,8 @@ WORKLOADS = {
     # ... a 100-step one, which the backward runs as a 96-step body with a 4-step head (67 174 400
     # neuron-steps) ...
     "t100": ((100, 4, 164, 32, 32), 0.5, 1.0, "float32"),
-    # ... and a 120-step one, which it cuts into 32-step segments (67 338 240 neuron-steps)
+    # ... and a 120-step one, which it cuts into a 32-step segment and an 88-step tail window (67 338 240
+    # neuron-steps)
     "t120": ((120, 4, 137, 32, 32), 0.5, 1.0, "float32"),
 }
 # HBM bytes per launch of the backward kernel, measured with rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs

@@ -788,7 +788,7 @@ lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* _
 }
 
 // ---------------------------------------------------------------------------------------------
-// Segmented backward for windows longer than one register window (kSegment steps).  Two phases per
+// Segmented backward for windows longer than the register-window forms take.  Two phases per
 // lane, no scratch memory in HBM:
 //   1. run the recurrence forward over all but the last segment and keep the membrane potential at
 //      every segment boundary in LDS (one value per neuron and segment, in a slot only this lane
@@ -800,8 +800,13 @@ lif_backward_fused_kernel(const S* __restrict__ x, const S* __restrict__ g, S* _
 // ---------------------------------------------------------------------------------------------
 constexpr int kSegment = 32;
 
-template <typename S, int V>
-__global__ void __launch_bounds__(kBwdBlock) SNNLIF_WAVES_PER_SIMD(backward_waves(kSegment))
+// TAIL > 0: the end of the window is not a (partial) 32-step segment but one register window of
+// 64 + T mod 32 steps -- a straight-line body of TAIL steps (the multiple of 8 below that) with a head --
+// so that two to three segments fewer are read twice: 12 + 4 * (T - 64 - T mod 32) / T bytes per
+// neuron-step instead of 12 + 4 * (T - T mod 32) / T (120 steps: 13.1 instead of 15.1).
+template <typename S, int V, int TAIL = 0>
+__global__ void __launch_bounds__(kBwdBlock)
+    SNNLIF_WAVES_PER_SIMD(backward_waves(TAIL > 0 ? TAIL + kHeadMax : kSegment))
 lif_backward_segmented_kernel(const S* __restrict__ x, const S* __restrict__ g,
                               S* __restrict__ gx, int T, int64_t N, int64_t GN, int64_t nvec,
                               typename Arith<S>::type alpha, typename Arith<S>::type thresh,
@@ -809,7 +814,9 @@ lif_backward_segmented_kernel(const S* __restrict__ x, const S* __restrict__ g,
     using C = typename Arith<S>::type;
     extern __shared__ __align__(16) unsigned char lds_raw[];
     C* boundary = reinterpret_cast<C*>(lds_raw);  // [segment][lane][V]
-    const int nseg = (T + kSegment - 1) / kSegment;
+    // segments in all, the last one being the partial segment or the long tail window
+    const int tail = 2 * kSegment + T % kSegment;
+    const int nseg = TAIL > 0 ? (T - tail) / kSegment + 1 : (T + kSegment - 1) / kSegment;
     constexpr int ROWS = 8;  // rows requested at a time in phase 1
     static_assert(kSegment % ROWS == 0, "a segment is a whole number of phase-1 groups");
 
@@ -844,8 +851,16 @@ lif_backward_segmented_kernel(const S* __restrict__ x, const S* __restrict__ g,
                 boundary[(static_cast<int64_t>(seg + 1) * blockDim.x + threadIdx.x) * V + j] = uc[j];
         }
 
-        // phase 2: the last (possibly partial) segment first; uc / sc already hold its boundary
-        {
+        // phase 2: the last (possibly partial) segment or the tail window first; uc / sc already hold
+        // its boundary
+        if constexpr (TAIL > 0) {
+            const int head = tail - TAIL;
+            const int t0 = (nseg - 1) * kSegment + head;  // first row of the tail's body
+            const int64_t off = static_cast<int64_t>(t0) * N;
+            backward_window<S, V, TAIL, true, true, false, kHeadMax>(
+                x + off, g + static_cast<int64_t>(t0) * GN, gx + off, TAIL, N, GN, col, uc, sc, gu, alpha,
+                thresh, beta, interval, head);
+        } else {
             const int t0 = (nseg - 1) * kSegment;
             const int64_t off = static_cast<int64_t>(t0) * N;
             backward_window<S, V, kSegment, false>(x + off, g + static_cast<int64_t>(t0) * GN, gx + off,
@@ -1416,9 +1431,25 @@ int backward_dispatch(const void* x_, const void* g_, void* gx_, int64_t T, int6
             const int threads =
                 backward_block(static_cast<size_t>(T) * static_cast<size_t>(N) * sizeof(S), 128);
             const size_t lds = static_cast<size_t>(nseg) * threads * V * sizeof(C);
-            launch_kernel(lif_backward_segmented_kernel<S, V>, dim3(grid_for(nvec, threads)),
-                               dim3(threads), lds, stream, x, g, gx, static_cast<int>(T), N, GN, nvec,
-                               C(alpha), C(thresh), C(beta), C(interval));
+            const dim3 grid(grid_for(nvec, threads)), block(threads);
+            const int Ti = static_cast<int>(T);
+            // fp32: the window ends in a long register window instead of a partial segment (see the
+            // kernel).  Cold, 64 Mi elements, % of the HBM peak of 12 bytes per neuron-step: 112 steps
+            // 53 -> 57, 120 steps 62 -> 68, 140 steps 61 -> 66, 250 steps 56 -> 63, 500 steps 54 -> 55.
+            // (bf16 and fp64 would not keep full lanes / enough wavefronts for it.)
+            if constexpr (std::is_same<S, float>::value) {
+                const int body = (2 * kSegment + static_cast<int>(T % kSegment)) / 8 * 8;
+#define SNNLIF_BWD_TAIL(TB)                                                                        \
+    if (body == TB) {                                                                              \
+        launch_kernel(lif_backward_segmented_kernel<S, V, TB>, grid, block, lds, stream, x, g, gx, \
+                      Ti, N, GN, nvec, C(alpha), C(thresh), C(beta), C(interval));                 \
+        return launch_status();                                                                    \
+    }
+                SNNLIF_BWD_TAIL(64) SNNLIF_BWD_TAIL(72) SNNLIF_BWD_TAIL(80) SNNLIF_BWD_TAIL(88)
+#undef SNNLIF_BWD_TAIL
+            }
+            launch_kernel(lif_backward_segmented_kernel<S, V>, grid, block, lds, stream, x, g, gx, Ti, N,
+                          GN, nvec, C(alpha), C(thresh), C(beta), C(interval));
             return launch_status();
         });
     }

@@ -216,11 +216,13 @@ def test_windows_with_a_head_other_storage_types(cabi, oracle, T, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
-@pytest.mark.parametrize("T", [33, 34, 39, 57, 63, 65, 66, 71, 95, 97, 105, 127, 129, 159, 160, 161, 191, 193, 250, 1023])
+@pytest.mark.parametrize("T", [33, 34, 39, 57, 63, 65, 66, 71, 95, 97, 105, 112, 115, 120, 127, 129, 138, 140, 159,
+                               160, 161, 191, 193, 200, 250, 1023])
 def test_segmented_windows(cabi, oracle, T, dtype):
-    """Windows cut into 32-step segments, the last one partial: one step into a new segment (33, 65, 97,
+    """Windows cut into 32-step segments, the last one partial (fp64, bf16) or a long register window of
+    64 + T mod 32 steps with a body of 64, 72, 80 or 88 steps (fp32): one step into a new segment (33, 65, 97,
     129, 161, 193), one short of a full one (63, 95, 127, 159, 191, 1023), whole segments only (160), many
-    segments (250, 1023).  A negative threshold makes a wrong spike flag at the start of the window
+    segments (250, 1023), every body length of the fp32 tail (129 / 138, 140 / 112, 115 / 120, 127).  A negative threshold makes a wrong spike flag at the start of the window
     visible.  Even and odd N."""
     for n_inner, thresh in ((128, THRESH), (77, -0.25)):
         x32, g32 = make_inputs((T, 2, n_inner), 0.1, 0.9, seed=7000 + T)
