@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the LIF fire forward+backward hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg5_bf16|cfg1|t96|t100]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg5_bf16|cfg1|t96|t100|t120]
                     [--no-cpu-baseline] [--no-extra-legs]
     python bench.py --workload train_step [--steps K] [--warmup W]     (context figure, see below)
     python bench.py --workload bn_fire    [--steps K] [--warmup W]     (next-row op, see below)
@@ -27,9 +27,10 @@ byte comes from HBM.
                  synchronisations).
 * ``roofline``   the streamed backward kernel (the dominant one): algorithmic bytes per launch
                  (12 B x neuron-steps in fp32: read x, read grad_spike, write grad_x) divided by its
-                 mean duration, measured inside the timed region with HIP events attached to the
-                 dispatches (kernel begin / kernel end) of about 25 steps spread evenly over it,
-                 against the 8 TB/s HBM peak.  ``fwd`` and ``fwd_bwd`` give the same figure for the
+                 mean time in the timed region, against the 8 TB/s HBM peak.  Every dispatch of the timed
+                 region carries a stop event on the launch stream; a kernel's time is the interval from
+                 the completion of the kernel before it to its own (no stream-time overhead, and the
+                 intervals add up to the wall clock: kernel duration plus a dispatch gap of about 1 us).  ``fwd`` and ``fwd_bwd`` give the same figure for the
                  forward kernel (8 B) and for the pair (20 B); ``module`` repeats the leg's wall-clock
                  figures and compares them with ``cabi_streamed``.
 * ``roofline.cabi_streamed`` the same rotation through the C ABI (ctypes, pre-allocated outputs,
@@ -197,47 +198,55 @@ def tensor_sets(tensor_bytes):
 
 
 def rotation_leg(torch, lif_cabi, sets, steps, warmup, forward, backward, bytes_fwd, bytes_bwd,
-                 neuron_steps, instrumented=25):
+                 neuron_steps, instrumented=None):
     """K steps over `sets` independent tensor sets in rounds: forward(j) for every set j of the round,
     then backward(j) for every set, so that between a set's forward and its backward lie the other
     sets' forwards and backwards, several times the capacity of the memory-side cache.  A round holds
-    `sets` steps (the last one what is left of K).  About `instrumented` steps spread evenly over the
-    timed region carry HIP events on their two dispatches (snnlif_time_next_kernel: kernel begin /
-    kernel end on the launch stream); the other steps are launched as any caller would."""
+    `sets` steps (the last one what is left of K).
+
+    Every dispatch of the timed region carries a stop event (snnlif_time_next_kernel with no start
+    event: the completion of the kernel on the launch stream); a kernel's time is the interval from the
+    completion of the kernel before it to its own.  A stop event alone adds nothing to the stream
+    (measured: the wall clock per step is the same with and without), the intervals add up to the wall
+    clock, and in a saturated stream they are the kernels' durations plus the dispatch gap of about a
+    microsecond -- what a kernel costs in a sequence of launches.  (A start event as well costs 4-5 us
+    of stream time per dispatch, and on a dispatch that follows an un-instrumented one that time falls
+    inside the bracket.)"""
     def run(n, events):
-        k = 0
+        k = i = 0
         while k < n:
             r = min(sets, n - k)
-            for j in range(r):
-                ev = events.get(k + j) if events else None
-                if ev is not None:
-                    lif_cabi.time_next_kernel(ev[0], ev[1])
-                forward(j)
-            for j in range(r):
-                ev = events.get(k + j) if events else None
-                if ev is not None:
-                    lif_cabi.time_next_kernel(ev[2], ev[3])
-                backward(j)
+            for fn in (forward, backward):
+                for j in range(r):
+                    if events is not None:
+                        lif_cabi.time_next_kernel(None, events[i][1])
+                        events[i][0] = fn is forward
+                        i += 1
+                    fn(j)
             k += r
         return time.perf_counter()
 
     run(max(warmup, sets), None)
-    stride = max(1, steps // instrumented)
-    events = {k: [torch.cuda.Event(enable_timing=True) for _ in range(4)] for k in range(0, steps, stride)}
-    for row in events.values():   # create them on the device side before handing out their handles
-        for e in row:
-            e.record()
+    events = [[None, torch.cuda.Event(enable_timing=True)] for _ in range(2 * steps)]
+    begin = torch.cuda.Event(enable_timing=True)
+    for e in events:   # create them on the device side before handing out their handles
+        e[1].record()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    begin.record()
     t_enqueued = run(steps, events)
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     wall = t1 - t0
-    fwd_ms = sum(e[0].elapsed_time(e[1]) for e in events.values()) / len(events)
-    bwd_ms = sum(e[2].elapsed_time(e[3]) for e in events.values()) / len(events)
+    # intervals between consecutive completions; the first one starts at a stream marker, not at a
+    # kernel's completion, and is left out
+    spans = [(events[i][0], events[i - 1][1].elapsed_time(events[i][1])) for i in range(1, len(events))]
+    fwd = [ms for is_fwd, ms in spans if is_fwd]
+    bwd = [ms for is_fwd, ms in spans if not is_fwd]
+    fwd_ms, bwd_ms = sum(fwd) / len(fwd), sum(bwd) / len(bwd)
     rate = lambda nbytes, ms: nbytes / (ms * 1e-3) / 1e9
     return {
-        "sets": sets, "steps": steps, "launches_timed": len(events),
+        "sets": sets, "steps": steps, "launches_timed": len(spans),
         "ms_per_step": wall / steps * 1e3,
         "host_enqueue_ms_per_step": (t_enqueued - t0) / steps * 1e3,
         "neuron_steps_per_s": neuron_steps * steps / wall,
@@ -621,13 +630,13 @@ def run_policy_sweep(args):
             torch, lif_cabi, sets, steps, sets,
             lambda j: lif_cabi.fire_s_fp_into(xs[j], spikes[j], ALPHA, THRESH, keep_spatial=False),
             lambda j: lif_cabi.fire_bp_into(xs[j], gs[j], gxs[j], ALPHA, THRESH, BETA, INTERVAL, keep_spatial=False),
-            8 * ns, 12 * ns, ns, instrumented=steps)
+            8 * ns, 12 * ns, ns)
         s_ref, gx_ref = spikes[0].clone(), gxs[0].clone()
         kept = rotation_leg(
             torch, lif_cabi, 1, 24, 4,
             lambda j: lif_cabi.fire_s_fp_into(x, spikes[0], ALPHA, THRESH, keep_spatial=True),
             lambda j: lif_cabi.fire_bp_into(x, g, gxs[0], ALPHA, THRESH, BETA, INTERVAL, keep_spatial=True),
-            8 * ns, 12 * ns, ns, instrumented=24)
+            8 * ns, 12 * ns, ns)
         same = bool(torch.equal(spikes[0], s_ref) and torch.equal(gxs[0], gx_ref))
         rows.append({"shape": list(shape), "what": what, "tensor_MiB": round(tensor_bytes / 2**20, 1),
                      "row_pitch_bytes": ns // T * 4, "no_hint": "kept" if tensor_bytes <= (32 << 20) else "streamed",
@@ -773,8 +782,8 @@ def main():
             "traffic_source": traffic.get("source"),
             "algorithmic_bytes_per_launch": bytes_bwd,
             "avg_launch_ms": head["bwd"]["avg_launch_ms"],
-            "timing": f"HIP events attached to the dispatches (kernel begin / kernel end) of {head['launches_timed']} "
-                      f"of the {args.steps} steps inside the timed region",
+            "timing": f"completion-to-completion intervals of stop events attached to every dispatch of the timed "
+                      f"region ({head['launches_timed']} intervals over {args.steps} steps; they add up to the wall clock)",
             "fwd": head["fwd"],
             "fwd_bwd": head["fwd_bwd"],
             "module": {"policy": "streamed", "ms_per_step": head["ms_per_step"],

@@ -1093,9 +1093,7 @@ int launch_forward_v(const S* x, M* mem, S* spike, int64_t T, int64_t N, float a
     if (T == ROWS && waves == WAVES)                                                               \
         return launch_forward_rows<S, M, V, ROWS, false, WRITE_U, WRITE_S, KEEP, WAVES>(            \
             x, mem, spike, T, N, alpha, thresh, threads, stream);
-        SNNLIF_FWD_EXACT(1, 8)
-        SNNLIF_FWD_EXACT(2, 8)
-        SNNLIF_FWD_EXACT(3, 8)
+        SNNLIF_FWD_EXACT(3, 8)  // (one and two steps: launch_forward_short)
         SNNLIF_FWD_EXACT(4, 8)
         SNNLIF_FWD_EXACT(5, 5)
         SNNLIF_FWD_EXACT(6, 5)
