@@ -105,7 +105,9 @@ const char* snnlif_strerror(int code);
  * snnlif_bn_fire_bp_dist2) get the events attached to that dispatch -- `start_event` completes when
  * the kernel begins, `stop_event` when it has finished -- so hipEventElapsedTime(start, stop) is the
  * kernel's own duration, without the dispatch gaps an interval between two hipEventRecord markers
- * contains.  Entry points that launch several kernels (snnlif_bn_stats, snnlif_bn_fire_bp and its
+ * contains.  A start event costs a few microseconds of stream time per dispatch, a stop event alone
+ * none: stop events on consecutive launches give completion-to-completion intervals that add up to the
+ * wall clock (kernel duration plus dispatch gap), which is how bench.py times a saturated stream.  Entry points that launch several kernels (snnlif_bn_stats, snnlif_bn_fire_bp and its
  * _static and _dist1 forms, snnlif_fire_bp beyond SNNLIF_BP_NO_WORKSPACE_MAX_T steps) record
  * `start_event` on the stream before their first kernel and `stop_event` after their last: the whole
  * operation, gaps between its kernels included.

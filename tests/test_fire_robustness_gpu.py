@@ -162,6 +162,36 @@ def test_events_attached_to_the_next_kernel(cabi):
     assert np.array_equal(spike.cpu().numpy(), spike_o)
 
 
+def test_stop_events_alone_give_completion_intervals_that_add_up(cabi):
+    """How bench.py times its kernels: a stop event on every dispatch and no start event.  The interval
+    between two consecutive completions is positive, the intervals of a sequence of launches add up to the
+    interval between the first and the last completion, and that is no longer than the span between two
+    stream markers around the sequence."""
+    x = (0.5 + torch.randn(8, 16, 64, 32, 32)).cuda()
+    g = torch.randn_like(x)
+    spike, gx = torch.empty_like(x), torch.empty_like(x)
+    n = 6
+    stops = [torch.cuda.Event(enable_timing=True) for _ in range(2 * n)]
+    m0, m1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for e in stops:
+        e.record()
+    cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)   # warm-up
+    torch.cuda.synchronize()
+    m0.record()
+    for i in range(n):
+        cabi.time_next_kernel(None, stops[2 * i])
+        cabi.fire_s_fp_into(x, spike, ALPHA, THRESH)
+        cabi.time_next_kernel(None, stops[2 * i + 1])
+        cabi.fire_bp_into(x, g, gx, ALPHA, THRESH, BETA, INTERVAL)
+    m1.record()
+    torch.cuda.synchronize()
+    spans = [stops[i - 1].elapsed_time(stops[i]) for i in range(1, 2 * n)]
+    assert all(ms > 0.0 for ms in spans), spans
+    total = stops[0].elapsed_time(stops[-1])
+    assert abs(sum(spans) - total) <= 1e-3 * total + 2e-3, (sum(spans), total)
+    assert total <= m0.elapsed_time(m1) * 1.02
+
+
 def test_an_armed_timer_does_not_outlive_a_failed_call(cabi):
     """An entry point that returns an argument error consumes the arming: the events must not end up
     on the next, unrelated launch."""
