@@ -533,6 +533,36 @@ def run_bn(args, plain):
             "outputs_equal_across_sets": bool(all(torch.equal(o, outs[0]) for o in outs[1:])
                                               and all(torch.equal(q, gxs[0]) for q in gxs[1:])),
         }
+        if plain:
+            # the bias gradient of a layer that ends in a convolution, the same reduction without the squares:
+            # snnlif_channel_sum against the framework's torch.sum over the same axes, both cold
+            total = torch.empty_like(weight)
+            sev = [[[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(sets)]
+                   for _ in range(rounds + 1)]
+            for per_round in sev:   # (torch only reads an event it has recorded itself once)
+                for per_set in per_round:
+                    per_set[0].record()
+                    per_set[1].record()
+            torch.cuda.synchronize()
+            for r in range(rounds + 1):
+                for k in range(sets):
+                    lif_cabi.time_next_kernel(sev[r][k][0], sev[r][k][1])
+                    lif_cabi.channel_sum_into(gs[k], total, stats_ws)
+                for k in range(sets):
+                    sev[r][k][2].record()
+                    framework_total = torch.sum(gs[k], dim=(0, 1, 3, 4))
+                    sev[r][k][3].record()
+            torch.cuda.synchronize()
+            timed = [e for per_round in sev[1:] for e in per_round]
+            ours = sum(e[0].elapsed_time(e[1]) for e in timed) / len(timed)
+            framework = sum(e[2].elapsed_time(e[3]) for e in timed) / len(timed)
+            exact = gs[0].double().sum(dim=(0, 1, 3, 4))
+            result["roofline"]["cold"]["channel_sum"] = {
+                "kernel": "bn_stats_wave_kernel + bn_stats_finalize_kernel (sums only)",
+                "avg_ms": ours, "achieved": rate(4 * ns, ours), "frac": rate(4 * ns, ours) / HBM_PEAK_GBPS,
+                "framework_sum_avg_ms": framework,
+                "max_error_vs_float64": float((total.double() - exact).abs().max()),
+                "framework_max_error_vs_float64": float((framework_total.double() - exact).abs().max())}
         del xs, gs, outs, gxs
 
     if not args.no_cpu_baseline:

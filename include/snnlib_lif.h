@@ -40,8 +40,9 @@ extern "C" {
 
 /* 2: cache hints in `dtype`, snnlif_fire_bp_strided, snnlif_bn_stats, snnlif_bn_fire_bp_static and
  *    SNNLIF_ERR_SCRATCH, the plain batch-norm entry points (snnlif_bn_fp, snnlif_bn_bp and its halves).
- *    A library of version 1 rejects hinted dtypes with SNNLIF_ERR_DTYPE and lacks those symbols. */
-#define SNNLIF_ABI_VERSION 2
+ *    A library of version 1 rejects hinted dtypes with SNNLIF_ERR_DTYPE and lacks those symbols.
+ * 3: snnlif_channel_sum. */
+#define SNNLIF_ABI_VERSION 3
 
 /* Storage types. */
 #define SNNLIF_DTYPE_F32  0 /* float storage, fp32 arithmetic (the reference's training dtype) */
@@ -203,6 +204,20 @@ size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t 
 int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64_t T, int64_t B,
                     int64_t C, int64_t HW, int raw_moments, void* workspace, size_t workspace_bytes,
                     void* stream);
+
+/*
+ * Per-channel sum of a [T, B, C, HW] gradient over (T, B, HW), fp32 or fp64 (bf16:
+ * SNNLIF_ERR_UNSUPPORTED); `sum` is [C] of the storage type.  The bias gradient of the layers that end
+ * in a convolution: replaces at::sum(grad_conv, dim_conv) in bn_fire_conv_bp_cuda, its _dist2 form,
+ * fire_conv_bp_cuda and conv_bp_cuda (snnlib/cuda/snn_kernel_bp.cu:1261, 1338, 1401, 1435) for the
+ * dim_conv the reference's layers pass, (0, 1, 3, 4), every axis but the channel's (snnlib/example/snnlib_func.py:182, 215, 247, 357).
+ * The pass of snnlif_bn_stats with another last step: summed in double precision in a fixed order
+ * (reproducible), `grad` loaded with the default cache policy.  T, B or HW of zero with C > 0 is
+ * SNNLIF_ERR_ARG.  `workspace`: snnlif_bn_stats_workspace_bytes() bytes, 16-byte aligned, private to
+ * the call until the stream has run it.
+ */
+int snnlif_channel_sum(const void* grad, void* sum, int dtype, int64_t T, int64_t B, int64_t C,
+                       int64_t HW, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Batch-norm + fire forward (dtype SNNLIF_DTYPE_F32 or SNNLIF_DTYPE_F64, which also is the type of the

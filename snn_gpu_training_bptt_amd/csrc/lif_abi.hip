@@ -308,11 +308,39 @@ int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64
     if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const OperationTimer whole_operation(st);
+    const int stats_mode = raw_moments != 0 ? snnlif::kStatsMoments : snnlif::kStatsVariance;
     return SNNLIF_BN_DISPATCH(
         es,
-        snnlif::bn_stats_f32(CF(spatial), MF(mean), MF(var), raw_moments != 0, T, B, C, HW,
+        snnlif::bn_stats_f32(CF(spatial), MF(mean), MF(var), stats_mode, T, B, C, HW,
                              MD(workspace), st),
-        snnlif::bn_stats_f64(CD(spatial), MD(mean), MD(var), raw_moments != 0, T, B, C, HW,
+        snnlif::bn_stats_f64(CD(spatial), MD(mean), MD(var), stats_mode, T, B, C, HW,
+                             MD(workspace), st));
+}
+
+int snnlif_channel_sum(const void* grad, void* sum, int dtype, int64_t T, int64_t B, int64_t C,
+                       int64_t HW, void* workspace, size_t workspace_bytes, void* stream) {
+    const TimerScope timer_scope;
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    if (C == 0) return SNNLIF_OK;
+    // the kernels read a channel's first element: nothing to read in an empty channel
+    if (T == 0 || B == 0 || HW == 0) return SNNLIF_ERR_ARG;
+    if (!grad || !sum) return SNNLIF_ERR_ARG;
+    const void* ptrs[2] = {grad, sum};
+    if (!all_aligned(ptrs, 2, es)) return SNNLIF_ERR_ALIGN;
+    const size_t need = snnlif::bn_stats_workspace_elems(T, B, C, HW) * sizeof(double);
+    if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
+    if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const OperationTimer whole_operation(st);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_stats_f32(CF(grad), MF(sum), nullptr, snnlif::kStatsSums, T, B, C, HW,
+                             MD(workspace), st),
+        snnlif::bn_stats_f64(CD(grad), MD(sum), nullptr, snnlif::kStatsSums, T, B, C, HW,
                              MD(workspace), st));
 }
 

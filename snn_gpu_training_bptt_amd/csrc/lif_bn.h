@@ -126,9 +126,12 @@ inline size_t bn_plain_workspace_elems(int64_t T, int64_t B, int64_t C, int64_t 
 
 enum class SpatialHint;  // lif_kernels.h
 
+// What bn_stats_* writes (see below).
+constexpr int kStatsVariance = 0, kStatsMoments = 1, kStatsSums = 2;
+
 // Per scalar type F (suffix f32 = float, f64 = double):
-//   bn_stats_*           per-channel mean and biased variance (moments = false) or E[x] and E[x^2]
-//                        (moments = true) over (T, B, HW);
+//   bn_stats_*           over (T, B, HW), per channel: mean and biased variance (mode kStatsVariance),
+//                        E[x] and E[x^2] (kStatsMoments), or the plain sum into out_a alone (kStatsSums);
 //   bn_forward_*         from_ivar = false: stat is the variance and ivar is written; true: stat is
 //                        the inverse standard deviation and ivar is not touched.  keep_x: the caller's
 //                        cache hint for x (lif_kernels.h).
@@ -143,7 +146,7 @@ enum class SpatialHint;  // lif_kernels.h
                             const F* mean, F* ivar, F* spike, bool from_ivar, int64_t T,           \
                             int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,\
                             SpatialHint keep_x, hipStream_t stream);                               \
-    int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,      \
+    int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B,          \
                           int64_t C, int64_t HW, double* workspace, hipStream_t stream);           \
     int bn_backward_stats_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,      \
                                    const F* mean, const F* g, F* grad_weight, F* grad_bias,        \

@@ -1,13 +1,15 @@
 // Per-channel batch statistics of a [T, B, C, HW] activation for MI355X: mean and biased variance over
 // (T, B, HW), or the first two raw moments E[x], E[x^2] that a batch sharded over several GPUs
-// all-reduces (F = float or double).
+// all-reduces, or the plain per-channel sum (F = float or double).
 //
 // Reference: the layers compute these with framework reductions before calling the native op --
 // torch.var_mean(x, dim_bn, unbiased=False) in snnlib/example/snnlib_op.py:36-37, 76-78, 113-115, 175-177
 // and torch.mean(x), torch.mean(x**2) in the sharded layers, snnlib/example/snnlib_op.py:263-264,
 // 326-327, 386-387.  On MI355X the framework's Welford reduction over a [8,64,128,32,32] tensor runs at
 // 0.7 TB/s and costs five times the fused batch-norm + fire forward it feeds, so the statistics get a
-// kernel of their own.
+// kernel of their own.  The per-channel sum is the bias gradient of the layers with a convolution,
+// at::sum(grad_conv, dim_conv) in snnlib/cuda/snn_kernel_bp.cu:1261, 1338, 1401, 1435 (on a
+// [8,64,128,32,32] gradient the framework's reduction takes 148 us where this pass takes 43).
 //
 // One pass over x (4 bytes per neuron-step in fp32), HBM-bound, two kernels:
 //   1. partial sums.  Planes of at least 32 positions: wavefronts are laid over the (batch entry,
@@ -160,8 +162,9 @@ bn_stats_column_kernel(const F* __restrict__ x, double* __restrict__ part_d,
 }
 
 // One workgroup per channel: adds the channel's partial sums in double and writes
-//   moments == false:  out_a = mean,  out_b = biased variance
-//   moments == true:   out_a = E[x],  out_b = E[x^2]
+//   mode kStatsVariance:  out_a = mean,  out_b = biased variance
+//   mode kStatsMoments:   out_a = E[x],  out_b = E[x^2]
+//   mode kStatsSums:      out_a = sum of x,  out_b not touched
 // Wave layout: entries (b*C + c)*G + i for b < B, i < G.  Column layout: entries s*CHW + c*HW + i for
 // s < S, i < HW.  Both are "outer" groups of "inner" consecutive entries, outer_stride apart.
 template <typename F>
@@ -169,7 +172,7 @@ __global__ void __launch_bounds__(kReduceBlock)
 bn_stats_finalize_kernel(const F* __restrict__ x, const double* __restrict__ part_d,
                          const double* __restrict__ part_dd, F* __restrict__ out_a,
                          F* __restrict__ out_b, int64_t HW, int64_t outer, int64_t inner,
-                         int64_t outer_stride, double count, bool moments) {
+                         int64_t outer_stride, double count, int mode) {
     const int c = blockIdx.x;
     const int64_t base = static_cast<int64_t>(c) * inner;
     const int64_t n = outer * inner;
@@ -196,17 +199,21 @@ bn_stats_finalize_kernel(const F* __restrict__ x, const double* __restrict__ par
             sdd += lds[1][w];
         }
         const double shift = static_cast<double>(x[static_cast<int64_t>(c) * HW]);
+        if (mode == kStatsSums) {  // the plain sum: out_b is not written
+            out_a[c] = static_cast<F>(shift * count + sd);
+            return;
+        }
         const double mean_d = sd / count;
         double var = (sdd - sd * mean_d) / count;
         if (var < 0.0) var = 0.0;
         const double mean = shift + mean_d;
         out_a[c] = static_cast<F>(mean);
-        out_b[c] = static_cast<F>(moments ? var + mean * mean : var);
+        out_b[c] = static_cast<F>(mode == kStatsMoments ? var + mean * mean : var);
     }
 }
 
 template <typename F>
-int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B, int64_t C,
+int bn_stats(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B, int64_t C,
              int64_t HW, double* workspace, hipStream_t stream) {
     const int64_t N = B * C * HW;
     const size_t P = bn_stats_partial_count(T, B, C, HW);
@@ -237,7 +244,7 @@ int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,
         });
         if (rc != SNNLIF_OK) return rc;
         launch_kernel(bn_stats_finalize_kernel<F>, dim3(static_cast<unsigned>(C)), dim3(kReduceBlock),
-                      0, stream, x, part_d, part_dd, out_a, out_b, HW, S, G, C * G, count, moments);
+                      0, stream, x, part_d, part_dd, out_a, out_b, HW, S, G, C * G, count, mode);
         return launch_status();
     }
     const int64_t rows = T * B, CHW = C * HW;
@@ -249,7 +256,7 @@ int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,
     if (rc != SNNLIF_OK) return rc;
     launch_kernel(bn_stats_finalize_kernel<F>, dim3(static_cast<unsigned>(C)), dim3(kReduceBlock), 0,
                   stream, x, part_d, part_dd, out_a, out_b, HW, static_cast<int64_t>(S), HW, CHW, count,
-                  moments);
+                  mode);
     return launch_status();
 }
 
@@ -257,9 +264,9 @@ int bn_stats(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,
 
 #define SNNLIF_DEFINE_BN_STATS_DTYPE(SUFFIX, F)                                                    \
     namespace snnlif {                                                                             \
-    int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, bool moments, int64_t T, int64_t B,      \
+    int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B,          \
                           int64_t C, int64_t HW, double* workspace, hipStream_t stream) {          \
-        return bn_stats<F>(x, out_a, out_b, moments, T, B, C, HW, workspace, stream);              \
+        return bn_stats<F>(x, out_a, out_b, mode, T, B, C, HW, workspace, stream);                 \
     }                                                                                              \
     }
 

@@ -217,6 +217,46 @@ Tensor conv_folded(const Tensor& in, const Tensor& weight, const Tensor& bias,
     return reshaped_result(conv, {in.size(0), in.size(1), conv.size(1), conv.size(2), conv.size(3)});
 }
 
+// The bias gradient of the layers that end in a convolution: at::sum(grad_conv, dim_conv) in the
+// reference (snnlib/cuda/snn_kernel_bp.cu:1261, 1338, 1401, 1435).  For the dim_conv its layers pass --
+// every axis but the channel's, (0, 1, 3, 4) -- a dense fp32 / fp64 gradient with planes of at least
+// kChannelSumMinPlane positions takes the hand-written per-channel reduction (snnlif_channel_sum, one
+// pass at the rate of the batch statistics; the framework's reduction over these axes runs at a
+// third of it); any other reduction stays with ATen.
+constexpr int64_t kChannelSumMinPlane = 32;
+
+bool all_axes_but_channel(const IntList& dims, int64_t rank) {
+    if (rank < 4 || static_cast<int64_t>(dims.size()) != rank - 1) return false;
+    std::vector<bool> seen(static_cast<size_t>(rank), false);
+    for (int64_t d : dims) {
+        if (d < 0) d += rank;
+        if (d < 0 || d >= rank || d == 2 || seen[static_cast<size_t>(d)]) return false;
+        seen[static_cast<size_t>(d)] = true;
+    }
+    return true;
+}
+
+Tensor bias_gradient(const Tensor& grad, const IntList& dims, const char* op) {
+    const bool native_type = grad.scalar_type() == at::kFloat || grad.scalar_type() == at::kDouble;
+    if (!grad.is_cuda() || !native_type || !all_axes_but_channel(dims, grad.dim()) ||
+        grad.numel() == 0)
+        return at::sum(grad, dims);
+    const BnDims d = bn_dims_of(grad, op);
+    if (d.HW < kChannelSumMinPlane) return at::sum(grad, dims);
+    const int dtype = grad.scalar_type() == at::kFloat ? SNNLIF_DTYPE_F32 : SNNLIF_DTYPE_F64;
+    const DeviceGuard guard(grad.device());
+    Tensor g = grad.contiguous();
+    Tensor sum = torch::empty({d.C}, g.options());
+    const size_t ws_bytes = snnlif_bn_stats_workspace_bytes(dtype, d.T, d.B, d.C, d.HW);
+    Tensor workspace =
+        torch::empty({static_cast<int64_t>(ws_bytes)}, g.options().dtype(at::kByte));
+    check_rc(snnlif_channel_sum(g.data_ptr(), sum.data_ptr(), dtype, d.T, d.B, d.C, d.HW,
+                                ws_bytes ? workspace.data_ptr() : nullptr, ws_bytes,
+                                current_stream()),
+             op);
+    return sum;
+}
+
 // -> {grad_in (shaped like `in`), grad_weight, grad_bias}
 std::vector<Tensor> conv_backward_folded(const Tensor& in, const Tensor& grad_conv,
                                          const Tensor& weight, const IntList& stride,
@@ -228,12 +268,13 @@ std::vector<Tensor> conv_backward_folded(const Tensor& in, const Tensor& grad_co
                     grad_conv.size(1) == in.size(1) && grad_conv.size(2) == weight.size(0),
                 "snnlib.", op, ": grad_conv must be [T, B, cout, Hout, Wout], got ",
                 grad_conv.sizes());
+    const Tensor grad_dense = grad_conv.contiguous();
     auto grads = at::convolution_backward(
-        fold_time(grad_conv.contiguous()), fold_time(in), weight, /*bias_sizes=*/c10::nullopt,
+        fold_time(grad_dense), fold_time(in), weight, /*bias_sizes=*/c10::nullopt,
         stride, padding, dilation, /*transposed=*/false, /*output_padding=*/{0, 0}, groups,
         /*output_mask=*/{true, true, false});
     return {reshaped_result(std::get<0>(grads), in.sizes()), std::get<1>(grads),
-            at::sum(grad_conv, dim_conv)};
+            bias_gradient(grad_dense, dim_conv, op)};
 }
 
 // ---- fire ---------------------------------------------------------------------------------------

@@ -34,6 +34,7 @@ SYMBOLS = {
                                       _sz, _vp]),
     "snnlif_bn_stats_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "snnlif_bn_stats": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
+    "snnlif_channel_sum": (_int, [_vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "snnlif_bn_fire_s_fp": (_int, [_vp] * 7 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _vp]),
     "snnlif_bn_fire_s_recompute": (_int, [_vp] * 6 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _vp]),
     "snnlif_bn_fire_bp_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
@@ -47,7 +48,7 @@ SYMBOLS = {
     "snnlif_bn_bp_dist1": (_int, [_vp] * 9 + [_int, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "snnlif_bn_bp_dist2": (_int, [_vp] * 8 + [_int, _i64, _i64, _i64, _i64, _vp]),
 }
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _lib = None
 
@@ -280,6 +281,20 @@ def bn_stats_into(spatial, mean, var, workspace, raw_moments=False):
                                 workspace.data_ptr(), workspace.numel(), _stream_handle(spatial))
     _check(rc, "snnlif_bn_stats")
     return mean, var
+
+
+def channel_sum_into(grad, total, workspace):
+    """``snnlif_channel_sum``: per-channel sum of ``grad`` ([T, B, C, ...]) over all axes but the
+    channel's; writes ``total`` ([C]).  ``workspace`` as for ``bn_stats_into``."""
+    T, B, C, HW = _bn_dims(grad)
+    _require_per_channel(grad, C, total=total)
+    _require_workspace(grad, workspace, bn_stats_workspace_bytes(_torch_dtype_code(grad), T, B, C, HW),
+                       "snnlif_channel_sum")
+    _require_dense_gpu(grad, total, workspace)
+    rc = load().snnlif_channel_sum(grad.data_ptr(), total.data_ptr(), _torch_dtype_code(grad), T, B, C,
+                                   HW, workspace.data_ptr(), workspace.numel(), _stream_handle(grad))
+    _check(rc, "snnlif_channel_sum")
+    return total
 
 
 def bn_fire_s_fp_into(spatial, weight, bias, var, mean, ivar, spike, eps, alpha, thresh, keep_spatial=None):

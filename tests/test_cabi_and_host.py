@@ -55,7 +55,7 @@ def test_constants_match_the_header():
     assert int(macros["SNNLIF_BP_FUSED_MAX_T"]) == lif_cabi.BP_FUSED_MAX_T
     assert int(macros["SNNLIF_BP_NO_WORKSPACE_MAX_T"]) == lif_cabi.BP_NO_WORKSPACE_MAX_T
     lib = lif_cabi.load()
-    assert lib.snnlif_abi_version() == int(macros["SNNLIF_ABI_VERSION"]) == lif_cabi.ABI_VERSION == 2
+    assert lib.snnlif_abi_version() == int(macros["SNNLIF_ABI_VERSION"]) == lif_cabi.ABI_VERSION == 3
     assert lif_cabi.bn_bp_workspace_bytes(lif_cabi.DTYPE_F32, 8, 64, 128, 1024) == (2 * 64 * 128 * 16 + 2 * 128) * 4
     assert lif_cabi.bn_bp_workspace_bytes(lif_cabi.DTYPE_F64, 6, 2, 8, 1) == (2 * 2 * 8 + 2 * 8) * 8
     assert lif_cabi.bn_bp_workspace_bytes(lif_cabi.DTYPE_BF16, 6, 2, 8, 1) == 0
