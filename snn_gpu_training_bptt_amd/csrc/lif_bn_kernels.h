@@ -439,24 +439,31 @@ bn_channel_reduce_finalize_kernel(const F* __restrict__ part_gy,
     }
 }
 
-// One lane per channel: fold the S slices and the HW positions of the channel in order, emit the
-// parameter gradients and the two coefficients the input-gradient sweep needs.
+// One wavefront per channel: lane l adds entries l, l + 64, ... of the channel's S*HW partial sums
+// (slice-major), the wavefront folds its lanes by shuffles -- an order fixed by S and HW alone -- and
+// lane 0 emits the parameter gradients and the two coefficients the input-gradient sweep needs.
+// (One lane per channel walking the S*HW entries one after the other took 68 us for 512 channels of 16
+// positions in 32 slices: a chain of dependent memory round trips.)
 template <typename F>
 __global__ void __launch_bounds__(kReduceBlock)
 bn_channel_finalize_kernel(const F* __restrict__ split, const F* __restrict__ weight,
                            F* __restrict__ grad_weight, F* __restrict__ grad_bias,
                            F* __restrict__ mean_gxhat, F* __restrict__ mean_gxhatx,
                            int64_t C, int64_t HW, int S, F count) {
-    const int64_t c = static_cast<int64_t>(blockIdx.x) * kReduceBlock + threadIdx.x;
-    if (c >= C) return;
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * (kReduceBlock / 64) + threadIdx.x / 64;
+    if (c >= C) return;  // whole wavefronts leave together
+    const int lane = threadIdx.x % 64;
     const int64_t CHW = C * HW;
+    const int64_t n = static_cast<int64_t>(S) * HW;
     F a = F(0), ax = F(0);
-    for (int s = 0; s < S; ++s) {
-        for (int64_t i = 0; i < HW; ++i) {
-            a += split[static_cast<int64_t>(s) * CHW + c * HW + i];
-            ax += split[(static_cast<int64_t>(S) + s) * CHW + c * HW + i];
-        }
+    for (int64_t e = lane; e < n; e += 64) {
+        const int64_t s = e / HW, i = e - s * HW;
+        a += split[s * CHW + c * HW + i];
+        ax += split[(static_cast<int64_t>(S) + s) * CHW + c * HW + i];
     }
+    a = wave_sum(a);
+    ax = wave_sum(ax);
+    if (lane != 0) return;
     grad_bias[c] = a;
     grad_weight[c] = ax;
     const F wgt = weight[c];

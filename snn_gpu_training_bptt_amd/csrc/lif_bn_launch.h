@@ -141,7 +141,7 @@ int bn_backward_stats_window(const F* x, const F* weight, const F* bias, const F
     rc = launch_status();
     if (rc != SNNLIF_OK) return rc;
     launch_kernel(bn_channel_finalize_kernel<F>,
-                  dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
+                  dim3(static_cast<unsigned>((C + kReduceBlock / 64 - 1) / (kReduceBlock / 64))),
                   dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias, mean_gxhat,
                   mean_gxhatx, C, HW, S, count);
     return launch_status();

@@ -377,7 +377,7 @@ int bn_plain_backward_stats(const F* x, const F* weight, const F* ivar, const F*
     int rc = launch_status();
     if (rc != SNNLIF_OK) return rc;
     launch_kernel(bn_channel_finalize_kernel<F>,
-                  dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)),
+                  dim3(static_cast<unsigned>((C + kReduceBlock / 64 - 1) / (kReduceBlock / 64))),
                   dim3(kReduceBlock), 0, stream, split, weight, grad_weight, grad_bias, mean_gxhat,
                   mean_gxhatx, C, HW, static_cast<int>(S), count);
     return launch_status();
