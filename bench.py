@@ -4,6 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2|cfg3|cfg5|cfg5_bf16|cfg1|t96|t100|t120]
                     [--no-cpu-baseline] [--no-extra-legs]
     python bench.py --workload train_step [--steps K] [--warmup W]     (context figure, see below)
+    python bench.py --workload cifar_step [--steps K] [--warmup W]     (context figure, see below)
     python bench.py --workload bn_fire    [--steps K] [--warmup W]     (next-row op, see below)
     python bench.py --workload bn         [--steps K] [--warmup W]     (next-row op, see below)
     python bench.py --workload policy_sweep                            (kernel rates over shapes, see below)
@@ -50,6 +51,14 @@ byte comes from HBM.
 spiking CNN on CIFAR-shaped random data (conv / linear / pooling on PyTorch-ROCm, the four LIF layers
 through ``snnlib_op.Fire``) and reports the end-to-end step time and the share of it spent in the
 fire kernels, measured with events around the ``snnlib.fire_s_fp`` / ``snnlib.fire_bp`` calls.
+
+``--workload cifar_step`` is a context figure too: one SGD step of the reference's CIFAR model
+(snnlib/example/models.py:8-61: nine 3x3 convolutions of 128 / 256 / 512 channels, 8192-1024-512 fully
+connected, every layer but the first a batch norm + fire fused with the dense op that follows) assembled from
+this package's ``snnlib_op`` layers, with the batch size, window and optimiser of the reference's training
+script (snnlib/example/train_test_cifar.py:19, 32: 64 images, SGD lr 1e-2 momentum 0.9; 6 steps) on random
+CIFAR-shaped data.  Reports the step time and the GPU time inside each native op of the ``snnlib`` module
+(events around the calls; a fused op's time includes its MIOpen / rocBLAS half).
 
 ``--workload bn_fire`` times the batch-norm + fire layer's training step (``snnlif_bn_stats``,
 ``snnlif_bn_fire_s_fp``, ``snnlif_bn_fire_bp``) at the headline shape through the C ABI: 4 B per
@@ -377,6 +386,107 @@ def run_train_step(args):
     }), flush=True)
 
 
+def run_cifar_step(args):
+    import torch
+    from snn_gpu_training_bptt_amd import snnlib_func as sf
+    from snn_gpu_training_bptt_amd import snnlib_op as sop
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no ROCm GPU visible")
+    dev = torch.device("cuda:0")
+    T, B = 6, 64
+    sf.time_step = T
+
+    class Cifar(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            s1, s2, p = (1, 1), (2, 2), (1, 1)
+            self.conv1_1 = sop.Conv(3, 128, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv1_2 = sop.BnFireConv(128, 128, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv1_3 = sop.BnFireConv(128, 128, kernel_size=(3, 3), stride=s2, padding=p)
+            self.conv2_1 = sop.BnFireConv(128, 256, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv2_2 = sop.BnFireConv(256, 256, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv2_3 = sop.BnFireConv(256, 256, kernel_size=(3, 3), stride=s2, padding=p)
+            self.conv3_1 = sop.BnFireConv(256, 512, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv3_2 = sop.BnFireConv(512, 512, kernel_size=(3, 3), stride=s1, padding=p)
+            self.conv3_3 = sop.BnFireConv(512, 512, kernel_size=(3, 3), stride=s2, padding=p)
+            self.fc1 = sop.BnFireFc(4 * 4 * 512, 1024, dim_bn=(0, 1, 3, 4), cin_bn=512)
+            self.fc2 = sop.BnFireFc(1024, 512, dim_bn=(0, 1))
+            self.bn = sop.BnFire(512, dim_bn=(0, 1))
+            self.fc3 = torch.nn.Linear(512, 10)
+            self.stack = ("conv1_1", "conv1_2", "conv1_3", "conv2_1", "conv2_2", "conv2_3", "conv3_1",
+                          "conv3_2", "conv3_3", "fc1", "fc2", "bn")
+
+        def forward(self, images):
+            x = torch.stack([images for _ in range(T)], dim=0)
+            for name in self.stack:
+                x = getattr(self, name)(x)
+            return self.fc3(x.mean(dim=0))
+
+    torch.manual_seed(SEED)
+    net = Cifar().to(dev)
+    gen = torch.Generator().manual_seed(SEED)
+    images = torch.rand((B, 3, 32, 32), generator=gen).to(dev)
+    labels = torch.randint(0, 10, (B,), generator=gen).to(dev)
+    opt = torch.optim.SGD([q for n, q in net.named_parameters() if "running" not in n], lr=1e-2, momentum=0.9)
+    crit = torch.nn.CrossEntropyLoss()
+
+    native = sf.snnlib
+    spans = []
+
+    class TimedOps:
+        def __getattr__(self, name):
+            fn = getattr(native, name)
+
+            def timed(*a):
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                e0.record()
+                out = fn(*a)
+                e1.record()
+                spans.append((name, e0, e1))
+                return out
+            return timed
+
+    def one_step():
+        opt.zero_grad(set_to_none=True)
+        loss = crit(net(images), labels)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(max(args.warmup, 2)):     # (MIOpen picks its algorithms during the first steps)
+        one_step()
+    torch.cuda.synchronize()
+    sf.snnlib = TimedOps()
+    try:
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = one_step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    finally:
+        sf.snnlib = native
+    step_ms = (t1 - t0) / args.steps * 1e3
+    per_op = {}
+    for name, e0, e1 in spans:
+        per_op[name] = per_op.get(name, 0.0) + e0.elapsed_time(e1) / args.steps
+    fused_free = sum(v for k, v in per_op.items() if k in ("bn_stats", "bn_fire_s_fp", "bn_fire_bp"))
+    print(json.dumps({
+        "metric": "CIFAR_BN training step (context figure, not the headline metric)",
+        "value": step_ms, "unit": "ms/step", "higher_is_better": False, "n_gpus": 1,
+        "steps": args.steps, "warmup": max(args.warmup, 2), "ms_per_step": step_ms, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "cifar_step: the reference's CIFAR_BN model (models.py:8-61) from snnlib_op layers, "
+                               f"T={T} B={B}, random CIFAR-shaped batch, SGD lr 1e-2 momentum 0.9, cross entropy"},
+        "images_per_s": B / (step_ms * 1e-3),
+        "native_op_ms_per_step": {k: round(v, 4) for k, v in sorted(per_op.items(), key=lambda kv: -kv[1])},
+        "native_ops_ms_per_step": sum(per_op.values()),
+        "ops_without_a_dense_half_ms_per_step": fused_free,
+        "final_loss": float(loss.item()),
+    }), flush=True)
+
+
 def run_bn(args, plain):
     """The training step of a batch-norm layer at the headline shape through the C ABI: batch statistics,
     forward, backward.  plain = False: batch norm folded into the fire recurrence (snnlif_bn_fire_*);
@@ -692,7 +802,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step", "bn_fire", "bn", "policy_sweep"])
+    ap.add_argument("--workload", default="cfg2", choices=sorted(WORKLOADS) + ["train_step", "cifar_step", "bn_fire", "bn", "policy_sweep"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra-legs", "--no-cold-leg", dest="no_extra_legs", action="store_true",
                     help="run the timed region only (fire workloads: no cabi_streamed / same_tensors / kept "
@@ -707,6 +817,12 @@ def main():
         sys.exit("bench.py: this build measures one GPU only (the fire op needs no communication; "
                  "neurons shard across GPUs with zero exchange). Run with --gpus 1.")
 
+    if args.workload == "cifar_step":
+        if args.steps == 200:
+            args.steps = 10
+        if args.warmup == 20:
+            args.warmup = 3
+        return run_cifar_step(args)
     if args.workload == "train_step":
         if args.steps == 200:
             args.steps = 10
