@@ -41,7 +41,7 @@ extern "C" {
 /* 2: cache hints in `dtype`, snnlif_fire_bp_strided, snnlif_bn_stats, snnlif_bn_fire_bp_static and
  *    SNNLIF_ERR_SCRATCH, the plain batch-norm entry points (snnlif_bn_fp, snnlif_bn_bp and its halves).
  *    A library of version 1 rejects hinted dtypes with SNNLIF_ERR_DTYPE and lacks those symbols.
- * 3: snnlif_channel_sum. */
+ * 3: snnlif_channel_sum, snnlif_bn_stats_running, snnlif_bn_moments_finish. */
 #define SNNLIF_ABI_VERSION 3
 
 /* Storage types. */
@@ -192,9 +192,8 @@ size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t 
  *   raw_moments == 0:  mean[c] = E[x],  var[c] = E[(x - mean[c])^2]  (biased: divided by T*B*HW)
  *   raw_moments != 0:  mean[c] = E[x],  var[c] = E[x^2]              (what a sharded batch all-reduces)
  * Replaces the framework reductions the reference's layers run before every batch-norm op:
- * torch.var_mean(x, dim_bn, unbiased=False) (snnlib/example/snnlib_op.py:36-37, 76-78, 113-115,
- * 175-177) and torch.mean(x), torch.mean(x**2) of the sharded layers (snnlib/example/snnlib_op.py:263-264,
- * 326-327, 386-387).  One pass over the tensor; sums are taken of x minus the channel's first element, in
+ * torch.var_mean(x, dim_bn, unbiased=False) (snnlib/example/snnlib_op.py:44, 78, 122, 184) and torch.mean(x), torch.mean(x**2) of the sharded layers (snnlib/example/snnlib_op.py:265-266,
+ * 328-329, 388-389).  One pass over the tensor; sums are taken of x minus the channel's first element, in
  * double precision throughout, and added up per channel in a fixed order (reproducible results).  `spatial` is
  * loaded with the default cache policy, so a tensor that fits the memory-side cache is still there
  * for the batch-norm op that follows.  T, B or HW of zero with C > 0 is SNNLIF_ERR_ARG (a channel
@@ -204,6 +203,39 @@ size_t snnlif_bn_stats_workspace_bytes(int dtype, int64_t T, int64_t B, int64_t 
 int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64_t T, int64_t B,
                     int64_t C, int64_t HW, int raw_moments, void* workspace, size_t workspace_bytes,
                     void* stream);
+
+/*
+ * snnlif_bn_stats (mean and biased variance) together with the layer's running statistics: what the
+ * reference's layers do after torch.var_mean in training mode (snnlib/example/snnlib_op.py:44-46, 78-80,
+ * 122-124, 184-186),
+ *   new_running_mean[c] = (running_mean[c] * keep) + (mean[c] * gain_mean)
+ *   new_running_var[c]  = (running_var[c]  * keep) + (var[c]  * gain_var)
+ * with keep = 0.9, gain_mean = 0.1, gain_var = 0.1 * n / (n - 1) there.  The factors are rounded to the
+ * storage type once and every product and sum is rounded in it, so the results carry the bits of the
+ * framework's element-wise expression; they are formed in the last step of the statistics pass (no
+ * further kernel: six small launches per layer and step less).  new_running_* may alias running_*.
+ * Arguments, workspace and errors as for snnlif_bn_stats; all seven tensors are required.
+ */
+int snnlif_bn_stats_running(const void* spatial, void* mean, void* var, const void* running_mean,
+                            const void* running_var, void* new_running_mean, void* new_running_var,
+                            double keep, double gain_mean, double gain_var, int dtype, int64_t T,
+                            int64_t B, int64_t C, int64_t HW, void* workspace, size_t workspace_bytes,
+                            void* stream);
+
+/*
+ * Statistics of a batch sharded over `world_size` ranks from its all-reduced raw moments, as the
+ * reference's sharded layers form them (snnlib/example/snnlib_op.py:271-275, 334-338, 394-398):
+ *   mean[c] = first[c] / world_size;   var[c] = second[c] / world_size - mean[c]^2
+ * and, when the four running pointers are given, the running pair as in snnlif_bn_stats_running (keep =
+ * 0.95, gains 0.05 and 0.05 * n / (n - 1) there).  The division is a product with 1 / world_size rounded
+ * to the storage type and the square a product, as the framework evaluates them: same bits as the
+ * reference's ten small element-wise launches, in one.  [C] vectors of fp32 or fp64; world_size >= 1.
+ */
+int snnlif_bn_moments_finish(const void* first, const void* second, void* mean, void* var,
+                             const void* running_mean, const void* running_var,
+                             void* new_running_mean, void* new_running_var, double world_size,
+                             double keep, double gain_mean, double gain_var, int dtype, int64_t C,
+                             void* stream);
 
 /*
  * Per-channel sum of a [T, B, C, HW] gradient over (T, B, HW), fp32 or fp64 (bf16:

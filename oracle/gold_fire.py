@@ -70,7 +70,7 @@ def gold_bn_fire(x, weight, bias, running_mean, running_var, training, eps, alph
     """Batch norm over the folded (T*B) batch, then the fire loop (snnlib/example/gold_op.py:67-87,
     whose ``bn`` is ``nn.BatchNorm1d`` / ``nn.BatchNorm2d``).  Returns ``(u, s)``.  With
     ``training=True`` the statistics are those of ``x`` itself, as in the reference layer's training
-    mode (snnlib/example/snnlib_op.py:76-78 computes them with ``torch.var_mean(..., unbiased=False)``)."""
+    mode (snnlib/example/snnlib_op.py:78 computes them with ``torch.var_mean(..., unbiased=False)``)."""
     shape = x.shape
     y = torch.nn.functional.batch_norm(x.reshape(shape[0] * shape[1], *shape[2:]), running_mean,
                                        running_var, weight, bias, training, 0.1, eps).reshape(shape)

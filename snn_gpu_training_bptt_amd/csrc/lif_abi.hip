@@ -317,6 +317,88 @@ int snnlif_bn_stats(const void* spatial, void* mean, void* var, int dtype, int64
                              MD(workspace), st));
 }
 
+}  // extern "C"
+
+template <typename F>
+static snnlif::RunningUpdate<F> running_update(const void* running_mean, const void* running_var,
+                                               void* new_running_mean, void* new_running_var,
+                                               double keep, double gain_mean, double gain_var) {
+    // the factors are rounded to the storage type once, as the framework rounds a Python scalar
+    return snnlif::RunningUpdate<F>{static_cast<const F*>(running_mean), static_cast<const F*>(running_var),
+                                    static_cast<F*>(new_running_mean), static_cast<F*>(new_running_var),
+                                    static_cast<F>(keep), static_cast<F>(gain_mean), static_cast<F>(gain_var)};
+}
+
+extern "C" {
+
+int snnlif_bn_stats_running(const void* spatial, void* mean, void* var, const void* running_mean,
+                            const void* running_var, void* new_running_mean, void* new_running_var,
+                            double keep, double gain_mean, double gain_var, int dtype, int64_t T,
+                            int64_t B, int64_t C, int64_t HW, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+    const TimerScope timer_scope;
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
+    const int se = bn_shape_error(T, B, C, HW);
+    if (se != SNNLIF_OK) return se;
+    if (C == 0) return SNNLIF_OK;
+    if (T == 0 || B == 0 || HW == 0) return SNNLIF_ERR_ARG;
+    if (!spatial || !mean || !var || !running_mean || !running_var || !new_running_mean ||
+        !new_running_var)
+        return SNNLIF_ERR_ARG;
+    const void* ptrs[7] = {spatial, mean, var, running_mean, running_var, new_running_mean, new_running_var};
+    if (!all_aligned(ptrs, 7, es)) return SNNLIF_ERR_ALIGN;
+    const size_t need = snnlif::bn_stats_workspace_elems(T, B, C, HW) * sizeof(double);
+    if (workspace == nullptr || workspace_bytes < need) return SNNLIF_ERR_WORKSPACE;
+    if (!snnlif::aligned_to(workspace, 16)) return SNNLIF_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const OperationTimer whole_operation(st);
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_stats_f32(CF(spatial), MF(mean), MF(var), snnlif::kStatsVariance, T, B, C, HW,
+                             MD(workspace), st,
+                             running_update<float>(running_mean, running_var, new_running_mean,
+                                                   new_running_var, keep, gain_mean, gain_var)),
+        snnlif::bn_stats_f64(CD(spatial), MD(mean), MD(var), snnlif::kStatsVariance, T, B, C, HW,
+                             MD(workspace), st,
+                             running_update<double>(running_mean, running_var, new_running_mean,
+                                                    new_running_var, keep, gain_mean, gain_var)));
+}
+
+int snnlif_bn_moments_finish(const void* first, const void* second, void* mean, void* var,
+                             const void* running_mean, const void* running_var,
+                             void* new_running_mean, void* new_running_var, double world_size,
+                             double keep, double gain_mean, double gain_var, int dtype, int64_t C,
+                             void* stream) {
+    const TimerScope timer_scope;
+    int rc = SNNLIF_OK;
+    const size_t es = bn_element_size(dtype, &rc);
+    if (es == 0) return rc;
+    if (C < 0 || !(world_size >= 1.0)) return SNNLIF_ERR_ARG;
+    if (C == 0) return SNNLIF_OK;
+    if (!first || !second || !mean || !var) return SNNLIF_ERR_ARG;
+    // the running pair is optional, but all four of its pointers go together
+    const int given = (running_mean != nullptr) + (running_var != nullptr) +
+                      (new_running_mean != nullptr) + (new_running_var != nullptr);
+    if (given != 0 && given != 4) return SNNLIF_ERR_ARG;
+    const void* ptrs[8] = {first, second, mean, var, running_mean, running_var, new_running_mean, new_running_var};
+    if (!all_aligned(ptrs, given ? 8 : 4, es)) return SNNLIF_ERR_ALIGN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    // 1 / world in the storage type: the framework divides by a scalar as a product with its reciprocal
+    return SNNLIF_BN_DISPATCH(
+        es,
+        snnlif::bn_moments_finish_f32(CF(first), CF(second), MF(mean), MF(var),
+                                      1.0f / static_cast<float>(world_size),
+                                      running_update<float>(running_mean, running_var, new_running_mean,
+                                                            new_running_var, keep, gain_mean, gain_var),
+                                      C, st),
+        snnlif::bn_moments_finish_f64(CD(first), CD(second), MD(mean), MD(var), 1.0 / world_size,
+                                      running_update<double>(running_mean, running_var, new_running_mean,
+                                                             new_running_var, keep, gain_mean, gain_var),
+                                      C, st));
+}
+
 int snnlif_channel_sum(const void* grad, void* sum, int dtype, int64_t T, int64_t B, int64_t C,
                        int64_t HW, void* workspace, size_t workspace_bytes, void* stream) {
     const TimerScope timer_scope;

@@ -129,9 +129,24 @@ enum class SpatialHint;  // lif_kernels.h
 // What bn_stats_* writes (see below).
 constexpr int kStatsVariance = 0, kStatsMoments = 1, kStatsSums = 2;
 
+// The running statistics a layer keeps beside the batch statistics, advanced as the reference's layers do
+// (snnlib/example/snnlib_op.py:79-80, 274-275): out = (in * keep) + (stat * gain), each product and the
+// sum rounded in F like the framework's element-wise ops.  Null outputs: no update.
+template <typename F>
+struct RunningUpdate {
+    const F* mean_in;
+    const F* var_in;
+    F* mean_out;
+    F* var_out;
+    F keep, gain_mean, gain_var;
+};
+
 // Per scalar type F (suffix f32 = float, f64 = double):
-//   bn_stats_*           over (T, B, HW), per channel: mean and biased variance (mode kStatsVariance),
+//   bn_stats_*           over (T, B, HW), per channel: mean and biased variance (mode kStatsVariance; with
+//                        `running`, the layer's running pair is advanced in the same finish),
 //                        E[x] and E[x^2] (kStatsMoments), or the plain sum into out_a alone (kStatsSums);
+//   bn_moments_finish_*  mean = first * inv_world, var = second * inv_world - mean^2 from the moments a
+//                        sharded batch has all-reduced, and the running pair, in one small kernel;
 //   bn_forward_*         from_ivar = false: stat is the variance and ivar is written; true: stat is
 //                        the inverse standard deviation and ivar is not touched.  keep_x: the caller's
 //                        cache hint for x (lif_kernels.h).
@@ -147,7 +162,10 @@ constexpr int kStatsVariance = 0, kStatsMoments = 1, kStatsSums = 2;
                             int64_t B, int64_t C, int64_t HW, float eps, float alpha, float thresh,\
                             SpatialHint keep_x, hipStream_t stream);                               \
     int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B,          \
-                          int64_t C, int64_t HW, double* workspace, hipStream_t stream);           \
+                          int64_t C, int64_t HW, double* workspace, hipStream_t stream,            \
+                          const RunningUpdate<F>& running = RunningUpdate<F>{});                   \
+    int bn_moments_finish_##SUFFIX(const F* first, const F* second, F* mean, F* var, F inv_world,  \
+                                   const RunningUpdate<F>& running, int64_t C, hipStream_t stream);\
     int bn_backward_stats_##SUFFIX(const F* x, const F* weight, const F* bias, const F* ivar,      \
                                    const F* mean, const F* g, F* grad_weight, F* grad_bias,        \
                                    F* mean_gxhat, F* mean_gxhatx, int64_t T, int64_t B, int64_t C, \

@@ -3,9 +3,9 @@
 // all-reduces, or the plain per-channel sum (F = float or double).
 //
 // Reference: the layers compute these with framework reductions before calling the native op --
-// torch.var_mean(x, dim_bn, unbiased=False) in snnlib/example/snnlib_op.py:36-37, 76-78, 113-115, 175-177
-// and torch.mean(x), torch.mean(x**2) in the sharded layers, snnlib/example/snnlib_op.py:263-264,
-// 326-327, 386-387.  On MI355X the framework's Welford reduction over a [8,64,128,32,32] tensor runs at
+// torch.var_mean(x, dim_bn, unbiased=False) in snnlib/example/snnlib_op.py:44, 78, 122, 184
+// and torch.mean(x), torch.mean(x**2) in the sharded layers, snnlib/example/snnlib_op.py:265-266,
+// 328-329, 388-389.  On MI355X the framework's Welford reduction over a [8,64,128,32,32] tensor runs at
 // 0.7 TB/s and costs five times the fused batch-norm + fire forward it feeds, so the statistics get a
 // kernel of their own.  The per-channel sum is the bias gradient of the layers with a convolution,
 // at::sum(grad_conv, dim_conv) in snnlib/cuda/snn_kernel_bp.cu:1261, 1338, 1401, 1435 (on a
@@ -172,7 +172,7 @@ __global__ void __launch_bounds__(kReduceBlock)
 bn_stats_finalize_kernel(const F* __restrict__ x, const double* __restrict__ part_d,
                          const double* __restrict__ part_dd, F* __restrict__ out_a,
                          F* __restrict__ out_b, int64_t HW, int64_t outer, int64_t inner,
-                         int64_t outer_stride, double count, int mode) {
+                         int64_t outer_stride, double count, int mode, RunningUpdate<F> running) {
     const int c = blockIdx.x;
     const int64_t base = static_cast<int64_t>(c) * inner;
     const int64_t n = outer * inner;
@@ -207,14 +207,20 @@ bn_stats_finalize_kernel(const F* __restrict__ x, const double* __restrict__ par
         double var = (sdd - sd * mean_d) / count;
         if (var < 0.0) var = 0.0;
         const double mean = shift + mean_d;
-        out_a[c] = static_cast<F>(mean);
-        out_b[c] = static_cast<F>(mode == kStatsMoments ? var + mean * mean : var);
+        const F mean_f = static_cast<F>(mean);
+        const F second_f = static_cast<F>(mode == kStatsMoments ? var + mean * mean : var);
+        out_a[c] = mean_f;
+        out_b[c] = second_f;
+        if (running.mean_out != nullptr) {  // (mode kStatsVariance) from the rounded statistics, as a reader of out_* would
+            running.mean_out[c] = running.mean_in[c] * running.keep + mean_f * running.gain_mean;
+            running.var_out[c] = running.var_in[c] * running.keep + second_f * running.gain_var;
+        }
     }
 }
 
 template <typename F>
 int bn_stats(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B, int64_t C,
-             int64_t HW, double* workspace, hipStream_t stream) {
+             int64_t HW, double* workspace, hipStream_t stream, const RunningUpdate<F>& running) {
     const int64_t N = B * C * HW;
     const size_t P = bn_stats_partial_count(T, B, C, HW);
     double* part_d = workspace;
@@ -244,7 +250,7 @@ int bn_stats(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B, int
         });
         if (rc != SNNLIF_OK) return rc;
         launch_kernel(bn_stats_finalize_kernel<F>, dim3(static_cast<unsigned>(C)), dim3(kReduceBlock),
-                      0, stream, x, part_d, part_dd, out_a, out_b, HW, S, G, C * G, count, mode);
+                      0, stream, x, part_d, part_dd, out_a, out_b, HW, S, G, C * G, count, mode, running);
         return launch_status();
     }
     const int64_t rows = T * B, CHW = C * HW;
@@ -256,7 +262,37 @@ int bn_stats(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B, int
     if (rc != SNNLIF_OK) return rc;
     launch_kernel(bn_stats_finalize_kernel<F>, dim3(static_cast<unsigned>(C)), dim3(kReduceBlock), 0,
                   stream, x, part_d, part_dd, out_a, out_b, HW, static_cast<int64_t>(S), HW, CHW, count,
-                  mode);
+                  mode, running);
+    return launch_status();
+}
+
+// Statistics of a sharded batch from its all-reduced moments, as the reference's sharded layers form
+// them (snnlib/example/snnlib_op.py:271-275): mean = first / world, var = second / world - mean^2 (the
+// framework divides by a scalar as a multiplication by its reciprocal, and squares by a product), and
+// the running pair.  One lane per channel.
+template <typename F>
+__global__ void __launch_bounds__(kReduceBlock)
+bn_moments_finish_kernel(const F* __restrict__ first, const F* __restrict__ second,
+                         F* __restrict__ mean, F* __restrict__ var, F inv_world,
+                         RunningUpdate<F> running, int64_t C) {
+    const int64_t c = static_cast<int64_t>(blockIdx.x) * kReduceBlock + threadIdx.x;
+    if (c >= C) return;
+    const F m = first[c] * inv_world;
+    const F v = second[c] * inv_world - m * m;
+    mean[c] = m;
+    var[c] = v;
+    if (running.mean_out != nullptr) {
+        running.mean_out[c] = running.mean_in[c] * running.keep + m * running.gain_mean;
+        running.var_out[c] = running.var_in[c] * running.keep + v * running.gain_var;
+    }
+}
+
+template <typename F>
+int bn_moments_finish(const F* first, const F* second, F* mean, F* var, F inv_world,
+                      const RunningUpdate<F>& running, int64_t C, hipStream_t stream) {
+    launch_kernel(bn_moments_finish_kernel<F>,
+                  dim3(static_cast<unsigned>((C + kReduceBlock - 1) / kReduceBlock)), dim3(kReduceBlock),
+                  0, stream, first, second, mean, var, inv_world, running, C);
     return launch_status();
 }
 
@@ -265,8 +301,14 @@ int bn_stats(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B, int
 #define SNNLIF_DEFINE_BN_STATS_DTYPE(SUFFIX, F)                                                    \
     namespace snnlif {                                                                             \
     int bn_stats_##SUFFIX(const F* x, F* out_a, F* out_b, int mode, int64_t T, int64_t B,          \
-                          int64_t C, int64_t HW, double* workspace, hipStream_t stream) {          \
-        return bn_stats<F>(x, out_a, out_b, mode, T, B, C, HW, workspace, stream);                 \
+                          int64_t C, int64_t HW, double* workspace, hipStream_t stream,            \
+                          const RunningUpdate<F>& running) {                                       \
+        return bn_stats<F>(x, out_a, out_b, mode, T, B, C, HW, workspace, stream, running);        \
+    }                                                                                              \
+    int bn_moments_finish_##SUFFIX(const F* first, const F* second, F* mean, F* var, F inv_world,  \
+                                   const RunningUpdate<F>& running, int64_t C,                     \
+                                   hipStream_t stream) {                                           \
+        return bn_moments_finish<F>(first, second, mean, var, inv_world, running, C, stream);      \
     }                                                                                              \
     }
 

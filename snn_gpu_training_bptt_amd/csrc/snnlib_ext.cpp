@@ -18,7 +18,7 @@
 // plus fire_us_fp(spatial, alpha, thresh) -> (mem, spike), the public face of the reference's
 // internal fire_us_fp_kernel (snnlib/cuda/snn_kernel_bp.cu:54-93), bn_stats(spatial) -> [var, mean] and
 // bn_moments(spatial) -> [E[x], E[x^2]], the batch statistics the reference's layers take from
-// torch.var_mean / torch.mean (snnlib/example/snnlib_op.py:76-78, 263-264), and the halves that a batch sharded
+// torch.var_mean / torch.mean (snnlib/example/snnlib_op.py:78, 263-264), and the halves that a batch sharded
 // over several GPUs runs on either side of its all-reduce (the all-reduce itself is the caller's):
 //
 //   bn_bp_dist1 / bn_bp_dist2                                                       snn.cpp:317-355
@@ -142,6 +142,14 @@ Tensor channel_param(const Tensor& p, const Tensor& like, int64_t C, const char*
     TORCH_CHECK(p.numel() == C, "snnlib.", op, ": ", name, " must have one value per channel (", C,
                 "), got ", p.sizes());
     return p.contiguous();
+}
+
+// A per-channel result of a backward op.  The kernels write every channel whenever the activation has
+// elements; only for an empty activation (which they leave alone) is it filled with zeros: an empty
+// local batch contributes nothing to the all-reduce and leaves the parameter gradients untouched.
+Tensor channel_result(const Tensor& like, const Tensor& activation) {
+    return activation.numel() == 0 ? torch::zeros_like(like, at::MemoryFormat::Contiguous)
+                                   : torch::empty_like(like, at::MemoryFormat::Contiguous);
 }
 
 // A freshly computed tensor under another shape, handed out as a tensor of its own rather than as
@@ -381,8 +389,8 @@ BnOperands bn_operands(const Tensor& spatial, const Tensor& weight_bn, const Ten
 
 // Per-channel batch statistics over every axis but the channel's (axis 2), on the hand-written
 // reduction behind snnlif_bn_stats: what the layers of snnlib/example/snnlib_op.py obtain from
-// torch.var_mean(x, dim_bn, unbiased=False) (:76-78) or, for a sharded batch, from torch.mean(x) and
-// torch.mean(x**2) (:263-264) before they call a batch-norm op.  Not part of the reference's binding
+// torch.var_mean(x, dim_bn, unbiased=False) (:78) or, for a sharded batch, from torch.mean(x) and
+// torch.mean(x**2) (:265-266) before they call a batch-norm op.  Not part of the reference's binding
 // table.  raw_moments = false -> {var (biased), mean}; true -> {E[x], E[x^2]}.
 std::vector<Tensor> batch_statistics(const Tensor& spatial, bool raw_moments, const char* op) {
     check_input(spatial, op, "spatial");
@@ -409,6 +417,72 @@ std::vector<Tensor> batch_statistics(const Tensor& spatial, bool raw_moments, co
 }
 
 std::vector<Tensor> bn_stats(Tensor spatial) { return batch_statistics(spatial, false, "bn_stats"); }
+
+// bn_stats with the layer's running statistics advanced in the same pass:
+//   -> {var, mean, running_var * keep + var * gain_var, running_mean * keep + mean * gain_mean}
+// what the reference's layers compute in Python after torch.var_mean in training mode
+// (snnlib/example/snnlib_op.py:78-80), bit for bit, without the six small element-wise launches.
+std::vector<Tensor> bn_stats_running(Tensor spatial, Tensor running_var, Tensor running_mean,
+                                     double keep, double gain_var, double gain_mean) {
+    const char* op = "bn_stats_running";
+    check_input(spatial, op, "spatial");
+    TORCH_CHECK(spatial.scalar_type() == at::kFloat || spatial.scalar_type() == at::kDouble,
+                "snnlib.", op, ": only float32 and float64 are supported, got ",
+                spatial.scalar_type());
+    const int dtype = spatial.scalar_type() == at::kFloat ? SNNLIF_DTYPE_F32 : SNNLIF_DTYPE_F64;
+    const BnDims d = bn_dims_of(spatial, op);
+    TORCH_CHECK(d.C == 0 || (d.T > 0 && d.B > 0 && d.HW > 0), "snnlib.", op,
+                ": no elements per channel in a tensor shaped ", spatial.sizes());
+    const DeviceGuard guard(spatial.device());
+    Tensor x = spatial.contiguous();
+    Tensor rv = channel_param(running_var.detach(), x, d.C, op, "running_var");
+    Tensor rm = channel_param(running_mean.detach(), x, d.C, op, "running_mean");
+    Tensor mean = torch::empty({d.C}, x.options());
+    Tensor var = torch::empty({d.C}, x.options());
+    Tensor new_rv = torch::empty({d.C}, x.options());
+    Tensor new_rm = torch::empty({d.C}, x.options());
+    const size_t ws_bytes = snnlif_bn_stats_workspace_bytes(dtype, d.T, d.B, d.C, d.HW);
+    Tensor workspace =
+        torch::empty({static_cast<int64_t>(ws_bytes)}, x.options().dtype(at::kByte));
+    check_rc(snnlif_bn_stats_running(x.data_ptr(), mean.data_ptr(), var.data_ptr(), rm.data_ptr(),
+                                     rv.data_ptr(), new_rm.data_ptr(), new_rv.data_ptr(), keep,
+                                     gain_mean, gain_var, dtype, d.T, d.B, d.C, d.HW,
+                                     ws_bytes ? workspace.data_ptr() : nullptr, ws_bytes,
+                                     current_stream()),
+             op);
+    return {var, mean, new_rv, new_rm};
+}
+
+// The statistics of a sharded batch from its all-reduced moments and the running pair, one small
+// kernel for the ten element-wise ops of snnlib/example/snnlib_op.py:271-275, with their bits:
+//   -> {var, mean, running_var * keep + var * gain_var, running_mean * keep + mean * gain_mean}
+std::vector<Tensor> bn_moments_finish(Tensor first, Tensor second, double world_size,
+                                      Tensor running_var, Tensor running_mean, double keep,
+                                      double gain_var, double gain_mean) {
+    const char* op = "bn_moments_finish";
+    TORCH_CHECK(first.defined() && first.is_cuda(), "snnlib.", op,
+                ": first must live on a ROCm GPU (this build has no CPU path)");
+    TORCH_CHECK(first.scalar_type() == at::kFloat || first.scalar_type() == at::kDouble, "snnlib.",
+                op, ": only float32 and float64 are supported, got ", first.scalar_type());
+    TORCH_CHECK(world_size >= 1.0, "snnlib.", op, ": world_size must be at least 1");
+    const int dtype = first.scalar_type() == at::kFloat ? SNNLIF_DTYPE_F32 : SNNLIF_DTYPE_F64;
+    const int64_t C = first.numel();
+    const DeviceGuard guard(first.device());
+    Tensor a = first.contiguous();
+    Tensor b = channel_param(second, a, C, op, "second");
+    Tensor rv = channel_param(running_var.detach(), a, C, op, "running_var");
+    Tensor rm = channel_param(running_mean.detach(), a, C, op, "running_mean");
+    Tensor mean = torch::empty({C}, a.options());
+    Tensor var = torch::empty({C}, a.options());
+    Tensor new_rv = torch::empty({C}, a.options());
+    Tensor new_rm = torch::empty({C}, a.options());
+    check_rc(snnlif_bn_moments_finish(a.data_ptr(), b.data_ptr(), mean.data_ptr(), var.data_ptr(),
+                                      rm.data_ptr(), rv.data_ptr(), new_rm.data_ptr(),
+                                      new_rv.data_ptr(), world_size, keep, gain_mean, gain_var, dtype,
+                                      C, current_stream()),
+             op);
+    return {var, mean, new_rv, new_rm};
+}
 
 std::vector<Tensor> bn_moments(Tensor spatial) { return batch_statistics(spatial, true, "bn_moments"); }
 
@@ -483,11 +557,10 @@ std::vector<Tensor> bn_fire_bp_dist1(Tensor spatial, Tensor weight_bn, Tensor bi
     check_same_shape(spatial, grad_spike, op, "spatial", "grad_spike");
     const DeviceGuard guard(spatial.device());
     Tensor g = grad_spike.contiguous();
-    // zeros: an empty local batch contributes nothing to the all-reduce
-    Tensor mean_gxhat = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
-    Tensor mean_gxhatx = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
-    Tensor grad_weight = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
-    Tensor grad_bias = torch::zeros_like(o.weight, at::MemoryFormat::Contiguous);
+    Tensor mean_gxhat = channel_result(o.weight, o.x);
+    Tensor mean_gxhatx = channel_result(o.weight, o.x);
+    Tensor grad_weight = channel_result(o.weight, o.x);
+    Tensor grad_bias = channel_result(o.weight, o.x);
     const size_t ws_bytes =
         snnlif_bn_fire_bp_workspace_bytes(o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW);
     Tensor workspace =
@@ -587,9 +660,8 @@ std::vector<Tensor> bn_bp(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, Tensor 
     Tensor g = dense_gradient(grad_y_bn, x_bn, op, "grad_y_bn");
     const DeviceGuard guard(x_bn.device());
     Tensor grad_x = torch::empty_like(o.x, at::MemoryFormat::Contiguous);
-    // zeros: a tensor without elements leaves the parameter gradients untouched
-    Tensor grad_weight = torch::zeros_like(w, at::MemoryFormat::Contiguous);
-    Tensor grad_bias = torch::zeros_like(w, at::MemoryFormat::Contiguous);
+    Tensor grad_weight = channel_result(w, o.x);
+    Tensor grad_bias = channel_result(w, o.x);
     const size_t ws_bytes = snnlif_bn_bp_workspace_bytes(o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW);
     Tensor workspace = byte_workspace(ws_bytes, o.x);
     check_rc(snnlif_bn_bp(o.x.data_ptr(), w.data_ptr(), iv.data_ptr(), m.data_ptr(), g.data_ptr(),
@@ -614,11 +686,10 @@ std::vector<Tensor> bn_bp_dist1(Tensor x_bn, Tensor weight_bn, Tensor bias_bn, T
     Tensor m = channel_param(mean, o.x, o.d.C, op, "mean");
     Tensor g = dense_gradient(grad_y_bn, x_bn, op, "grad_y_bn");
     const DeviceGuard guard(x_bn.device());
-    // zeros: an empty local batch contributes nothing to the all-reduce
-    Tensor mean_gxhat = torch::zeros_like(w, at::MemoryFormat::Contiguous);
-    Tensor mean_gxhatx = torch::zeros_like(w, at::MemoryFormat::Contiguous);
-    Tensor grad_weight = torch::zeros_like(w, at::MemoryFormat::Contiguous);
-    Tensor grad_bias = torch::zeros_like(w, at::MemoryFormat::Contiguous);
+    Tensor mean_gxhat = channel_result(w, o.x);
+    Tensor mean_gxhatx = channel_result(w, o.x);
+    Tensor grad_weight = channel_result(w, o.x);
+    Tensor grad_bias = channel_result(w, o.x);
     const size_t ws_bytes = snnlif_bn_bp_workspace_bytes(o.dtype, o.d.T, o.d.B, o.d.C, o.d.HW);
     Tensor workspace = byte_workspace(ws_bytes, o.x);
     check_rc(snnlif_bn_bp_dist1(o.x.data_ptr(), w.data_ptr(), iv.data_ptr(), m.data_ptr(),
@@ -877,6 +948,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
 
     m.def("bn_stats", &bn_stats, "per-channel [biased variance, mean] of a [T, B, C, ...] tensor");
     m.def("bn_moments", &bn_moments, "per-channel [E[x], E[x^2]] of a [T, B, C, ...] tensor");
+    m.def("bn_stats_running", &bn_stats_running,
+          "bn_stats plus the running statistics: [var, mean, new_running_var, new_running_mean]");
+    m.def("bn_moments_finish", &bn_moments_finish,
+          "[var, mean, new_running_var, new_running_mean] from a sharded batch's all-reduced moments");
 
     m.def("bn_fp", &bn_fp, "bn forward");
     m.def("bn_bp", &bn_bp, "bn backward");

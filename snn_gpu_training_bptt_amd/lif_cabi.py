@@ -21,6 +21,7 @@ BP_NO_WORKSPACE_MAX_T = 1024
 
 # name -> (restype, argtypes); must list every symbol include/snnlib_lif.h declares.
 _vp, _i64, _f32, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_float, ctypes.c_int, ctypes.c_size_t
+_f64 = ctypes.c_double
 SYMBOLS = {
     "snnlif_abi_version": (_int, []),
     "snnlif_target_arch": (ctypes.c_char_p, []),
@@ -34,6 +35,8 @@ SYMBOLS = {
                                       _sz, _vp]),
     "snnlif_bn_stats_workspace_bytes": (_sz, [_int, _i64, _i64, _i64, _i64]),
     "snnlif_bn_stats": (_int, [_vp, _vp, _vp, _int, _i64, _i64, _i64, _i64, _int, _vp, _sz, _vp]),
+    "snnlif_bn_stats_running": (_int, [_vp] * 7 + [_f64, _f64, _f64, _int, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
+    "snnlif_bn_moments_finish": (_int, [_vp] * 8 + [_f64, _f64, _f64, _f64, _int, _i64, _vp]),
     "snnlif_channel_sum": (_int, [_vp, _vp, _int, _i64, _i64, _i64, _i64, _vp, _sz, _vp]),
     "snnlif_bn_fire_s_fp": (_int, [_vp] * 7 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _f32, _vp]),
     "snnlif_bn_fire_s_recompute": (_int, [_vp] * 6 + [_int, _i64, _i64, _i64, _i64, _f32, _f32, _vp]),
@@ -280,6 +283,51 @@ def bn_stats_into(spatial, mean, var, workspace, raw_moments=False):
                                 _torch_dtype_code(spatial), T, B, C, HW, int(bool(raw_moments)),
                                 workspace.data_ptr(), workspace.numel(), _stream_handle(spatial))
     _check(rc, "snnlif_bn_stats")
+    return mean, var
+
+
+def bn_stats_running_into(spatial, mean, var, running_mean, running_var, new_running_mean, new_running_var,
+                          workspace, keep, gain_mean, gain_var):
+    """``snnlif_bn_stats_running``: ``bn_stats_into`` plus the layer's running statistics,
+    ``new = running * keep + statistic * gain`` rounded like the framework's element-wise expression."""
+    T, B, C, HW = _bn_dims(spatial)
+    _require_per_channel(spatial, C, mean=mean, var=var, running_mean=running_mean, running_var=running_var,
+                         new_running_mean=new_running_mean, new_running_var=new_running_var)
+    _require_workspace(spatial, workspace,
+                       bn_stats_workspace_bytes(_torch_dtype_code(spatial), T, B, C, HW),
+                       "snnlif_bn_stats_running")
+    _require_dense_gpu(spatial, mean, var, running_mean, running_var, new_running_mean, new_running_var, workspace)
+    rc = load().snnlif_bn_stats_running(spatial.data_ptr(), mean.data_ptr(), var.data_ptr(),
+                                        running_mean.data_ptr(), running_var.data_ptr(),
+                                        new_running_mean.data_ptr(), new_running_var.data_ptr(),
+                                        float(keep), float(gain_mean), float(gain_var),
+                                        _torch_dtype_code(spatial), T, B, C, HW, workspace.data_ptr(),
+                                        workspace.numel(), _stream_handle(spatial))
+    _check(rc, "snnlif_bn_stats_running")
+    return mean, var, new_running_mean, new_running_var
+
+
+def bn_moments_finish_into(first, second, mean, var, world_size, running=None):
+    """``snnlif_bn_moments_finish``: mean and variance of a sharded batch from its all-reduced moments;
+    ``running`` = (running_mean, running_var, new_running_mean, new_running_var, keep, gain_mean, gain_var)
+    also advances the running pair."""
+    C = first.numel()
+    _require_per_channel(first, C, second=second, mean=mean, var=var)
+    tensors = [first, second, mean, var]
+    ptrs = [0, 0, 0, 0]
+    factors = (1.0, 0.0, 0.0)
+    if running is not None:
+        _require_per_channel(first, C, running_mean=running[0], running_var=running[1],
+                             new_running_mean=running[2], new_running_var=running[3])
+        tensors += list(running[:4])
+        ptrs = [t.data_ptr() for t in running[:4]]
+        factors = tuple(float(f) for f in running[4:7])
+    _require_dense_gpu(*tensors)
+    rc = load().snnlif_bn_moments_finish(first.data_ptr(), second.data_ptr(), mean.data_ptr(), var.data_ptr(),
+                                         ptrs[0] or None, ptrs[1] or None, ptrs[2] or None, ptrs[3] or None,
+                                         float(world_size), factors[0], factors[1], factors[2],
+                                         _torch_dtype_code(first), C, _stream_handle(first))
+    _check(rc, "snnlif_bn_moments_finish")
     return mean, var
 
 

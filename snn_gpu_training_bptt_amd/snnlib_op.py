@@ -58,9 +58,12 @@ class _BatchStatistics(nn.Module):
             self.running_mean = self.running_mean.to(x.device)
         if not self.train_bn:
             return self.running_var, self.running_mean
-        var, mean = sf.snnlib.bn_stats(_channel_major_input(x, self.dim_bn))
-        self.running_var = nn.Parameter(self.running_var * 0.9 + var * (0.1 * self.factor))
-        self.running_mean = nn.Parameter(self.running_mean * 0.9 + mean * 0.1)
+        # one native call: the statistics and running * 0.9 + statistic * 0.1 (the variance's gain
+        # carries the unbiasing factor), the bits of the reference's element-wise expressions
+        var, mean, running_var, running_mean = sf.snnlib.bn_stats_running(
+            _channel_major_input(x, self.dim_bn), self.running_var, self.running_mean, 0.9, 0.1 * self.factor, 0.1)
+        self.running_var = nn.Parameter(running_var)
+        self.running_mean = nn.Parameter(running_mean)
         return var, mean
 
 
@@ -86,10 +89,12 @@ class _ShardedBatchStatistics(_BatchStatistics):
         first, second = sf.snnlib.bn_moments(_channel_major_input(x, self.dim_bn))
         torch.distributed.all_reduce(first, self.ReduceOp.SUM, self.process_group)
         torch.distributed.all_reduce(second, self.ReduceOp.SUM, self.process_group)
-        mean = first / self.world_size
-        var = second / self.world_size - mean ** 2
-        self.running_var = nn.Parameter(self.running_var * 0.95 + var * (0.05 * self.factor))
-        self.running_mean = nn.Parameter(self.running_mean * 0.95 + mean * 0.05)
+        # mean = first / world, var = second / world - mean ** 2 and the running pair (momentum 0.05), the
+        # bits of the reference's element-wise expressions, in one native call
+        var, mean, running_var, running_mean = sf.snnlib.bn_moments_finish(
+            first, second, self.world_size, self.running_var, self.running_mean, 0.95, 0.05 * self.factor, 0.05)
+        self.running_var = nn.Parameter(running_var)
+        self.running_mean = nn.Parameter(running_mean)
         return var, mean
 
     def _reduce_op(self):

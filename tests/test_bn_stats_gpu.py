@@ -2,8 +2,8 @@
 the C ABI.
 
 What it replaces is a library routine -- ``torch.var_mean(x, dim_bn, unbiased=False)`` in the
-reference's layers (snnlib/example/snnlib_op.py:76-78) and ``torch.mean(x)``, ``torch.mean(x**2)`` in the
-sharded ones (:263-264) -- so that routine, evaluated in float64 on the same values, is the checker:
+reference's layers (snnlib/example/snnlib_op.py:78) and ``torch.mean(x)``, ``torch.mean(x**2)`` in the
+sharded ones (:265-266) -- so that routine, evaluated in float64 on the same values, is the checker:
 fp32 results within 1e-6 of it (relative to the statistic's scale), fp64 within 1e-13.  The per-channel sum
 replaces ``at::sum(grad_conv, dim_conv)``, the bias gradient of the layers that end in a convolution
 (snnlib/cuda/snn_kernel_bp.cu:1261, 1338, 1401, 1435): checked against the float64 sum of the same
@@ -272,6 +272,98 @@ def test_convolution_bias_gradient_takes_the_channel_sum():
     torch.testing.assert_close(small, g[..., :4, :4].sum(dim=(0, 1, 3, 4)))   # planes of 16 positions: ATen's
 
 
+RUNNING_SHAPES = [(6, 2, 8), (6, 2, 8, 8, 8), (8, 16, 32, 16, 16), (4, 5, 7, 7, 7), (5, 2, 9, 31), (13, 3, 20, 5, 3),
+                  (8, 64, 1024), (6, 64, 8, 8, 8)]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("shape", RUNNING_SHAPES)
+def test_running_statistics_carry_the_bits_of_the_layer_expressions(cabi, shape, dtype):
+    """``snnlif_bn_stats_running`` = ``snnlif_bn_stats`` + what the reference's layers do next in Python
+    (snnlib/example/snnlib_op.py:79-80): ``running * 0.9 + statistic * gain`` as the framework's
+    element-wise ops evaluate it on the same device -- the same bits, also when written in place."""
+    x = make(shape, seed=60, dtype=dtype).cuda()
+    T, B, C, HW = dims_of(shape)
+    gen = torch.Generator().manual_seed(61)
+    running_var = (0.5 + torch.rand(C, generator=gen)).to(dtype).cuda()
+    running_mean = torch.randn(C, generator=gen).to(dtype).cuda()
+    n = T * B * HW
+    factor = n / (n - 1) if n > 1 else 1.0
+    mean_ref, var_ref = (t.cuda() for t in run_stats(cabi, x))
+    want_var = running_var * 0.9 + var_ref * (0.1 * factor)
+    want_mean = running_mean * 0.9 + mean_ref * 0.1
+    code = cabi.DTYPE_F32 if dtype == torch.float32 else cabi.DTYPE_F64
+    ws = torch.empty(cabi.bn_stats_workspace_bytes(code, T, B, C, HW), dtype=torch.uint8, device="cuda")
+    mean, var, new_mean, new_var = (torch.full((C,), float("nan"), dtype=dtype, device="cuda") for _ in range(4))
+    cabi.bn_stats_running_into(x, mean, var, running_mean, running_var, new_mean, new_var, ws,
+                               0.9, 0.1, 0.1 * factor)
+    torch.cuda.synchronize()
+    assert torch.equal(mean, mean_ref) and torch.equal(var, var_ref)
+    assert torch.equal(new_var, want_var) and torch.equal(new_mean, want_mean)
+    assert torch.equal(running_var, (0.5 + torch.rand(C, generator=torch.Generator().manual_seed(61))).to(dtype).cuda())
+    # in place
+    rm, rv = running_mean.clone(), running_var.clone()
+    cabi.bn_stats_running_into(x, mean, var, rm, rv, rm, rv, ws, 0.9, 0.1, 0.1 * factor)
+    torch.cuda.synchronize()
+    assert torch.equal(rv, want_var) and torch.equal(rm, want_mean)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("world", [1, 2, 3, 6, 7, 8])
+def test_moments_finish_carries_the_bits_of_the_sharded_layers_expressions(cabi, world, dtype):
+    """``snnlif_bn_moments_finish`` against snnlib/example/snnlib_op.py:271-275 evaluated by the framework on
+    the same device: ``mean = first / world``, ``var = second / world - mean ** 2`` and the running pair with
+    momentum 0.05; world sizes that are not powers of two show whether the division is the framework's."""
+    C = 1000
+    gen = torch.Generator().manual_seed(62 + world)
+    first = (world * (0.3 + torch.randn(C, generator=gen))).to(dtype).cuda()
+    second = (world * (1.5 + torch.rand(C, generator=gen) * 3)).to(dtype).cuda()
+    running_var = (0.5 + torch.rand(C, generator=gen)).to(dtype).cuda()
+    running_mean = torch.randn(C, generator=gen).to(dtype).cuda()
+    factor = 98304 / 98303
+    want_mean = first / world
+    want_var = second / world - want_mean ** 2
+    want_rv = running_var * 0.95 + want_var * (0.05 * factor)
+    want_rm = running_mean * 0.95 + want_mean * 0.05
+    mean, var, new_mean, new_var = (torch.full((C,), float("nan"), dtype=dtype, device="cuda") for _ in range(4))
+    cabi.bn_moments_finish_into(first, second, mean, var, world,
+                                running=(running_mean, running_var, new_mean, new_var, 0.95, 0.05, 0.05 * factor))
+    torch.cuda.synchronize()
+    assert torch.equal(mean, want_mean) and torch.equal(var, want_var)
+    assert torch.equal(new_var, want_rv) and torch.equal(new_mean, want_rm)
+    # without a running pair
+    mean2, var2 = torch.empty_like(mean), torch.empty_like(var)
+    cabi.bn_moments_finish_into(first, second, mean2, var2, world)
+    torch.cuda.synchronize()
+    assert torch.equal(mean2, want_mean) and torch.equal(var2, want_var)
+
+
+def test_running_and_moments_argument_errors(cabi):
+    lib = cabi.load()
+    x = torch.zeros(4, 2, 8, device="cuda")
+    p = [torch.zeros(8, device="cuda") for _ in range(6)]
+    ws = torch.zeros(1 << 16, dtype=torch.uint8, device="cuda")
+    f32 = cabi.DTYPE_F32
+    ptr = [t.data_ptr() for t in p]
+    run = lambda dtype, T, w, n, rm=ptr[2]: lib.snnlif_bn_stats_running(
+        x.data_ptr(), ptr[0], ptr[1], rm, ptr[3], ptr[4], ptr[5], 0.9, 0.1, 0.1, dtype, T, 2, 8, 1, w, n, None)
+    assert run(f32, 4, ws.data_ptr(), ws.numel()) == cabi.OK
+    assert run(cabi.DTYPE_BF16, 4, ws.data_ptr(), ws.numel()) == cabi.ERR_UNSUPPORTED
+    assert run(f32, 0, ws.data_ptr(), ws.numel()) == cabi.ERR_ARG
+    assert run(f32, 4, None, 0) == cabi.ERR_WORKSPACE
+    assert run(f32, 4, ws.data_ptr(), ws.numel(), rm=None) == cabi.ERR_ARG
+    fin = lambda world, rm, rv, nm, nv, C=8, dtype=f32: lib.snnlif_bn_moments_finish(
+        ptr[0], ptr[1], ptr[2], ptr[3], rm, rv, nm, nv, world, 0.95, 0.05, 0.05, dtype, C, None)
+    assert fin(2.0, None, None, None, None) == cabi.OK
+    assert fin(2.0, ptr[4], ptr[5], ptr[4], ptr[5]) == cabi.OK
+    assert fin(2.0, ptr[4], None, ptr[4], ptr[5]) == cabi.ERR_ARG        # the running pair goes together
+    assert fin(0.0, None, None, None, None) == cabi.ERR_ARG
+    assert fin(2.0, None, None, None, None, C=-1) == cabi.ERR_ARG
+    assert fin(2.0, None, None, None, None, C=0) == cabi.OK
+    assert fin(2.0, None, None, None, None, dtype=cabi.DTYPE_BF16) == cabi.ERR_UNSUPPORTED
+    torch.cuda.synchronize()
+
+
 def test_argument_errors(cabi):
     lib = cabi.load()
     x = torch.zeros(4, 2, 8, device="cuda")
@@ -314,8 +406,19 @@ def test_module_ops_and_layer_statistics():
         snnlib.bn_stats(x.cpu())
     with pytest.raises(RuntimeError, match="no elements per channel"):
         snnlib.bn_stats(torch.zeros(0, 2, 3, device="cuda"))
+    rv, rm = torch.rand(8, device="cuda") + 0.5, torch.randn(8, device="cuda")
+    n = x.numel() / 8
+    v3, m3, rv3, rm3 = snnlib.bn_stats_running(x, rv, rm, 0.9, 0.1 * n / (n - 1), 0.1)
+    assert torch.equal(v3, var) and torch.equal(m3, mean)
+    assert torch.equal(rv3, rv * 0.9 + var * (0.1 * n / (n - 1))) and torch.equal(rm3, rm * 0.9 + mean * 0.1)
+    v4, m4, rv4, rm4 = snnlib.bn_moments_finish(first * 3, second * 3, 3, rv, rm, 0.95, 0.05 * n / (n - 1), 0.05)
+    want_m = (first * 3) / 3
+    want_v = (second * 3) / 3 - want_m ** 2
+    assert torch.equal(m4, want_m) and torch.equal(v4, want_v)
+    assert torch.equal(rv4, rv * 0.95 + want_v * (0.05 * n / (n - 1))) and torch.equal(rm4, rm * 0.95 + want_m * 0.05)
     layer = sop.Bn(8, (0, 1, 3, 4)).cuda()
     layer(x.requires_grad_(True))
+    assert isinstance(layer.running_var, torch.nn.Parameter) and layer.running_var.is_leaf
     n = x.numel() / 8
     torch.testing.assert_close(layer.running_mean.detach().cpu().double(), 0.1 * mean_ref, rtol=1e-5, atol=1e-7)
     torch.testing.assert_close(layer.running_var.detach().cpu().double(), 0.9 + 0.1 * var_ref * n / (n - 1),

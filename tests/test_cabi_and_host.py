@@ -100,7 +100,8 @@ def test_snnlib_module_surface_and_cpu_rejection():
     import snnlib  # registered under the reference's top-level name by the package
     assert snnlib is sf.snnlib
     assert snnlib.__backend__ == "hip-gfx950"
-    for name in ("fire_s_fp", "fire_bp", "fire_us_fp", "bn_stats", "bn_moments"):
+    for name in ("fire_s_fp", "fire_bp", "fire_us_fp", "bn_stats", "bn_moments", "bn_stats_running",
+                 "bn_moments_finish"):
         assert callable(getattr(snnlib, name))
     # positional signatures of the reference binding (snnlib/cuda/snn.cpp:11-17, 270-279)
     with pytest.raises(TypeError):
